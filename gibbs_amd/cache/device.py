@@ -1,0 +1,62 @@
+"""Device memory behind the cache manager: key and value pages of every cache group and the
+arena of per-request state slots."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .manager import CacheManager
+
+
+@dataclass
+class LayerCache:
+    """What one layer's mixer sees of the cache during a step."""
+    group: Optional[int]                        # cache group of the pages (None: no pages)
+    kpages: Optional[torch.Tensor]              # [num_pages, kv_heads, page_size, head_dim]
+    vpages: Optional[torch.Tensor]
+    owns_pages: bool                            # False: reads another layer's pages, writes none
+    states: Dict[str, torch.Tensor]             # name -> [slots, *shape] float32 (slot stride = arena row)
+
+
+class DeviceCache:
+    """Pages are laid out [layer of group, k|v, page, kv head, slot in page, head_dim] in the
+    cache dtype (the activation dtype of the run); states are float32."""
+
+    def __init__(self, manager: CacheManager, cache_dtype: torch.dtype, device: torch.device):
+        self.manager = manager
+        self.device = device
+        self.pages: List[torch.Tensor] = []
+        for g, need in enumerate(manager.group_needs):
+            n_layers = len(manager.group_layers[g])
+            self.pages.append(torch.zeros(
+                (n_layers, 2, manager.pools[g].num_pages, need.kv_heads, manager.page_size, need.head_dim),
+                dtype=cache_dtype, device=device))
+        self.arena = torch.zeros((manager.max_requests, max(1, manager.slot_floats)),
+                                 dtype=torch.float32, device=device)
+
+    def nbytes(self) -> int:
+        return sum(p.numel() * p.element_size() for p in self.pages) + self.arena.numel() * 4
+
+    def layer_view(self, layer: int, kv_source: Optional[int] = None) -> LayerCache:
+        m = self.manager
+        src = layer if kv_source is None else kv_source
+        group = m.layer_group.get(src)
+        k = v = None
+        if group is not None:
+            idx = m.group_layers[group].index(src)
+            k, v = self.pages[group][idx, 0], self.pages[group][idx, 1]
+        states = {}
+        for (li, name), (off, shape) in m.state_layout.items():
+            if li == layer:
+                n = 1
+                for s in shape:
+                    n *= s
+                states[name] = self.arena[:, off:off + n].unflatten(1, shape) if shape else self.arena[:, off]
+        return LayerCache(group, k, v, kv_source is None and group is not None, states)
+
+    def clear_fresh_slots(self) -> None:
+        """Clears the state of slots that requests have taken since the last call."""
+        for slot in self.manager.take_fresh_slots():
+            self.arena[slot].zero_()

@@ -1,0 +1,30 @@
+"""What a mixer asks of the cache manager: paged keys and values, and fixed-size state."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """Keys and values of every cached position (`window` None), or of the last `window`
+    positions only.  Layers with equal needs form one group: one page pool and one block
+    table per request serve all of them."""
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A float32 tensor of fixed shape per request (for instance a short convolution's last
+    K-1 inputs), kept in the request's slot."""
+    name: str
+    shape: Tuple[int, ...]
+
+    @property
+    def numel(self) -> int:
+        n = 1
+        for s in self.shape:
+            n *= s
+        return n

@@ -1,0 +1,71 @@
+// RMSNorm over rows of the float32 residual stream, fused with the residual add that
+// precedes it:  v = x[r] (+ delta[r]);  (x[r] = v);  out[m] = v * rsqrt(mean(v^2) + eps) * gain.
+// Sums, the root and the gain product are float32; the output takes the activation type.
+// `rows` (optional) selects which rows are normed: out[m] comes from row rows[m].
+#include "common.h"
+
+template <typename T>
+__global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                   const float* __restrict__ gain, float eps, T* __restrict__ out,
+                                   const int* __restrict__ rows, int hidden, int write_x) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const int r = rows ? rows[m] : m;
+  float* xr = x + (size_t)r * hidden;
+  const T* dr = delta ? delta + (size_t)r * hidden : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = xr[i];
+    if (dr) {
+      v += to_float(dr[i]);
+      if (write_x) xr[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  T* o = out + (size_t)m * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = xr[i];
+    if (dr && !write_x) v += to_float(dr[i]);
+    o[i] = from_float<T>(v * scale * gain[i]);
+  }
+}
+
+// x: [n_x, hidden] float32 residual stream (updated in place when delta is given and rows is null);
+// out: [n_out, hidden]; rows: n_out row indices into x, or null with n_out == n_x.
+GIBBS_EXPORT int gibbs_add_rmsnorm(float* x, const void* delta, const float* gain, float eps, void* out,
+                                   int dtype, const int* rows, int n_out, int hidden, hipStream_t stream) {
+  GIBBS_REQUIRE(n_out >= 0 && hidden > 0, "rmsnorm: bad sizes n=%d hidden=%d", n_out, hidden);
+  if (n_out == 0) return 0;
+  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  const int write_x = rows == nullptr;
+  if (dtype == GIBBS_F32)
+    add_rmsnorm_kernel<float><<<n_out, threads, 0, stream>>>(x, (const float*)delta, gain, eps, (float*)out, rows, hidden, write_x);
+  else if (dtype == GIBBS_BF16)
+    add_rmsnorm_kernel<bf16><<<n_out, threads, 0, stream>>>(x, (const bf16*)delta, gain, eps, (bf16*)out, rows, hidden, write_x);
+  else
+    return gibbs_fail("rmsnorm: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("rmsnorm");
+}
+
+// x[r] += delta[r] alone (the last residual add of a model whose tail norms only some rows
+// still has to leave x whole for callers that read it).
+template <typename T>
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t count) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < count) x[i] += to_float(delta[i]);
+}
+
+GIBBS_EXPORT int gibbs_residual_add(float* x, const void* delta, int dtype, long count, hipStream_t stream) {
+  GIBBS_REQUIRE(count >= 0, "residual_add: bad count");
+  if (count == 0) return 0;
+  const int blocks = ceil_div(count, 256);
+  if (dtype == GIBBS_F32)
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)count);
+  else if (dtype == GIBBS_BF16)
+    residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (size_t)count);
+  else
+    return gibbs_fail("residual_add: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("residual_add");
+}

@@ -1,0 +1,108 @@
+// Per-head q/k RMSNorm, rotary position encoding and the write of k, v into cache pages,
+// in one pass over the fused projection qkv[N, (nh + 2 nkv) * hd].
+//
+//   q heads: (RMSNorm with a [hd] gain shared by all heads) -> rotation -> back in place
+//   k heads: the same with the k gain -> page[table[req][pos / ps]][kv head][pos % ps]
+//   v heads: copied to their page
+// The norm comes before the rotation.  Rotation of pair (i0, i1) by angle = float(pos) * inv_freq[j]
+// (a float32 product): half-split pairs (j, j + rot/2), interleaved pairs (2j, 2j+1); elements
+// beyond rotary_dim pass through.  Sums, the root, angles, sine and cosine are float32.
+// One wave per (row, head).  Pages are laid out [page, kv head, slot in page, hd].
+#include "common.h"
+
+namespace {
+enum { ROPE_HALF_SPLIT = 0, ROPE_INTERLEAVED = 1 };
+
+struct QkRopeArgs {
+  const float* q_gain;  // [hd] or null: no q norm
+  const float* k_gain;  // [hd] or null: no k norm
+  float eps;
+  const float* inv_freq;  // [rot / 2] or null: no rotation
+  int rot, variant;
+  const int* pos;      // [N] absolute position of each row
+  const int* row_req;  // [N] batch index of each row's request
+  const int* table;    // [n_req, max_pages] page ids of the layer's cache group
+  int max_pages, page_size, num_pages;
+  int nh, nkv, hd;
+  long ld;  // row stride of qkv
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_rope_kv_kernel(T* __restrict__ qkv, T* __restrict__ kpages,
+                                                         T* __restrict__ vpages, QkRopeArgs a) {
+  const int n = blockIdx.x;
+  const int hs = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  if (hs >= a.nh + 2 * a.nkv) return;
+  const int hd = a.hd;
+  T* src = qkv + (size_t)n * a.ld + (size_t)hs * hd;
+  const bool is_q = hs < a.nh, is_k = !is_q && hs < a.nh + a.nkv;
+  const int p = a.pos[n];
+
+  T* dst = src;  // q goes back in place
+  if (!is_q) {
+    if (!kpages) return;  // a layer that reads another layer's cache writes none
+    const int r = a.row_req[n];
+    const int page = a.table[(size_t)r * a.max_pages + p / a.page_size];
+    if (page < 0 || page >= a.num_pages) return;  // the host never asks for this; never write outside
+    const int g = is_k ? hs - a.nh : hs - a.nh - a.nkv;
+    T* base = is_k ? kpages : vpages;
+    dst = base + (((size_t)page * a.nkv + g) * a.page_size + p % a.page_size) * hd;
+  }
+  if (!is_q && !is_k) {
+    for (int e = lane; e < hd; e += WAVE) dst[e] = src[e];
+    return;
+  }
+  const float* gain = is_q ? a.q_gain : a.k_gain;
+  float scale = 1.f;
+  if (gain) {
+    float ss = 0.f;
+    for (int e = lane; e < hd; e += WAVE) {
+      const float v = to_float(src[e]);
+      ss += v * v;
+    }
+    ss = wave_sum(ss);
+    scale = 1.0f / sqrtf(ss / (float)hd + a.eps);
+  }
+  auto normed = [&](int e) -> float {
+    const float v = to_float(src[e]);
+    return gain ? v * scale * gain[e] : v;
+  };
+  const int half = a.inv_freq ? a.rot / 2 : 0;
+  // Each lane reads both elements of its pairs before it writes either, so in-place is safe.
+  for (int j = lane; j < half; j += WAVE) {
+    const int i0 = a.variant == ROPE_HALF_SPLIT ? j : 2 * j;
+    const int i1 = a.variant == ROPE_HALF_SPLIT ? j + half : 2 * j + 1;
+    const float x0 = normed(i0), x1 = normed(i1);
+    const float angle = (float)p * a.inv_freq[j];
+    const float c = cosf(angle), s = sinf(angle);
+    dst[i0] = from_float<T>(x0 * c - x1 * s);
+    dst[i1] = from_float<T>(x0 * s + x1 * c);
+  }
+  for (int e = 2 * half + lane; e < hd; e += WAVE) dst[e] = from_float<T>(normed(e));
+}
+}  // namespace
+
+GIBBS_EXPORT int gibbs_qk_rope_kv(void* qkv, void* kpages, void* vpages, int dtype, const float* q_gain,
+                                  const float* k_gain, float eps, const float* inv_freq, int rot, int variant,
+                                  const int* pos, const int* row_req, const int* table, int max_pages,
+                                  int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ld,
+                                  hipStream_t stream) {
+  GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv >= 0 && hd > 0, "qk_rope_kv: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
+  GIBBS_REQUIRE(ld >= (long)(nh + 2 * nkv) * hd, "qk_rope_kv: row stride %ld shorter than (nh + 2 nkv) * hd", ld);
+  GIBBS_REQUIRE(!inv_freq || (rot > 0 && rot % 2 == 0 && rot <= hd), "qk_rope_kv: rotary_dim %d must be even and <= head size %d", rot, hd);
+  GIBBS_REQUIRE(variant == ROPE_HALF_SPLIT || variant == ROPE_INTERLEAVED, "qk_rope_kv: unknown rotation variant %d", variant);
+  GIBBS_REQUIRE(!kpages || (vpages && table && page_size > 0 && max_pages > 0 && num_pages > 0), "qk_rope_kv: cache pages without a block table");
+  if (n_rows == 0) return 0;
+  QkRopeArgs a{q_gain, k_gain, eps, inv_freq, rot, variant, pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ld};
+  const int slots = nh + 2 * nkv;
+  dim3 grid(n_rows, ceil_div(slots, 4));
+  GIBBS_REQUIRE(grid.y <= 65535, "qk_rope_kv: too many heads (%d)", slots);
+  if (dtype == GIBBS_F32)
+    qk_rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, (float*)kpages, (float*)vpages, a);
+  else if (dtype == GIBBS_BF16)
+    qk_rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, (bf16*)kpages, (bf16*)vpages, a);
+  else
+    return gibbs_fail("qk_rope_kv: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("qk_rope_kv");
+}

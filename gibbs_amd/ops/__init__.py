@@ -1,0 +1,218 @@
+"""Python entry points of the HIP kernels: each checks on the host that operand shapes match
+what the kernel and its grid assume, then queues the kernel on the current stream."""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .lib import KernelError, call, dtype_code, library, ptr, require_cuda, stream
+
+ROPE_VARIANTS = {"half_split": 0, "interleaved": 1}
+ACTIVATIONS = {"silu": 0}
+
+
+def _i32(t: torch.Tensor, n: int, what: str) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < n:
+        raise KernelError(f"{what} must be a contiguous int32 tensor of at least {n} elements")
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, n: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[n, :] = float32(table[ids[n], :])."""
+    require_cuda(table, ids)
+    vocab, hidden = table.shape
+    _i32(ids, n, "ids")
+    if out is None:
+        out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
+    assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (n, hidden)
+    assert table.is_contiguous()
+    call("gibbs_embed", ptr(table), dtype_code(table.dtype), ptr(ids), ptr(out), n, hidden, vocab, stream())
+    return out
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
+                out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, n_out: Optional[int] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """v = x (+ delta); x <- v when all rows are normed; out = v * rsqrt(mean(v^2) + eps) * gain.
+    With `rows`, only those rows are normed (and x is left as it is)."""
+    require_cuda(x, delta, gain, rows)
+    n, hidden = x.shape
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    assert gain.dtype == torch.float32 and gain.shape == (hidden,) and gain.is_contiguous()
+    if delta is not None:
+        assert delta.shape == x.shape and delta.dtype == out_dtype and delta.is_contiguous()
+    if rows is None:
+        n_out = n
+    else:
+        n_out = rows.numel() if n_out is None else n_out
+        _i32(rows, n_out, "rows")
+    if out is None:
+        out = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device)
+    assert out.shape == (n_out, hidden) and out.dtype == out_dtype and out.is_contiguous()
+    call("gibbs_add_rmsnorm", ptr(x), ptr(delta), ptr(gain), float(eps), ptr(out), dtype_code(out_dtype),
+         ptr(rows), n_out, hidden, stream())
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
+    require_cuda(x, delta)
+    assert x.dtype == torch.float32 and x.is_contiguous() and delta.is_contiguous() and delta.shape == x.shape
+    call("gibbs_residual_add", ptr(x), ptr(delta), dtype_code(delta.dtype), x.numel(), stream())
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, o] = sum_k a[n, k] * w[o, k], all float32, plain FMA."""
+    require_cuda(a, w)
+    assert a.dtype == torch.float32 and w.dtype == torch.float32
+    assert a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], (a.shape, w.shape)
+    assert a.stride(1) == 1 and w.stride(1) == 1
+    n, i = a.shape
+    o = w.shape[0]
+    if out is None:
+        out = torch.empty((n, o), dtype=torch.float32, device=a.device)
+    assert out.shape == (n, o) and out.dtype == torch.float32 and out.stride(1) == 1
+    call("gibbs_gemm_f32", ptr(a), ptr(w), ptr(out), n, o, i, a.stride(0) if n > 1 else i,
+         w.stride(0), out.stride(0) if n > 1 else o, stream())
+    return out
+
+
+def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, o] = sum_k a[n, k] * w[o, k]: bfloat16 operands on the matrix cores, float32
+    accumulation, bfloat16 or float32 output."""
+    require_cuda(a, w)
+    assert a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], (a.shape, w.shape)
+    assert a.stride(1) == 1 and w.stride(1) == 1
+    n, i = a.shape
+    o = w.shape[0]
+    lda = a.stride(0) if n > 1 else i
+    if i % 8 or lda % 8 or w.stride(0) % 8:
+        raise KernelError(f"gemm_bf16: inner size {i} and row strides must be multiples of 8")
+    if out is None:
+        out = torch.empty((n, o), dtype=out_dtype, device=a.device)
+    assert out.shape == (n, o) and out.dtype == out_dtype and out.stride(1) == 1
+    call("gibbs_gemm_bf16", ptr(a), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i, lda, w.stride(0),
+         out.stride(0) if n > 1 else o, stream())
+    return out
+
+
+def glu(gu: torch.Tensor, activation: str = "silu", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, f] = act(gu[n, f]) * gu[n, F + f]."""
+    require_cuda(gu)
+    n, two_f = gu.shape
+    assert two_f % 2 == 0 and gu.is_contiguous()
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"glu: activation {activation!r} is not implemented; known: {sorted(ACTIVATIONS)}")
+    f = two_f // 2
+    if out is None:
+        out = torch.empty((n, f), dtype=gu.dtype, device=gu.device)
+    assert out.shape == (n, f) and out.dtype == gu.dtype and out.is_contiguous()
+    call("gibbs_glu", ptr(gu), ptr(out), dtype_code(gu.dtype), n, f, ACTIVATIONS[activation], stream())
+    return out
+
+
+def shortconv(bcx: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+              cu: torch.Tensor, ctx: torch.Tensor, slot: torch.Tensor, n_rows: int, n_req: int,
+              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Gated short convolution of a ragged batch with its per-request state.
+    bcx: [N, 3C]; taps: [C, K] float32; state: [slots, K-1, C] float32 (slot stride free)."""
+    require_cuda(bcx, taps, bias, state, cu, ctx, slot)
+    c, k = taps.shape
+    assert bcx.shape == (n_rows, 3 * c) and bcx.is_contiguous()
+    assert taps.dtype == torch.float32 and taps.is_contiguous()
+    assert bias is None or (bias.dtype == torch.float32 and bias.shape == (c,) and bias.is_contiguous())
+    assert state.dtype == torch.float32 and state.shape[1:] == (k - 1, c)
+    assert state.stride(2) == 1 and state.stride(1) == c
+    _i32(cu, n_req + 1, "cu"); _i32(ctx, n_req, "ctx"); _i32(slot, n_req, "slot")
+    if out is None:
+        out = torch.empty((n_rows, c), dtype=bcx.dtype, device=bcx.device)
+    assert out.shape == (n_rows, c) and out.dtype == bcx.dtype and out.is_contiguous()
+    call("gibbs_shortconv", ptr(bcx), ptr(taps), ptr(bias), ptr(state), state.stride(0), ptr(cu), ptr(ctx),
+         ptr(slot), ptr(out), dtype_code(bcx.dtype), n_rows, n_req, c, k, stream())
+    return out
+
+
+def _check_pages(pages: torch.Tensor, nkv: int, hd: int, dtype: torch.dtype) -> tuple[int, int]:
+    assert pages.dim() == 4 and pages.shape[1] == nkv and pages.shape[3] == hd, (pages.shape, nkv, hd)
+    assert pages.is_contiguous() and pages.dtype == dtype
+    return pages.shape[0], pages.shape[2]
+
+
+def qk_rope_kv(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, *, q_gain: Optional[torch.Tensor],
+               k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor], rotary_dim: int,
+               variant: str, pos: torch.Tensor, row_req: torch.Tensor, kpages: Optional[torch.Tensor],
+               vpages: Optional[torch.Tensor], table: Optional[torch.Tensor], n_req: int) -> None:
+    """In place on the q heads of qkv[N, (nh + 2 nkv) hd]: per-head RMSNorm then rotation; k heads the
+    same and into their cache page; v heads copied to theirs.  With kpages None only q is treated
+    (nkv then counts the k, v heads that the rows hold, usually 0)."""
+    require_cuda(qkv, q_gain, k_gain, inv_freq, pos, row_req, kpages, vpages, table)
+    assert qkv.dim() == 2 and qkv.shape[0] == n_rows and qkv.stride(1) == 1
+    assert qkv.shape[1] >= (nh + 2 * nkv) * hd
+    for g in (q_gain, k_gain):
+        assert g is None or (g.dtype == torch.float32 and g.shape == (hd,) and g.is_contiguous())
+    if inv_freq is not None:
+        assert inv_freq.dtype == torch.float32 and inv_freq.shape == (rotary_dim // 2,) and inv_freq.is_contiguous()
+    if variant not in ROPE_VARIANTS:
+        raise KernelError(f"rotation variant {variant!r} is not implemented; known: {sorted(ROPE_VARIANTS)}")
+    _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    num_pages = page_size = max_pages = 0
+    if kpages is not None:
+        num_pages, page_size = _check_pages(kpages, nkv, hd, qkv.dtype)
+        assert _check_pages(vpages, nkv, hd, qkv.dtype) == (num_pages, page_size)
+        assert table is not None and table.dim() == 2 and table.shape[0] >= n_req
+        _i32(table, n_req, "block table")
+        max_pages = table.shape[1]
+    call("gibbs_qk_rope_kv", ptr(qkv), ptr(kpages), ptr(vpages), dtype_code(qkv.dtype), ptr(q_gain), ptr(k_gain),
+         float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(pos), ptr(row_req), ptr(table),
+         max_pages, page_size, num_pages, n_rows, nh, nkv, hd, qkv.stride(0) if n_rows > 1 else qkv.shape[1],
+         stream())
+
+
+def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
+                    vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
+                    scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Causal grouped-query attention of every row over its request's cache pages.
+    q: [N, >= nh*hd] (row stride free); pages: [num_pages, nkv, page_size, hd]; table: [R, max_pages]."""
+    require_cuda(q, kpages, vpages, table, pos, row_req)
+    assert q.dim() == 2 and q.shape[0] == n_rows and q.stride(1) == 1 and q.shape[1] >= nh * hd
+    num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
+    assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
+    assert table.dim() == 2 and table.shape[0] >= n_req
+    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    if out is None:
+        out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
+    assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
+    call("gibbs_attention_plain", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
+         ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), stream())
+    return out
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Index of the first largest value of each row (NaN never wins), int32 [M]."""
+    require_cuda(logits)
+    m, v = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    if out is None:
+        out = torch.empty((m,), dtype=torch.int32, device=logits.device)
+    _i32(out, m, "out")
+    call("gibbs_argmax", ptr(logits), ptr(out), m, v, logits.stride(0) if m > 1 else v, stream())
+    return out
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, top_k: torch.Tensor,
+           u: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row: top-k, softmax at the row's temperature, top-p cut, draw with u in [0, 1)."""
+    require_cuda(logits, temperature, top_p, top_k, u)
+    m, v = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    for t in (temperature, top_p, u):
+        assert t.dtype == torch.float32 and t.numel() >= m and t.is_contiguous()
+    _i32(top_k, m, "top_k")
+    if out is None:
+        out = torch.empty((m,), dtype=torch.int32, device=logits.device)
+    _i32(out, m, "out")
+    call("gibbs_sample", ptr(logits), ptr(out), m, v, logits.stride(0) if m > 1 else v, ptr(temperature),
+         ptr(top_p), ptr(top_k), ptr(u), stream())
+    return out

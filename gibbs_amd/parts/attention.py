@@ -1,0 +1,99 @@
+"""Grouped-query attention mixer over the paged cache.
+
+In the reference's order (/root/reference/arch/lib/transformer.json5:46-87): q, k, v
+projections; optional RMSNorm of every head of q and k with one [head_dim] gain (`qk_norm:
+"before"` the rotation, as LFM2 has it, /root/reference/arch/families/lfm2.json5:80-83);
+position encoding of q and k; k, v written to the cache at their positions; causal attention of
+each row over the keys up to its own position (within `window`, if given), query head h reading
+kv head h // (heads / kv_heads) with scale `scale`; output projection.  A mixer whose params
+name `kv_source` projects no k, v and reads that layer's pages (the reference's `write: false`).
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from ..cache.needs import CacheNeed
+from ..ops.linear import linear
+from ..weights.loader import FLOAT32, TensorDecl, WeightStore
+from .base import Mixer, Runtime, build_position, register_mixer
+
+
+@register_mixer("attention")
+class AttentionMixer(Mixer):
+    def __init__(self, spec, hidden, layer_index):
+        super().__init__(spec, hidden, layer_index)
+        p = spec.params
+        self.heads, self.kv_heads, self.head_dim = int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        self.scale = float(p["scale"])
+        self.window = p.get("window")
+        self.qk_norm = p.get("qk_norm")
+        self.qk_norm_eps = float(p.get("qk_norm_eps", 0.0))
+        self.source = p.get("kv_source")
+        if self.heads % self.kv_heads:
+            raise ValueError(f"{self.heads} heads are not a multiple of {self.kv_heads} kv heads")
+        if self.qk_norm not in (None, "before"):
+            raise ValueError(f"qk_norm {self.qk_norm!r} is not implemented (None or 'before')")
+        if self.window is not None and int(self.window) <= 0:
+            raise ValueError(f"attention window {self.window} must be positive")
+        self.position = build_position(spec.position, self.head_dim)
+
+    # ------------------------------------------------------------------ what it asks for
+    def cache_need(self) -> Optional[CacheNeed]:
+        if self.source is not None:
+            return None
+        return CacheNeed(self.kv_heads, self.head_dim, None if self.window is None else int(self.window))
+
+    def kv_source(self) -> Optional[int]:
+        return self.source
+
+    def tensor_decls(self) -> List[TensorDecl]:
+        t, H, hd = self.spec.tensors, self.hidden, self.head_dim
+        decls = [TensorDecl(t["q_proj"], (self.heads * hd, H))]
+        if self.source is None:
+            decls += [TensorDecl(t["k_proj"], (self.kv_heads * hd, H)), TensorDecl(t["v_proj"], (self.kv_heads * hd, H))]
+        decls.append(TensorDecl(t["out_proj"], (H, self.heads * hd)))
+        if self.qk_norm:
+            decls.append(TensorDecl(t["q_norm"], (hd,), FLOAT32, init="gain"))
+            if self.source is None:
+                decls.append(TensorDecl(t["k_norm"], (hd,), FLOAT32, init="gain"))
+        return decls
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        t = self.spec.tensors
+        if self.source is None:
+            # one product for q, k and v: rows [Wq; Wk; Wv]
+            self.w_qkv = torch.cat([weights[t["q_proj"]], weights[t["k_proj"]], weights[t["v_proj"]]], dim=0).contiguous()
+        else:
+            self.w_qkv = weights[t["q_proj"]]
+        self.w_out = weights[t["out_proj"]]
+        self.q_gain = weights[t["q_norm"]] if self.qk_norm else None
+        self.k_gain = weights[t["k_norm"]] if self.qk_norm and self.source is None else None
+        if self.position is not None:
+            self.position.bind(weights, rt)
+
+    # ------------------------------------------------------------------ one step
+    def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
+        n = batch.n_rows
+        qkv = linear(h, self.w_qkv)
+        table = batch.tables[cache.group]
+        owns = self.source is None
+        pos = self.position
+        ops.qk_rope_kv(qkv, n, self.heads, self.kv_heads if owns else 0, self.head_dim,
+                       q_gain=self.q_gain, k_gain=self.k_gain, eps=self.qk_norm_eps,
+                       inv_freq=None if pos is None else pos.inv_freq,
+                       rotary_dim=0 if pos is None else pos.rotary_dim,
+                       variant="half_split" if pos is None else pos.variant,
+                       pos=batch.pos, row_req=batch.row_req,
+                       kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None,
+                       table=table, n_req=batch.n_req)
+        a = self.attend(qkv, batch, cache, table)
+        return linear(a, self.w_out)
+
+    def attend(self, qkv, batch, cache, table) -> torch.Tensor:
+        return ops.attention_plain(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
+                                   cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
+                                   self.window)

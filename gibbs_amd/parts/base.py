@@ -1,0 +1,161 @@
+"""Interfaces of the parts a layer is put together from, and the registries that map a
+spec's `kind` to the class that implements it.
+
+A part is built from its spec alone (sizes and constants are the spec's parameters), declares
+the checkpoint tensors it reads, and is later bound to loaded weights.  No part knows which
+model it is in.  To add a part: subclass the interface, decorate the class with the matching
+`register_*`, and name its kind in a spec; nothing else in the framework changes.
+
+  Norm            forward(x, delta, rows) -> normed rows in the activation dtype (adds delta first)
+  PositionEncoding  tables and parameters that a mixer hands to its kernels
+  Mixer           forward(h, batch, cache) -> delta [N, hidden]; may ask for cache pages
+                  (`cache_need`) and per-request state of fixed size (`state_needs`)
+  FeedForward     forward(h, batch) -> delta [N, hidden]
+  Block           forward(x, pending, batch, cache) -> pending delta (arrangement of the above)
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Sequence, Type
+
+import torch
+
+from ..cache.needs import CacheNeed, StateNeed
+from ..config.spec import FeedForwardSpec, LayerSpec, MixerSpec, NormSpec, PositionSpec
+from ..weights.loader import TensorDecl, WeightStore
+
+
+@dataclass
+class Runtime:
+    """What a part needs to know about the run it is bound into."""
+    device: torch.device
+    act_dtype: torch.dtype          # activations and cache pages: bfloat16, or float32 for the 32-bit path
+
+
+class Part:
+    def tensor_decls(self) -> List[TensorDecl]:
+        return []
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        """Takes its tensors from the store and prepares the layouts its kernels want."""
+        self.rt = rt
+
+
+class Norm(Part):
+    def __init__(self, spec: NormSpec, width: int):
+        self.spec, self.width = spec, width
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
+                n_rows: Optional[int] = None) -> torch.Tensor:
+        """x (float32 residual stream) += delta (if given and all rows are normed); returns norm(x)
+        in the activation dtype.  With `rows` only those rows (of x + delta) are normed."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def __init__(self, spec: PositionSpec, head_dim: int):
+        self.spec, self.head_dim = spec, head_dim
+
+
+class Mixer(Part):
+    def __init__(self, spec: MixerSpec, hidden: int, layer_index: int):
+        self.spec, self.hidden, self.layer_index = spec, hidden, layer_index
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        """Paged keys/values this mixer owns (None: none)."""
+        return None
+
+    def kv_source(self) -> Optional[int]:
+        """Index of the layer whose pages this mixer reads instead of owning pages."""
+        return None
+
+    def state_needs(self) -> Sequence[StateNeed]:
+        return ()
+
+    def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def __init__(self, spec: FeedForwardSpec, hidden: int):
+        self.spec, self.hidden = spec, hidden
+
+    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """One layer: an arrangement of two norms, a mixer and a feed-forward."""
+
+    def __init__(self, spec: LayerSpec, hidden: int, layer_index: int):
+        self.spec = spec
+        self.mixer_norm = build_norm(spec.mixer_norm, hidden)
+        self.mixer = build_mixer(spec.mixer, hidden, layer_index)
+        self.ffn_norm = build_norm(spec.ffn_norm, hidden)
+        self.ffn = build_feed_forward(spec.ffn, hidden)
+
+    def parts(self) -> List[Part]:
+        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+
+    def tensor_decls(self) -> List[TensorDecl]:
+        return [d for p in self.parts() for d in p.tensor_decls()]
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        for p in self.parts():
+            p.bind(weights, rt)
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], batch, cache) -> torch.Tensor:
+        """x: float32 residual stream, updated in place; `pending`: the previous block's last delta,
+        not yet added.  Returns this block's last delta, for the next norm to add."""
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registries
+NORMS: Dict[str, Type[Norm]] = {}
+POSITIONS: Dict[str, Type[PositionEncoding]] = {}
+MIXERS: Dict[str, Type[Mixer]] = {}
+FEED_FORWARDS: Dict[str, Type[FeedForward]] = {}
+ARRANGEMENTS: Dict[str, Type[Block]] = {}
+
+
+def _register(table: Dict[str, type], kind: str) -> Callable[[type], type]:
+    def deco(cls: type) -> type:
+        table[kind] = cls
+        return cls
+    return deco
+
+
+def register_norm(kind: str): return _register(NORMS, kind)
+def register_position(kind: str): return _register(POSITIONS, kind)
+def register_mixer(kind: str): return _register(MIXERS, kind)
+def register_feed_forward(kind: str): return _register(FEED_FORWARDS, kind)
+def register_arrangement(kind: str): return _register(ARRANGEMENTS, kind)
+
+
+def _lookup(table: Dict[str, type], kind: str, what: str) -> type:
+    if kind not in table:
+        raise KeyError(f"no {what} of kind {kind!r} is registered; known: {sorted(table)}")
+    return table[kind]
+
+
+def build_norm(spec: NormSpec, width: int) -> Norm:
+    return _lookup(NORMS, spec.kind, "norm")(spec, width)
+
+
+def build_position(spec: Optional[PositionSpec], head_dim: int) -> Optional[PositionEncoding]:
+    if spec is None or spec.kind == "none":
+        return None
+    return _lookup(POSITIONS, spec.kind, "position encoding")(spec, head_dim)
+
+
+def build_mixer(spec: MixerSpec, hidden: int, layer_index: int) -> Mixer:
+    return _lookup(MIXERS, spec.kind, "mixer")(spec, hidden, layer_index)
+
+
+def build_feed_forward(spec: FeedForwardSpec, hidden: int) -> FeedForward:
+    return _lookup(FEED_FORWARDS, spec.kind, "feed-forward")(spec, hidden)
+
+
+def build_block(spec: LayerSpec, hidden: int, layer_index: int) -> Block:
+    return _lookup(ARRANGEMENTS, spec.arrangement, "block arrangement")(spec, hidden, layer_index)

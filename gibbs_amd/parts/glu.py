@@ -1,0 +1,38 @@
+"""Dense gated feed-forward: down(act(gate(h)) * up(h)); with `activation: "silu"` this is
+SwiGLU (/root/reference/arch/lib/transformer.json5:117-130, /root/reference/src/graph/cpu.rs:378-390).
+Gate and up are one product against [W_gate; W_up]."""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from .. import ops
+from ..ops.linear import linear
+from ..weights.loader import TensorDecl, WeightStore
+from .base import FeedForward, Runtime, register_feed_forward
+
+
+@register_feed_forward("glu")
+class GluFeedForward(FeedForward):
+    def __init__(self, spec, hidden):
+        super().__init__(spec, hidden)
+        self.inter = int(spec.params["inter"])
+        self.activation = spec.params.get("activation", "silu")
+        if self.activation not in ops.ACTIVATIONS:
+            raise ValueError(f"feed-forward activation {self.activation!r} is not implemented")
+
+    def tensor_decls(self) -> List[TensorDecl]:
+        t = self.spec.tensors
+        return [TensorDecl(t["gate"], (self.inter, self.hidden)), TensorDecl(t["up"], (self.inter, self.hidden)),
+                TensorDecl(t["down"], (self.hidden, self.inter))]
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        t = self.spec.tensors
+        self.w_gate_up = torch.cat([weights[t["gate"]], weights[t["up"]]], dim=0).contiguous()
+        self.w_down = weights[t["down"]]
+
+    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
+        gu = linear(h, self.w_gate_up)
+        return linear(ops.glu(gu, self.activation), self.w_down)

@@ -1,0 +1,25 @@
+"""RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * gain, eps inside the root, the gain multiplied
+last, no (1 + gain) offset (/root/reference/src/model/simd.rs:75-110,
+/root/reference/arch/lib/transformer.json5:9-11)."""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+
+from .. import ops
+from ..weights.loader import FLOAT32, TensorDecl, WeightStore
+from .base import Norm, Runtime, register_norm
+
+
+@register_norm("rms")
+class RMSNorm(Norm):
+    def tensor_decls(self) -> List[TensorDecl]:
+        return [TensorDecl(self.spec.weight, (self.width,), FLOAT32, init="gain")]
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        self.gain = weights[self.spec.weight]
+
+    def forward(self, x, delta, rows=None, n_rows=None):
+        return ops.add_rmsnorm(x, delta, self.gain, self.spec.eps, self.rt.act_dtype, rows, n_rows)

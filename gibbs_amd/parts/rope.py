@@ -1,0 +1,46 @@
+"""Rotary position encoding: the table of inverse frequencies and the pairing variant that an
+attention mixer hands to its kernel.
+
+inv_freq[j] = 1 / theta^(2j / rotary_dim); with `precision: "f32"` every step of that is a
+float32 operation, as LFM2's spec asks (/root/reference/src/arch/gen.rs:154-164,
+/root/reference/arch/families/lfm2.json5:64).  The angle of position p is float32(p) * inv_freq[j]
+(/root/reference/src/graph/cpu.rs:673); variant `half_split` turns the pair (j, j + rot/2),
+`interleaved` the pair (2j, 2j + 1) (:676-695).
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..weights.loader import WeightStore
+from .base import PositionEncoding, Runtime, register_position
+
+
+def rope_inv_freq(rotary_dim: int, theta: float, precision: str = "f64") -> np.ndarray:
+    half = rotary_dim // 2
+    if precision == "f32":
+        t = np.float32(theta)
+        return np.array([np.float32(1.0) / np.power(t, np.float32(2 * j) / np.float32(rotary_dim), dtype=np.float32)
+                         for j in range(half)], dtype=np.float32)
+    if precision == "f64":
+        return np.array([1.0 / (float(theta) ** (2.0 * j / rotary_dim)) for j in range(half)]).astype(np.float32)
+    raise ValueError(f"rope precision {precision!r} is neither 'f32' nor 'f64'")
+
+
+@register_position("rope")
+class RotaryPosition(PositionEncoding):
+    def __init__(self, spec, head_dim):
+        super().__init__(spec, head_dim)
+        p = spec.params
+        self.rotary_dim = int(p.get("rotary_dim", head_dim))
+        self.variant = p.get("variant", "half_split")
+        self.theta = float(p["theta"])
+        self.precision = p.get("precision", "f64")
+        if self.rotary_dim <= 0 or self.rotary_dim % 2 or self.rotary_dim > head_dim:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and within the head size {head_dim}")
+        if self.variant not in ("half_split", "interleaved"):
+            raise ValueError(f"rope variant {self.variant!r} is not implemented")
+
+    def bind(self, weights: WeightStore, rt: Runtime) -> None:
+        self.rt = rt
+        self.inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)

@@ -1,0 +1,58 @@
+"""Random-weights mode: a model folder (config.json, model.safetensors) from a
+configuration and a seed.
+
+Every tensor has its own stream seeded by hash(name) ^ seed, so values do not depend on the
+order tensors are written in: the idea of the reference's synthetic checkpoints
+(/root/reference/src/arch/load.rs:2355-2420, per-name seed :1410), with a normal
+distribution of standard deviation 0.02 instead of its uniform +-0.02.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+from typing import Dict, Iterable
+
+import torch
+
+from ..config.base import ArchConfig
+from .loader import COMPUTE, FLOAT32, INT32, TensorDecl
+from .safetensors_io import write_safetensors
+
+
+def _stream(name: str, seed: int) -> torch.Generator:
+    h = int.from_bytes(hashlib.sha256(name.encode()).digest()[:8], "little")
+    g = torch.Generator(device="cpu")
+    g.manual_seed((h ^ (seed * 0x9E3779B97F4A7C15)) & ((1 << 63) - 1))
+    return g
+
+
+def random_tensor(decl: TensorDecl, seed: int, store_dtype: torch.dtype, std: float = 0.02,
+                  gain_std: float = 0.0, bias_std: float = 0.02) -> torch.Tensor:
+    g = _stream(decl.name, seed)
+    if decl.dtype == INT32:
+        return torch.zeros(decl.shape, dtype=torch.int32)
+    if decl.init == "gain":
+        t = torch.ones(decl.shape, dtype=torch.float32)
+        if gain_std > 0:
+            t += torch.randn(decl.shape, generator=g, dtype=torch.float32) * gain_std
+    elif decl.init == "bias":
+        t = torch.randn(decl.shape, generator=g, dtype=torch.float32) * bias_std
+    elif decl.init == "zeros":
+        t = torch.zeros(decl.shape, dtype=torch.float32)
+    else:
+        t = torch.randn(decl.shape, generator=g, dtype=torch.float32) * std
+    keep32 = decl.dtype == FLOAT32 or len(decl.shape) <= 1
+    return t if keep32 else t.to(store_dtype)
+
+
+def write_random_model(folder: str, config: ArchConfig, decls: Iterable[TensorDecl], seed: int,
+                       dtype: str = "bfloat16", std: float = 0.02, gain_std: float = 0.0,
+                       bias_std: float = 0.02) -> None:
+    """Matrices are stored in `dtype`, gains and biases in float32."""
+    store = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}[dtype]
+    os.makedirs(folder, exist_ok=True)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(config.to_dict(), f, indent=1)
+    tensors = ((d.name, random_tensor(d, seed, store, std, gain_std, bias_std)) for d in decls)
+    write_safetensors(os.path.join(folder, "model.safetensors"), list(tensors))

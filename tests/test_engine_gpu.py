@@ -1,0 +1,188 @@
+"""The engine against the plain implementation, in 32-bit and in bfloat16: each request alone
+and whole; most of it in one step and the last 32 tokens one by one; in portions of changing
+size, down to two tokens; mixed, up to four live requests with so few pages that they are used
+again; long decoding; the first tokens of a sequence."""
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ["A", "B", "C"]
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": 150, "B": 200, "C": 130}
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {n: H.make_model_dir(str(root), n, seed=11 + i) for i, n in enumerate(NAMES)}
+
+
+def make_engine(model_dir, dtype, **kw):
+    from gibbs_amd import Engine
+    kw.setdefault("max_tokens", 2048)
+    kw.setdefault("max_requests", 4)
+    return Engine(model_dir, dtype=dtype, **kw)
+
+
+def run_steps(engine, steps):
+    """steps: list of (entries, ends); entries: list of (rid, tokens, want).  Returns
+    {(rid, position): logits row} for every wanted place."""
+    from gibbs_amd import Entry
+    out, at = {}, {}
+    for entries, ends in steps:
+        logits = engine.step([Entry(r, t, w) for r, t, w in entries])
+        rows = None if logits is None else logits.cpu().numpy()
+        i = 0
+        for rid, toks, want in entries:
+            base = at.get(rid, 0)
+            for w in want:
+                out[(rid, base + w)] = rows[i]
+                i += 1
+            at[rid] = base + len(toks)
+        assert rows is None or i == rows.shape[0]
+        for rid in ends:
+            engine.release(rid)
+            at.pop(rid, None)
+    return out
+
+
+def check(model_dir, seqs, got, dtype, what):
+    """Every wanted place of every request against the plain logits of its whole sequence."""
+    for rid, ids in seqs.items():
+        want = H.plain_logits(model_dir, ids)
+        places = sorted(p for r, p in got if r == rid)
+        assert places, f"{what}: no logits for {rid}"
+        H.assert_close(np.stack([got[(rid, p)] for p in places]), want[places], dtype, f"{what} request {rid}")
+
+
+def portions(n, sizes):
+    out, at, i = [], 0, 0
+    while at < n:
+        s = min(sizes[i % len(sizes)], n - at)
+        out.append((at, at + s))
+        at += s
+        i += 1
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_whole(model_dirs, name, dtype):
+    d = model_dirs[name]
+    ids = H.tokens(1, LENGTHS[name], H.TINY[name]["vocab_size"])
+    eng = make_engine(d, dtype)
+    got = run_steps(eng, [([("r", ids, list(range(len(ids))))], ["r"])])
+    check(d, {"r": ids}, got, dtype, f"whole {name} {dtype}")
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.pools[0].num_pages
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_bulk_then_last_32_one_by_one(model_dirs, name, dtype):
+    d = model_dirs[name]
+    ids = H.tokens(2, LENGTHS[name], H.TINY[name]["vocab_size"])
+    cut = len(ids) - 32
+    steps = [([("r", ids[:cut], list(range(cut)))], [])]
+    steps += [([("r", [t], [0])], []) for t in ids[cut:]]
+    got = run_steps(make_engine(d, dtype), steps)
+    check(d, {"r": ids}, got, dtype, f"bulk+tail {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_changing_portions(model_dirs, name, dtype):
+    d = model_dirs[name]
+    ids = H.tokens(3, LENGTHS[name], H.TINY[name]["vocab_size"])
+    steps = [([("r", ids[a:b], list(range(b - a)))], []) for a, b in portions(len(ids), [7, 2, 13, 3, 2, 64, 5, 2, 17])]
+    got = run_steps(make_engine(d, dtype), steps)
+    check(d, {"r": ids}, got, dtype, f"portions {name} {dtype}")
+
+
+def mixed_schedule(seqs, rng, max_live=4):
+    """Requests start and finish at different steps; a step holds portions of some requests beside
+    single decoded tokens of others; a request may sit a step out."""
+    waiting = list(seqs)
+    live, done_at, steps = {}, {}, []
+    prompt_len = {r: max(2, int(len(ids) * 0.6)) for r, ids in seqs.items()}
+    while waiting or live:
+        while waiting and len(live) < max_live and (not live or rng.random() < 0.6):
+            live[waiting.pop(0)] = 0
+        entries, ends = [], []
+        for rid in list(live):
+            at, ids = live[rid], seqs[rid]
+            if len(live) > 1 and rng.random() < 0.15:
+                continue                                        # left out of this step
+            if at < prompt_len[rid]:
+                n = min(int(rng.choice([2, 3, 5, 8, 16, 33])), prompt_len[rid] - at)
+            else:
+                n = 1
+            entries.append((rid, ids[at:at + n], list(range(n))))
+            live[rid] = at + n
+            if live[rid] == len(ids):
+                ends.append(rid)
+                del live[rid]
+        if entries:
+            steps.append((entries, ends))
+    return steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_mixed_with_page_reuse(model_dirs, name, dtype):
+    d = model_dirs[name]
+    rng = np.random.default_rng(5)
+    vocab = H.TINY[name]["vocab_size"]
+    seqs = {f"q{i}": H.tokens(100 + i, int(n), vocab) for i, n in enumerate([70, 45, 90, 33, 64, 81, 50])}
+    steps = mixed_schedule(seqs, rng)
+    assert max(len(e) for e, _ in steps) >= 3
+    assert any(len(t) > 1 for e, _ in steps for _, t, _ in e) and any(len(t) == 1 for e, _ in steps for _, t, _ in e)
+    # pool: four live requests of at most 90 tokens, each rounded up to 64: 4 * 128 tokens
+    eng = make_engine(d, dtype, max_tokens=512, max_requests=4, page_size=16)
+    total_pages = sum(-(-len(s) // 16) for s in seqs.values())
+    assert total_pages > eng.cache.pools[0].num_pages, "the pool must be too small to avoid reuse"
+    got = run_steps(eng, steps)
+    check(d, seqs, got, dtype, f"mixed {name} {dtype}")
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.pools[0].num_pages and eng.cache.free_slots() == 4
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_long_decoding(model_dirs, dtype):
+    d = model_dirs["A"]
+    ids = H.tokens(9, 400, 256)
+    steps = [([("r", ids[:8], list(range(8)))], [])] + [([("r", [t], [0])], []) for t in ids[8:]]
+    got = run_steps(make_engine(d, dtype), steps)
+    check(d, {"r": ids}, got, dtype, f"long decoding {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", NAMES)
+def test_first_tokens(model_dirs, name, dtype):
+    """Positions 0, 1, 2 fed one by one: empty history in the convolution and a single key."""
+    d = model_dirs[name]
+    ids = H.tokens(4, 5, H.TINY[name]["vocab_size"])
+    got = run_steps(make_engine(d, dtype), [([("r", [t], [0])], []) for t in ids])
+    check(d, {"r": ids}, got, dtype, f"first tokens {name} {dtype}")
+
+
+def test_step_errors(model_dirs):
+    from gibbs_amd import Entry, OutOfPages, StepError
+    eng = make_engine(model_dirs["A"], "float32", max_tokens=64, max_requests=2, page_size=16)
+    with pytest.raises(StepError, match="no tokens"):
+        eng.step([Entry("a", [], [])])
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        eng.step([Entry("a", [1, 256], [])])
+    with pytest.raises(StepError, match="context limit"):
+        eng.step([Entry("a", [1] * 513, [])])
+    with pytest.raises(OutOfPages):
+        eng.step([Entry("a", [1] * 65, [])])
+    eng.cache.check()
+    assert eng.cache.free_pages() == 4 and eng.cache.free_slots() == 2, "a refused step must change nothing"
+    assert eng.step([Entry("a", [1] * 64, [63])]).shape == (1, 256)
+    with pytest.raises(OutOfPages):
+        eng.step([Entry("a", [2], [0])])

@@ -1,0 +1,290 @@
+"""Each kernel alone against a plain float32 PyTorch reference of the same operation, at sizes
+other than the engine's tiny models use (sizes that are no power of two, several head sizes)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DT = [torch.float32, torch.bfloat16]
+
+
+def rnd(*shape, dtype=torch.float32, scale=1.0, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+def close(got, want, dtype, what="", f32=1e-5, bf16=1.2e-2):
+    got, want = got.float().cpu(), want.float().cpu()
+    tol = f32 if dtype == torch.float32 else bf16
+    scale = want.abs().max().item() + 1e-30
+    err = (got - want).abs().max().item()
+    assert err <= tol * scale, f"{what}: error {err:.3e} > {tol} x {scale:.3e}"
+
+
+@pytest.mark.parametrize("table_dtype", DT)
+def test_embed(table_dtype):
+    from gibbs_amd import ops
+    table = rnd(331, 72, dtype=table_dtype)
+    ids = i32([0, 330, 5, 5, 17])
+    out = ops.embed(table, ids, 5)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("hidden", [48, 200, 2048, 5000])
+def test_add_rmsnorm(dtype, hidden):
+    from gibbs_amd import ops
+    x = rnd(7, hidden, scale=3.0)
+    delta = rnd(7, hidden, dtype=dtype, seed=1)
+    gain = rnd(hidden, seed=2) + 1.0
+    x0 = x.clone()
+    out = ops.add_rmsnorm(x, delta, gain, 1e-6, dtype)
+    v = x0 + delta.float()
+    assert torch.equal(x, v), "the residual stream must hold x + delta exactly"
+    want = F.rms_norm(v.double(), (hidden,), gain.double(), eps=1e-6)
+    close(out, want, dtype, "add_rmsnorm")
+    # without delta; and on chosen rows only (x untouched)
+    out2 = ops.add_rmsnorm(x, None, gain, 1e-6, dtype)
+    close(out2, want, dtype, "rmsnorm")
+    rows = i32([6, 0, 3])
+    x1 = x.clone()
+    out3 = ops.add_rmsnorm(x, delta, gain, 1e-6, dtype, rows)
+    assert torch.equal(x, x1)
+    want3 = F.rms_norm((x1 + delta.float())[rows.long()].double(), (hidden,), gain.double(), eps=1e-6)
+    close(out3, want3, dtype, "rmsnorm rows")
+
+
+@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 331, 112), (130, 200, 72), (257, 129, 1000)])
+def test_gemm_f32(shape):
+    from gibbs_amd import ops
+    n, o, i = shape
+    a, w = rnd(n, i), rnd(o, i, seed=1)
+    close(ops.gemm_f32(a, w), a.double() @ w.double().t(), torch.float32, f"gemm_f32 {shape}")
+    # a row's result does not depend on the other rows of the call
+    assert torch.equal(ops.gemm_f32(a[:1].contiguous(), w), ops.gemm_f32(a, w)[:1])
+
+
+@pytest.mark.parametrize("out_dtype", DT)
+@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 331, 112), (130, 200, 72), (257, 129, 1000), (300, 512, 2048)])
+def test_gemm_bf16(shape, out_dtype):
+    from gibbs_amd import ops
+    n, o, i = shape
+    a, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
+    want = a.double() @ w.double().t()
+    got = ops.gemm_bf16(a, w, out_dtype)
+    assert got.dtype == out_dtype
+    # float32 output: only the accumulation order differs from the exact product
+    close(got, want, out_dtype, f"gemm_bf16 {shape}", f32=2e-5, bf16=4e-3)
+    # a view with a row stride (the q part of a fused projection)
+    big = rnd(n, i + 64, dtype=torch.bfloat16, seed=3)
+    close(ops.gemm_bf16(big[:, :i], w, out_dtype), big[:, :i].double() @ w.double().t(), out_dtype, "strided", f32=2e-5, bf16=4e-3)
+
+
+def test_gemm_bf16_refuses_unaligned():
+    from gibbs_amd import ops
+    from gibbs_amd.ops.lib import KernelError
+    with pytest.raises(KernelError, match="multiples of 8"):
+        ops.gemm_bf16(rnd(3, 20, dtype=torch.bfloat16), rnd(4, 20, dtype=torch.bfloat16))
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_glu(dtype):
+    from gibbs_amd import ops
+    gu = rnd(9, 2 * 200, dtype=dtype, scale=2.0)
+    want = F.silu(gu.double()[:, :200]) * gu.double()[:, 200:]
+    close(ops.glu(gu), want, dtype, "glu")
+    one = torch.tensor([[0.0, 2.0, 1.0, 3.0]], device=DEV)              # silu(0)*1 = 0, silu(2)*3
+    out = ops.glu(one)
+    assert out[0, 0].item() == 0.0 and abs(out[0, 1].item() - 2 / (1 + math.exp(-2)) * 3) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("K,C,bias", [(3, 40, False), (4, 300, True), (2, 72, True), (7, 16, False)])
+def test_shortconv_ragged_with_state(dtype, K, C, bias):
+    """Three requests in one call: a fresh one, one with history shorter than K-1 before this chunk,
+    one decoding a single token; against conv1d over each whole sequence."""
+    from gibbs_amd import ops
+    taps = rnd(C, K, seed=4)
+    b = rnd(C, seed=5) if bias else None
+    lens_before, lens_now = [0, 1, 9], [6, 2, 1]
+    slots = [2, 0, 3]
+    seqs = [rnd(lb + ln, 3 * C, dtype=dtype, seed=10 + i) for i, (lb, ln) in enumerate(zip(lens_before, lens_now))]
+    state = torch.full((4, K - 1, C), 7.0, device=DEV)                   # stale content of a reused slot
+    def reference(seq):
+        s = seq.double()
+        bx = s[:, :C] * s[:, 2 * C:]
+        cv = F.conv1d(bx.t()[None], taps.double()[:, None, :], None if b is None else b.double(), groups=C,
+                      padding=K - 1)[0, :, :seq.shape[0]].t()
+        return s[:, C:2 * C] * cv, bx
+    # first call: the histories (requests 1 and 2 only)
+    cu = i32([0, lens_before[1], lens_before[1] + lens_before[2]])
+    hist = torch.cat([seqs[1][:lens_before[1]], seqs[2][:lens_before[2]]])
+    ops.shortconv(hist, taps, b, state, cu, i32([0, 0]), i32(slots[1:]), hist.shape[0], 2)
+    # second call: all three together
+    now = torch.cat([s[lb:] for s, lb in zip(seqs, lens_before)])
+    cu = i32(np.concatenate([[0], np.cumsum(lens_now)]))
+    y = ops.shortconv(now, taps, b, state, cu, i32(lens_before), i32(slots), now.shape[0], 3)
+    at = 0
+    for seq, lb, ln, slot in zip(seqs, lens_before, lens_now, slots):
+        want, bx = reference(seq)
+        close(y[at:at + ln], want[lb:], dtype, f"shortconv rows K={K}")
+        at += ln
+        full = torch.cat([torch.zeros(K - 1, C, device=DEV, dtype=torch.float64), bx])
+        close(state[slot], full[-(K - 1):], torch.float32, "state", f32=1e-6)
+    assert torch.all(state[1] == 7.0), "a slot of no request was written"
+
+
+def paged_setup(dtype, nkv, hd, page_size, seq_lens, num_pages, seed=0):
+    """Random keys and values of several requests scattered over shuffled pages (the rest of the
+    pool holds large garbage)."""
+    rng = np.random.default_rng(seed)
+    kp = torch.full((num_pages, nkv, page_size, hd), 50.0, dtype=dtype, device=DEV)
+    vp = torch.full((num_pages, nkv, page_size, hd), -50.0, dtype=dtype, device=DEV)
+    free = rng.permutation(num_pages).tolist()
+    width = max(-(-l // page_size) for l in seq_lens)
+    table = np.full((len(seq_lens), width), -1, dtype=np.int32)
+    ks, vs = [], []
+    for r, l in enumerate(seq_lens):
+        k, v = rnd(l, nkv, hd, dtype=dtype, seed=seed + 2 * r), rnd(l, nkv, hd, dtype=dtype, seed=seed + 2 * r + 1)
+        ks.append(k); vs.append(v)
+        for j in range(-(-l // page_size)):
+            p = free.pop()
+            table[r, j] = p
+            n = min(page_size, l - j * page_size)
+            kp[p, :, :n] = k[j * page_size:j * page_size + n].transpose(0, 1)
+            vp[p, :, :n] = v[j * page_size:j * page_size + n].transpose(0, 1)
+    return kp, vp, i32(table), ks, vs
+
+
+def attention_reference(q, k, v, positions, scale, window):
+    """q: [n, nh, hd] rows at `positions` of one request with keys k, v: [L, nkv, hd]."""
+    nh, nkv = q.shape[1], k.shape[1]
+    kk, vv = k.double().repeat_interleave(nh // nkv, 1), v.double().repeat_interleave(nh // nkv, 1)
+    out = torch.zeros(q.shape, dtype=torch.float64, device=q.device)
+    for i, p in enumerate(positions):
+        lo = 0 if not window else max(0, p - window + 1)
+        s = torch.einsum("hd,lhd->hl", q[i].double(), kk[lo:p + 1]) * scale
+        out[i] = torch.einsum("hl,lhd->hd", s.softmax(-1), vv[lo:p + 1])
+    return out
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
+                                                   (8, 2, 128, 16, None), (2, 2, 256, 64, 100)])
+def test_attention_plain_paged(dtype, nh, nkv, hd, page, window):
+    from gibbs_amd import ops
+    seq_lens = [150, 3, 77]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 40)
+    # request 0: a portion of 20 rows ending at its last key; request 1: all 3 rows; request 2: one decoded row
+    rows = [(0, list(range(130, 150))), (1, [0, 1, 2]), (2, [76])]
+    pos = i32([p for _, ps in rows for p in ps])
+    row_req = i32([r for r, ps in rows for _ in ps])
+    n = pos.numel()
+    q = rnd(n, nh * hd, dtype=dtype, seed=9)
+    scale = 1 / math.sqrt(hd)
+    out = ops.attention_plain(q, n, nh, nkv, hd, kp, vp, table, 3, pos, row_req, scale, window)
+    at = 0
+    for r, ps in rows:
+        want = attention_reference(q[at:at + len(ps)].view(-1, nh, hd), ks[r], vs[r], ps, scale, window)
+        close(out[at:at + len(ps)].view(-1, nh, hd), want, dtype, f"attention request {r}", f32=2e-5, bf16=1e-2)
+        at += len(ps)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_attention_far_key_stands_out(dtype):
+    """One key far back among hundreds gets a large score: its value must dominate the output."""
+    from gibbs_amd import ops
+    nh = nkv = 1; hd = 32; L = 700
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, 16, [L], 64, seed=3)
+    q = rnd(1, hd, dtype=dtype, seed=1)
+    far = 5
+    page, off = table[0, far // 16].item(), far % 16
+    kp[page, 0, off] = (q[0].float() * 8).to(dtype)
+    ks[0][far, 0] = kp[page, 0, off]
+    out = ops.attention_plain(q, 1, nh, nkv, hd, kp, vp, table, 1, i32([L - 1]), i32([0]), 1 / math.sqrt(hd))
+    want = attention_reference(q.view(1, 1, hd), ks[0], vs[0], [L - 1], 1 / math.sqrt(hd), None)
+    close(out.view(1, 1, hd), want, dtype, "far key", f32=2e-5, bf16=1e-2)
+    assert (out.float() - vs[0][far, 0].float()).abs().max() < 0.05 * vs[0][far, 0].float().abs().max() + 0.05
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("variant", ["half_split", "interleaved"])
+@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 2, 128, 128)])
+def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot):
+    from gibbs_amd import ops
+    from gibbs_amd.parts.rope import rope_inv_freq
+    n, page, num_pages = 6, 8, 10
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype)
+    qkv0 = qkv.clone()
+    qg, kg = rnd(hd, seed=1) + 1, rnd(hd, seed=2) + 1
+    inv = torch.from_numpy(rope_inv_freq(rot, 10000.0, "f32")).to(DEV)
+    positions = [3, 4, 5, 0, 17, 9]
+    row_req = [0, 0, 0, 1, 1, 2]
+    table = i32([[4, 7, -1], [2, 9, 0], [5, 1, -1]])
+    kp = torch.zeros(num_pages, nkv, page, hd, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    ops.qk_rope_kv(qkv, n, nh, nkv, hd, q_gain=qg, k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
+                   pos=i32(positions), row_req=i32(row_req), kpages=kp, vpages=vp, table=table, n_req=3)
+
+    def ref(x, gain):                                     # x: [n, heads, hd] float64
+        x = F.rms_norm(x, (hd,), gain.double(), eps=1e-6)
+        ang = torch.tensor(positions, dtype=torch.float32, device=DEV)[:, None] * inv[None, :]
+        c, s = ang.double().cos()[:, None, :], ang.double().sin()[:, None, :]
+        out = x.clone()
+        half = rot // 2
+        i0 = torch.arange(half) if variant == "half_split" else torch.arange(half) * 2
+        i1 = i0 + half if variant == "half_split" else i0 + 1
+        out[..., i0] = x[..., i0] * c - x[..., i1] * s
+        out[..., i1] = x[..., i0] * s + x[..., i1] * c
+        return out
+    q0 = qkv0[:, :nh * hd].double().view(n, nh, hd)
+    k0 = qkv0[:, nh * hd:(nh + nkv) * hd].double().view(n, nkv, hd)
+    v0 = qkv0[:, (nh + nkv) * hd:].view(n, nkv, hd)
+    close(qkv[:, :nh * hd].view(n, nh, hd), ref(q0, qg), dtype, "q", bf16=8e-3)
+    kr = ref(k0, kg)
+    for i, (p, r) in enumerate(zip(positions, row_req)):
+        pg = table[r, p // page].item()
+        close(kp[pg, :, p % page], kr[i], dtype, "k page", bf16=8e-3)
+        assert torch.equal(vp[pg, :, p % page], v0[i])
+    assert kp.float().abs().sum(dim=(1, 3)).count_nonzero().item() == n, "exactly one page slot per row was written"
+
+
+def test_argmax_rules():
+    from gibbs_amd import ops
+    nan, inf = float("nan"), float("inf")
+    rows = torch.tensor([[1.0, 3.0, 3.0, 2.0, 0.0], [nan, 1.0, nan, 1.0, 0.0], [-inf] * 5, [nan] * 5,
+                         [0.0, -1.0, -2.0, -3.0, 5.0]], device=DEV)
+    assert ops.argmax(rows).tolist() == [1, 1, 0, 0, 4]
+    big = rnd(3, 65536 + 37)
+    big[1, 40000] = big[1, 70] = 99.0
+    assert ops.argmax(big).tolist() == [big[0].argmax().item(), 70, big[2].argmax().item()]
+
+
+def test_sample_against_plain():
+    from gibbs_amd import ops
+    from tests.plain import lfm2_plain as P
+    V, M = 1000, 12
+    logits = rnd(M, V, scale=3.0, seed=5)
+    rng = np.random.default_rng(0)
+    temp = np.array([0.8, 1.0, 0.3, 1.5] * 3, dtype=np.float32)
+    top_p = np.array([0.9, 0.5, 1.0, 0.95] * 3, dtype=np.float32)
+    top_k = np.array([50, 64, 5, 1] * 3, dtype=np.int32)
+    u = rng.random(M).astype(np.float32)
+    got = ops.sample(logits, torch.tensor(temp, device=DEV), torch.tensor(top_p, device=DEV), i32(top_k),
+                     torch.tensor(u, device=DEV)).tolist()
+    for m in range(M):
+        cand, probs = P.nucleus(logits[m].cpu().numpy(), float(temp[m]), int(top_k[m]), float(top_p[m]))
+        assert got[m] == P.draw(cand, probs, float(u[m])), f"row {m}"
+    # temperature <= 1e-4 is greedy
+    g = ops.sample(logits, torch.zeros(M, device=DEV), torch.tensor(top_p, device=DEV), i32(top_k), torch.tensor(u, device=DEV))
+    assert g.tolist() == logits.argmax(-1).tolist()
