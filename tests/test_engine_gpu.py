@@ -50,13 +50,30 @@ def run_steps(engine, steps):
     return out
 
 
-def check(model_dir, seqs, got, dtype, what):
-    """Every wanted place of every request against the plain logits of its whole sequence."""
+_whole_cache = {}
+
+
+def whole_logits(model_dir, ids, dtype):
+    """The engine's own logits for the request alone and whole, in the same precision."""
+    key = (model_dir, tuple(ids), dtype)
+    if key not in _whole_cache:
+        eng = make_engine(model_dir, dtype, max_tokens=1024, max_requests=1)
+        _whole_cache[key] = eng.step([("w", ids, list(range(len(ids))))]).cpu().numpy()
+    return _whole_cache[key]
+
+
+def check(model_dir, seqs, got, dtype, what, against_whole=True):
+    """Every wanted place of every request against the plain logits of its whole sequence, and
+    (tightly) against what the engine gives for the request alone and whole."""
     for rid, ids in seqs.items():
         want = H.plain_logits(model_dir, ids)
         places = sorted(p for r, p in got if r == rid)
         assert places, f"{what}: no logits for {rid}"
-        H.assert_close(np.stack([got[(rid, p)] for p in places]), want[places], dtype, f"{what} request {rid}")
+        mine = np.stack([got[(rid, p)] for p in places])
+        H.assert_close(mine, want[places], dtype, f"{what} request {rid} vs plain")
+        if against_whole:
+            H.assert_close(mine, whole_logits(model_dir, ids, dtype)[places], dtype,
+                           f"{what} request {rid} vs whole", tol=H.consistency(dtype))
 
 
 def portions(n, sizes):
@@ -76,7 +93,7 @@ def test_whole(model_dirs, name, dtype):
     ids = H.tokens(1, LENGTHS[name], H.TINY[name]["vocab_size"])
     eng = make_engine(d, dtype)
     got = run_steps(eng, [([("r", ids, list(range(len(ids))))], ["r"])])
-    check(d, {"r": ids}, got, dtype, f"whole {name} {dtype}")
+    check(d, {"r": ids}, got, dtype, f"whole {name} {dtype}", against_whole=False)
     eng.cache.check()
     assert eng.cache.free_pages() == eng.cache.pools[0].num_pages
 
@@ -141,8 +158,8 @@ def test_mixed_with_page_reuse(model_dirs, name, dtype):
     steps = mixed_schedule(seqs, rng)
     assert max(len(e) for e, _ in steps) >= 3
     assert any(len(t) > 1 for e, _ in steps for _, t, _ in e) and any(len(t) == 1 for e, _ in steps for _, t, _ in e)
-    # pool: four live requests of at most 90 tokens, each rounded up to 64: 4 * 128 tokens
-    eng = make_engine(d, dtype, max_tokens=512, max_requests=4, page_size=16)
+    # pool: any four live requests hold at most 6 + 6 + 5 + 4 pages of 16 tokens
+    eng = make_engine(d, dtype, max_tokens=384, max_requests=4, page_size=16)
     total_pages = sum(-(-len(s) // 16) for s in seqs.values())
     assert total_pages > eng.cache.pools[0].num_pages, "the pool must be too small to avoid reuse"
     got = run_steps(eng, steps)
