@@ -42,6 +42,7 @@ class StepBatch:
     slots: List[int] = field(default_factory=list)
     max_q: int = 0
     max_seq: int = 0
+    decode_graph: bool = False   # metadata lives in static buffers that a captured graph replays over
 
 
 class BatchStager:

@@ -1,0 +1,164 @@
+"""Steady decoding of a fixed set of live requests: one token per request per step, sampled on the
+device and fed back on the device, the whole step replayed as one captured HIP graph.
+
+The step is the engine's own: `model.forward` over a `StepBatch` whose metadata lives in static
+device buffers.  What changes between steps (positions, cached lengths, the sampled ids, the random
+draws) is updated by a kernel at the end of the step, so a replay needs no host work; pages for all
+steps of a `run` are reserved, and the block tables uploaded, before the first of them.
+"""
+from __future__ import annotations
+
+from typing import Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..sampling.rng import request_key, uniform
+from ..sampling.sampler import SamplingParams
+from .batch import StepBatch
+from .engine import Engine, OutOfPages, StepError
+
+
+class DecodeLoop:
+    def __init__(self, engine: Engine, rids: Sequence[Hashable], last_tokens: Sequence[int],
+                 params: Optional[Sequence[SamplingParams]] = None, use_graph: bool = True,
+                 max_steps: int = 4096, first_index: Optional[Sequence[int]] = None):
+        """`rids`: live requests whose prompts are cached; `last_tokens`: the token each one feeds
+        next (sampled from its last logits).  `params`: per-request sampling (default greedy);
+        `first_index`: for sampled requests, the output index of their next token (for the draws)."""
+        self.engine, self.rids = engine, list(rids)
+        b = self.n = len(self.rids)
+        if b == 0 or len(last_tokens) != b:
+            raise StepError("a decode loop needs one last token per request")
+        for rid in self.rids:
+            if rid not in engine.cache:
+                raise StepError(f"request {rid!r} is not live")
+        self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * b
+        self.greedy = all(p.greedy for p in self.params)
+        self.index = list(first_index) if first_index is not None else [0] * b
+        self.use_graph = use_graph
+        self.capacity = max_steps
+        cm, dev = engine.cache, engine.device
+        self.width = [cm.pages_for(engine.ctx_limit) for _ in range(cm.n_groups)]
+        # static metadata: ids pos row_req cu ctx slot logit_rows tables...
+        sizes = [b, b, b, b + 1, b, b, b] + [b * w for w in self.width]
+        offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])
+        self._host = np.zeros(int(offs[-1]), dtype=np.int32)
+        self._dev = torch.zeros(int(offs[-1]), dtype=torch.int32, device=dev)
+        sec = lambda i: slice(int(offs[i]), int(offs[i]) + sizes[i])
+        self._sec = [sec(i) for i in range(len(sizes))]
+        h = self._host
+        h[self._sec[0]] = np.asarray(last_tokens, dtype=np.int32)
+        lens = np.array([cm.tokens(r) for r in self.rids], dtype=np.int32)
+        h[self._sec[1]] = lens
+        h[self._sec[2]] = np.arange(b)
+        h[self._sec[3]] = np.arange(b + 1)
+        h[self._sec[4]] = lens
+        h[self._sec[5]] = [cm.slot(r) for r in self.rids]
+        h[self._sec[6]] = np.arange(b)
+        self._fill_tables()
+        self._dev.copy_(torch.from_numpy(h))
+        d = self._dev
+        self.batch = StepBatch(
+            n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
+            cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
+            tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
+            q_lens=[1] * b, ctx_lens=lens.tolist(), slots=h[self._sec[5]].tolist(), max_q=1,
+            max_seq=engine.ctx_limit, decode_graph=True)
+        self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
+        self.counter = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.steps_done = 0
+        if not self.greedy:
+            self.temperature = torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32, device=dev)
+            self.top_p = torch.tensor([p.resolved_top_p for p in self.params], dtype=torch.float32, device=dev)
+            self.top_k = torch.tensor([p.top_k for p in self.params], dtype=torch.int32, device=dev)
+            self.u_all = torch.zeros((self.capacity, b), dtype=torch.float32, device=dev)
+            self.u = torch.zeros(b, dtype=torch.float32, device=dev)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+
+    # ------------------------------------------------------------------ host side
+    def _fill_tables(self) -> None:
+        cm = self.engine.cache
+        for g, w in enumerate(self.width):
+            self._host[self._sec[7 + g]] = cm.block_table(self.rids, g, w).reshape(-1)
+
+    def _reserve(self, n_steps: int) -> None:
+        cm = self.engine.cache
+        for rid in self.rids:
+            if cm.tokens(rid) + self.pending + n_steps > self.engine.ctx_limit:
+                raise StepError(f"request {rid!r} would pass the context limit {self.engine.ctx_limit}")
+        need = [0] * cm.n_groups
+        for rid in self.rids:
+            for g, k in enumerate(cm.pages_needed(rid, self.pending + n_steps)):
+                need[g] += k
+        for g, k in enumerate(need):
+            if k > cm.free_pages(g):
+                raise OutOfPages(f"{n_steps} decode steps need {k} pages of cache group {g}, {cm.free_pages(g)} are free")
+        grew = any(need)
+        for rid in self.rids:
+            assert cm.reserve(rid, self.pending + n_steps)
+        if grew:
+            self._fill_tables()
+            for g in range(cm.n_groups):
+                s = self._sec[7 + g]
+                self._dev[s].copy_(torch.from_numpy(self._host[s]))
+
+    pending = 0         # steps run on the device whose tokens the cache manager has not counted yet
+
+    # ------------------------------------------------------------------ one step on the device
+    def _step(self) -> None:
+        logits = self.engine.model.forward(self.batch, self.engine._views)
+        if self.greedy:
+            ops.argmax(logits, out=self.batch.ids)
+            ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, None, None, self.n)
+        else:
+            ops.sample(logits, self.temperature, self.top_p, self.top_k, self.u, out=self.batch.ids)
+            ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, self.u, self.u_all,
+                        self.n)
+
+    def run(self, n_steps: int) -> None:
+        """Runs `n_steps` decode steps; tokens collect on the device (see `tokens`)."""
+        if self.steps_done + n_steps > self.capacity:
+            raise StepError(f"the decode loop was made for {self.capacity} steps")
+        self._reserve(n_steps)
+        if not self.greedy:
+            rows = np.array([[uniform(p.seed, request_key(r), self.index[i] + self.steps_done + s)
+                              for i, (r, p) in enumerate(zip(self.rids, self.params))]
+                             for s in range(n_steps)], dtype=np.float32)
+            self.u_all[self.steps_done:self.steps_done + n_steps].copy_(torch.from_numpy(rows))
+            self.u.copy_(self.u_all[self.steps_done])
+        if self.use_graph and self.graph is None:
+            # warm up outside capture (lazy initialisation inside libraries), then capture one step
+            # (the warm-up step is undone: metadata and per-request state are put back; its key and
+            # value writes are rewritten with the same values by the first replay)
+            arena = self.engine.device_cache.arena
+            state = self._dev.clone(), self.counter.clone(), self.log.clone(), arena.clone()
+            self._step()
+            torch.cuda.synchronize()
+            self._dev.copy_(state[0]); self.counter.copy_(state[1]); self.log.copy_(state[2]); arena.copy_(state[3])
+            if not self.greedy:
+                self.u.copy_(self.u_all[self.steps_done])
+            g = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with torch.cuda.graph(g):
+                self._step()
+            self.graph = g                                  # the capture itself ran nothing
+        for _ in range(n_steps):
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self._step()
+        self.pending += n_steps
+        self.steps_done += n_steps
+        self.sync_cache()
+
+    def sync_cache(self) -> None:
+        """Tells the cache manager about the positions the device has filled."""
+        for rid in self.rids:
+            self.engine.cache.commit(rid, self.pending)
+        self.pending = 0
+
+    def tokens(self) -> List[List[int]]:
+        """Tokens sampled so far, per request (row s of the log is what step s sampled)."""
+        return self.log[:self.steps_done].cpu().numpy().T.tolist()

@@ -1,0 +1,105 @@
+"""Generation through the scheduler: the Python entry point and what the command line prints.
+
+`Generator` ties an `Engine` to a `ContinuousBatchScheduler` and a `Sampler`, in the manner of the
+reference's one-shot path (/root/reference/src/scheduler/mod.rs:1080-1120,
+/root/reference/src/main.rs:741-772): submit, step until done, report prefill and decode speed.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import torch
+
+from ..sampling.sampler import Draw, Sampler, SamplingParams
+from .batch import Entry
+from .engine import Engine
+from .scheduler import MAX_PREFILL_CHUNK, ContinuousBatchScheduler, FinishReason, StepOutput
+
+
+@dataclass
+class Generation:
+    rid: Hashable
+    prompt_tokens: List[int]
+    tokens: List[int]
+    finish_reason: str
+    error: Optional[str] = None
+    preemptions: int = 0
+
+
+@dataclass
+class GenerationStats:
+    prefill_tokens: int = 0
+    prefill_seconds: float = 0.0
+    decode_tokens: int = 0
+    decode_seconds: float = 0.0
+    steps: int = 0
+
+    @property
+    def prefill_tok_s(self) -> float:
+        return self.prefill_tokens / max(self.prefill_seconds, 1e-9)
+
+    @property
+    def decode_tok_s(self) -> float:
+        return self.decode_tokens / max(self.decode_seconds, 1e-9)
+
+
+class Generator:
+    def __init__(self, engine: Engine, *, max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
+                 eos_token_ids: Optional[Sequence[int]] = None):
+        self.engine = engine
+        self.sampler = Sampler(engine.device)
+        eos = engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids
+        self.scheduler = ContinuousBatchScheduler(engine.cache, self._run, context_len=engine.ctx_limit,
+                                                  max_batch_tokens=max_batch_tokens, chunk=chunk, eos_token_ids=eos)
+        self.stats = GenerationStats()
+
+    def _run(self, entries: Sequence[Entry], draws: Sequence[Draw]) -> List[int]:
+        logits = self.engine.step(entries)
+        if logits is None:
+            return []
+        return self.sampler.sample(logits, draws)
+
+    def submit(self, prompt_tokens: Sequence[int], params: Optional[SamplingParams] = None,
+               rid: Optional[Hashable] = None) -> Hashable:
+        return self.scheduler.submit(prompt_tokens, params, rid)
+
+    def step(self) -> StepOutput:
+        """One scheduler step, timed: a step that holds prompt tokens counts as prefill (with its
+        decoded tokens riding along), any other as decode."""
+        torch.cuda.synchronize(self.engine.device)
+        t0 = time.perf_counter()
+        out = self.scheduler.step()
+        torch.cuda.synchronize(self.engine.device)
+        dt = time.perf_counter() - t0
+        self.stats.steps += 1
+        if out.prefill_tokens:
+            self.stats.prefill_tokens += out.prefill_tokens
+            self.stats.prefill_seconds += dt
+        elif out.decode_tokens:
+            self.stats.decode_tokens += out.decode_tokens
+            self.stats.decode_seconds += dt
+        return out
+
+    def run(self) -> Dict[Hashable, Generation]:
+        while self.scheduler.has_work():
+            self.step()
+        return self.results()
+
+    def results(self) -> Dict[Hashable, Generation]:
+        return {rid: Generation(rid, s.prompt_tokens, list(s.output_tokens),
+                                s.finish_reason.value if s.finish_reason else "stop", s.error, s.preemptions)
+                for rid, s in self.scheduler.finished.items()}
+
+
+def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_tokens: int = 64,
+             temperature: Optional[float] = None, top_p: Optional[float] = None, top_k: int = 50, seed: int = 0,
+             ignore_eos: bool = False, max_batch_tokens: int = MAX_PREFILL_CHUNK,
+             chunk: Optional[int] = None) -> List[Generation]:
+    """Generates a continuation of every prompt (lists of token ids), batched continuously."""
+    gen = Generator(engine, max_batch_tokens=max_batch_tokens, chunk=chunk)
+    params = SamplingParams(temperature, top_p, top_k, max_tokens, seed, ignore_eos)
+    rids = [gen.submit(p, params) for p in prompts]
+    results = gen.run()
+    return [results[r] for r in rids]

@@ -216,3 +216,20 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     call("gibbs_sample", ptr(logits), ptr(out), m, v, logits.stride(0) if m > 1 else v, ptr(temperature),
          ptr(top_p), ptr(top_k), ptr(u), stream())
     return out
+
+
+def advance(pos: torch.Tensor, ctx: torch.Tensor, ids: torch.Tensor, log: torch.Tensor, counter: torch.Tensor,
+            u: Optional[torch.Tensor], u_all: Optional[torch.Tensor], n: int) -> None:
+    """End of a decode step on the device: logs the tokens in `ids`, moves pos and ctx on by one,
+    loads the next step's draws and counts the step."""
+    require_cuda(pos, ctx, ids, log, counter, u, u_all)
+    for t, what in ((pos, "pos"), (ctx, "ctx"), (ids, "ids")):
+        _i32(t, n, what)
+    _i32(counter, 1, "counter")
+    assert log.dtype == torch.int32 and log.is_contiguous() and log.numel() % n == 0
+    capacity = log.numel() // n
+    if u is not None:
+        assert u.dtype == torch.float32 and u.numel() >= n and u_all is not None
+        assert u_all.dtype == torch.float32 and u_all.is_contiguous() and u_all.numel() >= capacity * n
+    call("gibbs_advance", ptr(pos), ptr(ctx), ptr(ids), ptr(log), ptr(counter), ptr(u), ptr(u_all), n, capacity,
+         stream())

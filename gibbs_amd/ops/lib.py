@@ -36,6 +36,7 @@ _SIGNATURES = {
                          c_void_p],
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p],
+    "gibbs_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gibbs_sample": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
 }

@@ -75,6 +75,13 @@ class AttentionMixer(Mixer):
         if self.position is not None:
             self.position.bind(weights, rt)
 
+    def matrices(self):
+        return [self.w_qkv, self.w_out]
+
+    def small_tensors(self):
+        return [t for t in (self.q_gain, self.k_gain, None if self.position is None else self.position.inv_freq)
+                if t is not None]
+
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         n = batch.n_rows

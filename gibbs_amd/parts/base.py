@@ -40,6 +40,15 @@ class Part:
         """Takes its tensors from the store and prepares the layouts its kernels want."""
         self.rt = rt
 
+    def matrices(self) -> List[torch.Tensor]:
+        """The matrices [out, in] that every row of a step is multiplied with (what a decode step
+        has to stream, and 2 * numel flops per row)."""
+        return []
+
+    def small_tensors(self) -> List[torch.Tensor]:
+        """Gains, biases, taps and tables that a step also reads."""
+        return []
+
 
 class Norm(Part):
     def __init__(self, spec: NormSpec, width: int):
@@ -104,6 +113,12 @@ class Block(Part):
         self.rt = rt
         for p in self.parts():
             p.bind(weights, rt)
+
+    def matrices(self) -> List[torch.Tensor]:
+        return [m for p in self.parts() for m in p.matrices()]
+
+    def small_tensors(self) -> List[torch.Tensor]:
+        return [m for p in self.parts() for m in p.small_tensors()]
 
     def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], batch, cache) -> torch.Tensor:
         """x: float32 residual stream, updated in place; `pending`: the previous block's last delta,

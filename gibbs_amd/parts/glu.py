@@ -33,6 +33,9 @@ class GluFeedForward(FeedForward):
         self.w_gate_up = torch.cat([weights[t["gate"]], weights[t["up"]]], dim=0).contiguous()
         self.w_down = weights[t["down"]]
 
+    def matrices(self):
+        return [self.w_gate_up, self.w_down]
+
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         gu = linear(h, self.w_gate_up)
         return linear(ops.glu(gu, self.activation), self.w_down)

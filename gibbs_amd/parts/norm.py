@@ -23,3 +23,6 @@ class RMSNorm(Norm):
 
     def forward(self, x, delta, rows=None, n_rows=None):
         return ops.add_rmsnorm(x, delta, self.gain, self.spec.eps, self.rt.act_dtype, rows, n_rows)
+
+    def small_tensors(self):
+        return [self.gain]

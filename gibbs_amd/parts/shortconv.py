@@ -51,6 +51,12 @@ class ShortConvMixer(Mixer):
         self.w_out = weights[t["out_proj"]]
         self.conv_bias = weights[t["conv_bias"]] if self.bias else None
 
+    def matrices(self):
+        return [self.w_in, self.w_out]
+
+    def small_tensors(self):
+        return [self.taps] + ([self.conv_bias] if self.bias else [])
+
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         bcx = linear(h, self.w_in)
         y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,

@@ -1,0 +1,63 @@
+"""What a step must at least move and compute, for the roofline figures of the bench and the
+command line (the reference reports decode speed against bytes-per-token at a bandwidth ceiling,
+/root/reference/src/bench.rs:298-308)."""
+from __future__ import annotations
+
+from typing import Sequence
+
+# MI355X's published peaks.
+HBM_BYTES_PER_S = 8.0e12
+PEAK_FLOPS = {"bfloat16": 2.5e15, "float16": 2.5e15, "float8": 5.0e15, "float32": 157.3e12}
+
+
+def _nbytes(t) -> int:
+    return t.numel() * t.element_size()
+
+
+def weight_bytes_per_step(engine) -> int:
+    """Every weight a decode step uses, once: the matrices and small tensors of every run of the
+    layer order, the final norm and the head matrix.  (The token table is read by rows only,
+    unless it is also the head.)"""
+    m = engine.model
+    total = 0
+    for i in m.spec.order:
+        b = m.blocks[i]
+        total += sum(_nbytes(t) for t in b.matrices()) + sum(_nbytes(t) for t in b.small_tensors())
+    total += sum(_nbytes(t) for t in m.final_norm.small_tensors())
+    total += _nbytes(m.head)
+    return total
+
+
+def cache_bytes(engine, seq_lens: Sequence[int]) -> int:
+    """Keys and values that the live requests' next tokens attend over, and their state slots."""
+    cm = engine.cache
+    elem = engine.device_cache.pages[0].element_size() if engine.device_cache.pages else 0
+    total = 0
+    for g, need in enumerate(cm.group_needs):
+        per_token = 2 * need.kv_heads * need.head_dim * elem * len(cm.group_layers[g])
+        for n in seq_lens:
+            total += per_token * (n if need.window is None else min(n, need.window))
+    total += len(seq_lens) * cm.slot_floats * 4
+    return total
+
+
+def decode_bytes(engine, seq_lens: Sequence[int]) -> int:
+    return weight_bytes_per_step(engine) + cache_bytes(engine, seq_lens)
+
+
+def prefill_flops(engine, n_tokens: int, n_logit_rows: int = 1, start: int = 0) -> float:
+    """Multiply-adds x 2 of a prompt portion of `n_tokens` rows starting at position `start`:
+    every matrix once per row, the head for the wanted rows, and causal attention (each row over
+    the keys up to its own position)."""
+    m = engine.model
+    flops = 0.0
+    keys = sum(start + t + 1 for t in range(n_tokens))
+    for i in m.spec.order:
+        b = m.blocks[i]
+        flops += 2.0 * n_tokens * sum(t.numel() for t in b.matrices())
+        need = b.mixer.cache_need()
+        if need is not None or b.mixer.kv_source() is not None:
+            heads, hd = b.mixer.heads, b.mixer.head_dim
+            flops += 2.0 * 2.0 * keys * heads * hd
+    flops += 2.0 * n_logit_rows * m.head.numel()
+    return flops

@@ -56,3 +56,30 @@ def write_random_model(folder: str, config: ArchConfig, decls: Iterable[TensorDe
         json.dump(config.to_dict(), f, indent=1)
     tensors = ((d.name, random_tensor(d, seed, store, std, gain_std, bias_std)) for d in decls)
     write_safetensors(os.path.join(folder, "model.safetensors"), list(tensors))
+
+
+def random_weights_on_device(decls: Iterable[TensorDecl], seed: int, compute_dtype: torch.dtype,
+                             device: torch.device | str, std: float = 0.02, gain_std: float = 0.0,
+                             bias_std: float = 0.02):
+    """The same kinds of random tensors, made on the device without a model folder (benchmarks of
+    large shapes).  Values differ from the folder mode's: the device has its own generator."""
+    from .loader import WeightStore
+    device = torch.device(device)
+    out: Dict[str, torch.Tensor] = {}
+    for d in decls:
+        g = torch.Generator(device=device)
+        g.manual_seed(_stream(d.name, seed).initial_seed())
+        want = d.resolved_dtype(compute_dtype)
+        if d.dtype == INT32:
+            out[d.name] = torch.zeros(d.shape, dtype=torch.int32, device=device)
+        elif d.init == "gain":
+            t = torch.ones(d.shape, dtype=torch.float32, device=device)
+            if gain_std > 0:
+                t += torch.randn(d.shape, generator=g, dtype=torch.float32, device=device) * gain_std
+            out[d.name] = t.to(want)
+        elif d.init == "zeros":
+            out[d.name] = torch.zeros(d.shape, dtype=want, device=device)
+        else:
+            scale = bias_std if d.init == "bias" else std
+            out[d.name] = (torch.randn(d.shape, generator=g, dtype=torch.float32, device=device) * scale).to(want)
+    return WeightStore(out, compute_dtype, device)

@@ -65,7 +65,7 @@ class SafetensorsFile:
         e = self.entries[name]
         if self._map is None:
             with open(self.path, "rb") as f:
-                self._map = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_READ)
+                self._map = mmap.mmap(f.fileno(), 0, access=mmap.ACCESS_COPY)
         dtype = _TORCH_DTYPES[e.dtype]
         count = int(np.prod(e.shape)) if e.shape else 1
         if count == 0:
