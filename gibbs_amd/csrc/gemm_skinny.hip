@@ -1,0 +1,138 @@
+// Matrix product for few rows (decode: one row per live request, up to 64):
+//   Y[n, o] = sum_k X[n, k] * W[o, k],  bfloat16 operands, float32 accumulation.
+// The work is reading W once, so the layout serves that: a workgroup owns 16 output features and a
+// range of k; its 8 waves split the range, each streaming its part of the 16 rows of W straight
+// from memory into the A operand of v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of one
+// row, so no LDS staging is needed), with X (small, cache resident) as the B operand: 16 rows of
+// X per MFMA, NT such tiles for up to 64 rows.  The waves' sums meet in LDS.  When 16-feature
+// blocks alone cannot fill the chip, k is also split over workgroups (`k_splits`), each writing
+// its float32 partial Y[s] for the consumer to add in a fixed order.
+#include "common.h"
+
+namespace {
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+enum { OUT_BF16 = 0, OUT_F32 = 1 };
+constexpr int WAVES = 8;
+
+template <int NT, int OUT>
+__global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ W, const bf16* __restrict__ X,
+                                                          void* __restrict__ Yv, int N, int O, int I, long ldw,
+                                                          long ldx, long ldy, int k_per_block, long split_stride) {
+  __shared__ floatx4 red[WAVES - 1][NT][WAVE];
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int o0 = blockIdx.x * 16;
+  const int kb0 = blockIdx.y * k_per_block;
+  const int kb1 = min(I, kb0 + k_per_block);
+  // the wave's share of the block's range, in whole MFMA steps of 32
+  const int steps = (kb1 - kb0 + 31) / 32;
+  const int per_wave = (steps + WAVES - 1) / WAVES;
+  const int k_begin = kb0 + wave * per_wave * 32;
+  const int k_end = min(kb1, k_begin + per_wave * 32);
+
+  const bool row_ok = o0 + r < O;
+  const bf16* wrow = W + (size_t)(row_ok ? o0 + r : 0) * ldw + g * 8;
+  const bf16* xrow[NT];
+  bool x_ok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    x_ok[t] = t * 16 + r < N;
+    xrow[t] = X + (size_t)(x_ok[t] ? t * 16 + r : 0) * ldx + g * 8;
+  }
+  floatx4 acc[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int U = 4;  // MFMA steps per iteration: 4 loads of W in flight per lane
+  for (int k = k_begin; k < k_end; k += 32 * U) {
+    bf16x8 a[U], b[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k + u * 32;
+      const bool k_ok = kk + g * 8 < k_end;
+      a[u] = (row_ok && k_ok) ? *(const bf16x8*)(wrow + kk) : zero;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][t], acc[t], 0, 0, 0);
+  }
+
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave - 1][t][lane] = acc[t];
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+#pragma unroll
+    for (int w = 0; w < WAVES - 1; ++w) acc[t] += red[w][t][lane];
+    // D[feature (lane/16)*4 + i][row lane%16]: 4 consecutive features of one row of Y
+    const int n = t * 16 + r, o = o0 + g * 4;
+    if (n >= N) continue;
+    if (OUT == OUT_BF16) {
+      bf16* y = (bf16*)Yv + (size_t)n * ldy + o;
+      if (o + 3 < O && (ldy % 4 == 0)) {
+        typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+        bf16x4 v = {(bf16)acc[t][0], (bf16)acc[t][1], (bf16)acc[t][2], (bf16)acc[t][3]};
+        *(bf16x4*)y = v;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (o + i < O) y[i] = (bf16)acc[t][i];
+      }
+    } else {
+      float* y = (float*)Yv + (size_t)blockIdx.y * split_stride + (size_t)n * ldy + o;
+      if (o + 3 < O && (ldy % 4 == 0)) {
+        *(floatx4*)y = acc[t];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (o + i < O) y[i] = acc[t][i];
+      }
+    }
+  }
+}
+
+template <int NT>
+void launch(int out, dim3 grid, hipStream_t s, const bf16* W, const bf16* X, void* Y, int N, int O, int I, long ldw,
+            long ldx, long ldy, int kpb, long ss) {
+  if (out == OUT_BF16)
+    gemm_skinny_kernel<NT, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else
+    gemm_skinny_kernel<NT, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+}
+}  // namespace
+
+// X: [N <= 64, I], W: [O, I] bfloat16.  k_splits == 1: Y [N, O] bfloat16 (out_dtype 1) or float32 (0).
+// k_splits > 1: Y is float32 [k_splits, N, O] (split stride N * ldy): partial sums over k ranges.
+GIBBS_EXPORT int gibbs_gemm_skinny(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx,
+                                   long ldw, long ldy, int k_splits, hipStream_t stream) {
+  GIBBS_REQUIRE(N > 0 && N <= 64 && O > 0 && I > 0, "gemm_skinny: bad sizes N=%d O=%d I=%d (N up to 64)", N, O, I);
+  GIBBS_REQUIRE(I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: inner size %d and row strides (%ld, %ld) must be multiples of 8", I, ldx, ldw);
+  GIBBS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny: operands must be 16-byte aligned");
+  GIBBS_REQUIRE(ldx >= I && ldw >= I && ldy >= O, "gemm_skinny: row strides shorter than rows");
+  GIBBS_REQUIRE(k_splits >= 1 && k_splits <= 1024, "gemm_skinny: %d k splits", k_splits);
+  GIBBS_REQUIRE(k_splits == 1 || out_dtype == GIBBS_F32, "gemm_skinny: partial sums are float32");
+  GIBBS_REQUIRE(out_dtype == GIBBS_F32 || out_dtype == GIBBS_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
+  // each block's k range is a whole number of 128-element steps (what one wave does per iteration)
+  int kpb = ceil_div(ceil_div(I, k_splits), 128) * 128;
+  const int used = ceil_div(I, kpb);
+  GIBBS_REQUIRE(used == k_splits, "gemm_skinny: %d k splits leave some empty for inner size %d (use %d)", k_splits, I, used);
+  dim3 grid(ceil_div(O, 16), k_splits);
+  const int out = out_dtype == GIBBS_BF16 ? OUT_BF16 : OUT_F32;
+  const long ss = (long)N * ldy;
+  const bf16 *w = (const bf16*)W, *x = (const bf16*)X;
+  const int nt = ceil_div(N, 16);
+  if (nt == 1) launch<1>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else if (nt == 2) launch<2>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else if (nt == 3) launch<3>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else launch<4>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  GIBBS_LAUNCH_STATUS("gemm_skinny");
+}

@@ -49,6 +49,57 @@ GIBBS_EXPORT int gibbs_add_rmsnorm(float* x, const void* delta, const float* gai
   GIBBS_LAUNCH_STATUS("rmsnorm");
 }
 
+// The same with the delta given as float32 partial sums of a product split over k:
+// delta[r] = sum_s partials[s][r], added in ascending s.
+template <typename T>
+__global__ void add_partials_rmsnorm_kernel(float* __restrict__ x, const float* __restrict__ partials, int n_partials,
+                                            long partial_stride, const float* __restrict__ gain, float eps,
+                                            T* __restrict__ out, const int* __restrict__ rows, int hidden,
+                                            int write_x) {
+  __shared__ float scratch[16];
+  const int m = blockIdx.x;
+  const int r = rows ? rows[m] : m;
+  float* xr = x + (size_t)r * hidden;
+  const float* pr = partials + (size_t)r * hidden;
+  T* o = out + (size_t)m * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float d = 0.f;
+    for (int s = 0; s < n_partials; ++s) d += pr[(size_t)s * partial_stride + i];
+    const float v = xr[i] + d;
+    if (write_x) xr[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float scale = 1.0f / sqrtf(ss / (float)hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = xr[i];
+    if (!write_x) {
+      float d = 0.f;
+      for (int s = 0; s < n_partials; ++s) d += pr[(size_t)s * partial_stride + i];
+      v += d;
+    }
+    o[i] = from_float<T>(v * scale * gain[i]);
+  }
+}
+
+// partials: [n_partials, n_x, hidden] float32 (stride between partials given in elements).
+GIBBS_EXPORT int gibbs_add_partials_rmsnorm(float* x, const float* partials, int n_partials, long partial_stride,
+                                            const float* gain, float eps, void* out, int dtype, const int* rows,
+                                            int n_out, int hidden, hipStream_t stream) {
+  GIBBS_REQUIRE(n_out >= 0 && hidden > 0 && n_partials >= 1, "rmsnorm: bad sizes n=%d hidden=%d partials=%d", n_out, hidden, n_partials);
+  if (n_out == 0) return 0;
+  const int threads = hidden >= 2048 ? 512 : (hidden >= 512 ? 256 : 64);
+  const int write_x = rows == nullptr;
+  if (dtype == GIBBS_F32)
+    add_partials_rmsnorm_kernel<float><<<n_out, threads, 0, stream>>>(x, partials, n_partials, partial_stride, gain, eps, (float*)out, rows, hidden, write_x);
+  else if (dtype == GIBBS_BF16)
+    add_partials_rmsnorm_kernel<bf16><<<n_out, threads, 0, stream>>>(x, partials, n_partials, partial_stride, gain, eps, (bf16*)out, rows, hidden, write_x);
+  else
+    return gibbs_fail("rmsnorm: unknown dtype %d", dtype);
+  GIBBS_LAUNCH_STATUS("rmsnorm");
+}
+
 // x[r] += delta[r] alone (the last residual add of a model whose tail norms only some rows
 // still has to leave x whole for callers that read it).
 template <typename T>

@@ -34,12 +34,16 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, n_out: Optional[int] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """v = x (+ delta); x <- v when all rows are normed; out = v * rsqrt(mean(v^2) + eps) * gain.
-    With `rows`, only those rows are normed (and x is left as it is)."""
+    With `rows`, only those rows are normed (and x is left as it is).  `delta` is [N, H] in the
+    output dtype, or float32 [S, N, H]: partial sums that are added in ascending s."""
     require_cuda(x, delta, gain, rows)
     n, hidden = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
     assert gain.dtype == torch.float32 and gain.shape == (hidden,) and gain.is_contiguous()
-    if delta is not None:
+    partials = delta is not None and delta.dim() == 3
+    if partials:
+        assert delta.dtype == torch.float32 and delta.shape[1:] == x.shape and delta.is_contiguous()
+    elif delta is not None:
         assert delta.shape == x.shape and delta.dtype == out_dtype and delta.is_contiguous()
     if rows is None:
         n_out = n
@@ -49,6 +53,10 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
     if out is None:
         out = torch.empty((n_out, hidden), dtype=out_dtype, device=x.device)
     assert out.shape == (n_out, hidden) and out.dtype == out_dtype and out.is_contiguous()
+    if partials:
+        call("gibbs_add_partials_rmsnorm", ptr(x), ptr(delta), delta.shape[0], delta.stride(0), ptr(gain), float(eps),
+             ptr(out), dtype_code(out_dtype), ptr(rows), n_out, hidden, stream())
+        return out
     call("gibbs_add_rmsnorm", ptr(x), ptr(delta), ptr(gain), float(eps), ptr(out), dtype_code(out_dtype),
          ptr(rows), n_out, hidden, stream())
     return out
@@ -94,6 +102,43 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     assert out.shape == (n, o) and out.dtype == out_dtype and out.stride(1) == 1
     call("gibbs_gemm_bf16", ptr(a), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i, lda, w.stride(0),
          out.stride(0) if n > 1 else o, stream())
+    return out
+
+
+def skinny_splits(n_out: int, inner: int, want_blocks: int = 512) -> int:
+    """How many ranges of k `gemm_skinny` should cut a product into so that at least `want_blocks`
+    workgroups run (a workgroup owns 16 output features), each with at least 1024 of k."""
+    blocks = -(-n_out // 16)
+    s = max(1, min(-(-want_blocks // blocks), inner // 1024))
+    per = -(-(-(-inner // s)) // 128) * 128
+    return -(-inner // per)
+
+
+def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, k_splits: int = 1,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x @ w^T for at most 64 rows of x, streaming w once.  k_splits > 1 returns float32
+    partial sums [k_splits, N, O] (ranges of k) for the consumer to add."""
+    require_cuda(x, w)
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], (x.shape, w.shape)
+    assert x.stride(1) == 1 and w.stride(1) == 1
+    n, i = x.shape
+    o = w.shape[0]
+    if not 1 <= n <= 64:
+        raise KernelError(f"gemm_skinny takes 1..64 rows, not {n}")
+    ldx = x.stride(0) if n > 1 else i
+    if i % 8 or ldx % 8 or w.stride(0) % 8:
+        raise KernelError(f"gemm_skinny: inner size {i} and row strides must be multiples of 8")
+    if k_splits > 1:
+        out_dtype = torch.float32
+        shape = (k_splits, n, o)
+    else:
+        shape = (n, o)
+    if out is None:
+        out = torch.empty(shape, dtype=out_dtype, device=x.device)
+    assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
+    call("gibbs_gemm_skinny", ptr(x), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i, ldx, w.stride(0), o, k_splits,
+         stream())
     return out
 
 
@@ -186,6 +231,46 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
     call("gibbs_attention_plain", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
          ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
          q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), stream())
+    return out
+
+
+def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int) -> int:
+    """Key slices per (row, kv head) for the decode attention: enough workgroups to fill 256 compute
+    units a few times over, but at least 64 keys to a slice."""
+    gt = 8 if group >= 8 else (4 if group > 2 else group)
+    per_split = n_rows * nkv * -(-group // gt)
+    want = -(-1024 // per_split)
+    return max(1, min(want, max_seq // 64, 256))
+
+
+def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
+                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
+                     scale: float, window: Optional[int] = None, max_seq: int = 0, n_splits: Optional[int] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bfloat16 paged attention for rows with few queries and long caches (decoded tokens): the
+    keys of each (row, kv head) are cut into `n_splits` slices that run as workgroups of their own
+    and are merged afterwards.  Same operands and result as `attention_plain`."""
+    require_cuda(q, kpages, vpages, table, pos, row_req)
+    if q.dtype != torch.bfloat16:
+        raise KernelError("attention_decode is the bfloat16 kernel; the float32 path uses attention_plain")
+    assert q.dim() == 2 and q.shape[0] == n_rows and q.stride(1) == 1 and q.shape[1] >= nh * hd
+    if hd % 8 or hd > 256:
+        raise KernelError(f"attention_decode: head size {hd} must be a multiple of 8 up to 256")
+    num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
+    assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
+    assert table.dim() == 2 and table.shape[0] >= n_req
+    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    if n_splits is None:
+        n_splits = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+    partial = None
+    if n_splits > 1:
+        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=q.device)
+    if out is None:
+        out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
+    assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
+    call("gibbs_attention_decode", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(pos), ptr(row_req),
+         ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, stream())
     return out
 
 

@@ -28,6 +28,10 @@ _SIGNATURES = {
     "gibbs_residual_add": [c_void_p, c_void_p, c_int, c_long, c_void_p],
     "gibbs_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
+    "gibbs_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
+                          c_void_p],
+    "gibbs_add_partials_rmsnorm": [c_void_p, c_void_p, c_int, c_long, c_void_p, c_float, c_void_p, c_int, c_void_p,
+                                   c_int, c_int, c_void_p],
     "gibbs_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_shortconv": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                         c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -37,6 +41,9 @@ _SIGNATURES = {
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p],
     "gibbs_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
+                               c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gibbs_sample": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
 }

@@ -1,8 +1,9 @@
 """y = x @ W^T for weights stored [out, in], in the precision of the run.
 
 float32: the hand-written plain-FMA kernel (a true 32-bit product whose per-row result does not
-depend on the batch).  bfloat16: float32 accumulation; the output is bfloat16, or float32 where
-the caller asks for it (logits).
+depend on the batch).  bfloat16: matrix cores with float32 accumulation; up to 64 rows take the
+kernel that streams W once (decode), more rows the tiled kernel (prefill).  The output is
+bfloat16, or float32 where the caller asks for it (logits).
 """
 from __future__ import annotations
 
@@ -10,11 +11,17 @@ from typing import Optional
 
 import torch
 
-from . import gemm_bf16, gemm_f32
+from . import gemm_bf16, gemm_f32, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
+SKINNY_ROWS = 64
 
-def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+
+def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
+           partial_ok: bool = False) -> torch.Tensor:
+    """`partial_ok`: the caller can take float32 partial sums [S, N, O] (to be added in order)
+    instead of the finished product; the few-row kernel then also splits k over workgroups when
+    the output alone is too narrow to fill the chip."""
     require_cuda(x, w)
     if x.dtype != w.dtype:
         raise KernelError(f"linear: activations are {x.dtype}, weights {w.dtype}")
@@ -24,5 +31,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
             raise KernelError("linear: the float32 path writes float32")
         return gemm_f32(x, w)
     if x.dtype == torch.bfloat16:
+        if 1 <= x.shape[0] <= SKINNY_ROWS:
+            splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
+            return gemm_skinny(x, w, out_dtype, splits)
         return gemm_bf16(x, w, out_dtype)
     raise KernelError(f"linear: unsupported dtype {x.dtype}")

@@ -98,9 +98,15 @@ class AttentionMixer(Mixer):
                        kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None,
                        table=table, n_req=batch.n_req)
         a = self.attend(qkv, batch, cache, table)
-        return linear(a, self.w_out)
+        return linear(a, self.w_out, partial_ok=True)
 
     def attend(self, qkv, batch, cache, table) -> torch.Tensor:
+        """Attention of the step's rows over the cache.  bfloat16 rows that are all single decoded
+        tokens take the kernel that splits the keys; everything else the plain kernel."""
+        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1:
+            return ops.attention_decode(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
+                                        cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
+                                        self.window, max_seq=batch.max_seq)
         return ops.attention_plain(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
                                    cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
                                    self.window)

@@ -8,7 +8,8 @@ model it is in.  To add a part: subclass the interface, decorate the class with 
 
   Norm            forward(x, delta, rows) -> normed rows in the activation dtype (adds delta first)
   PositionEncoding  tables and parameters that a mixer hands to its kernels
-  Mixer           forward(h, batch, cache) -> delta [N, hidden]; may ask for cache pages
+  Mixer           forward(h, batch, cache) -> delta [N, hidden] (or float32 parts [S, N, hidden]
+                  that the next norm adds in order); may ask for cache pages
                   (`cache_need`) and per-request state of fixed size (`state_needs`)
   FeedForward     forward(h, batch) -> delta [N, hidden]
   Block           forward(x, pending, batch, cache) -> pending delta (arrangement of the above)
@@ -57,7 +58,9 @@ class Norm(Part):
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
                 n_rows: Optional[int] = None) -> torch.Tensor:
         """x (float32 residual stream) += delta (if given and all rows are normed); returns norm(x)
-        in the activation dtype.  With `rows` only those rows (of x + delta) are normed."""
+        in the activation dtype.  With `rows` only those rows (of x + delta) are normed.  `delta` is
+        [N, width] in the activation dtype, or float32 [S, N, width]: parts that are added in
+        ascending s (a product that was split over its inner dimension)."""
         raise NotImplementedError
 
 

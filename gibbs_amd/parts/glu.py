@@ -38,4 +38,4 @@ class GluFeedForward(FeedForward):
 
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         gu = linear(h, self.w_gate_up)
-        return linear(ops.glu(gu, self.activation), self.w_down)
+        return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True)

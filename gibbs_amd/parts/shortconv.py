@@ -61,4 +61,4 @@ class ShortConvMixer(Mixer):
         bcx = linear(h, self.w_in)
         y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,
                           batch.n_rows, batch.n_req)
-        return linear(y, self.w_out)
+        return linear(y, self.w_out, partial_ok=True)

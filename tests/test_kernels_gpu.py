@@ -90,6 +90,59 @@ def test_gemm_bf16(shape, out_dtype):
     close(ops.gemm_bf16(big[:, :i], w, out_dtype), big[:, :i].double() @ w.double().t(), out_dtype, "strided", f32=2e-5, bf16=4e-3)
 
 
+@pytest.mark.parametrize("out_dtype", DT)
+@pytest.mark.parametrize("n,o,i,splits", [(1, 64, 128, 1), (8, 331, 1000, 1), (16, 2048, 2048, 2), (17, 200, 8192, 8),
+                                          (33, 48, 72, 1), (64, 515, 1024, 1), (5, 2048, 8192, 4), (64, 96, 4096, 3)])
+def test_gemm_skinny(n, o, i, splits, out_dtype):
+    from gibbs_amd import ops
+    x, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
+    want = x.double() @ w.double().t()
+    if splits > 1:
+        if out_dtype == torch.bfloat16:
+            pytest.skip("partial sums are float32")
+        parts = ops.gemm_skinny(x, w, torch.float32, splits)
+        assert parts.shape == (splits, n, o)
+        close(parts.sum(0), want, torch.float32, "skinny partial sums", f32=2e-5)
+    got = ops.gemm_skinny(x, w, out_dtype)
+    assert got.dtype == out_dtype and got.shape == (n, o)
+    close(got, want, out_dtype, f"gemm_skinny {(n, o, i)}", f32=2e-5, bf16=4e-3)
+    # a strided view of x (rows of a wider buffer)
+    big = rnd(n, i + 64, dtype=torch.bfloat16, seed=3)
+    close(ops.gemm_skinny(big[:, :i], w, out_dtype), big[:, :i].double() @ w.double().t(), out_dtype, "strided",
+          f32=2e-5, bf16=4e-3)
+
+
+def test_skinny_splits_cover_k():
+    from gibbs_amd import ops
+    for o, i in [(2048, 2048), (2048, 8192), (6144, 2048), (65536, 2048), (96, 96), (200, 1000), (64, 12800)]:
+        s = ops.skinny_splits(o, i)
+        per = -(-(-(-i // s)) // 128) * 128
+        assert s >= 1 and -(-i // per) == s, (o, i, s)
+        x, w = rnd(3, i, dtype=torch.bfloat16), rnd(min(o, 64), i, dtype=torch.bfloat16, seed=1)
+        parts = ops.gemm_skinny(x, w, torch.float32, s)
+        got = parts.sum(0) if s > 1 else parts
+        close(got, x.double() @ w.double().t(), torch.float32, f"splits {s}", f32=2e-5)
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_add_partials_rmsnorm(dtype):
+    from gibbs_amd import ops
+    hidden, n, s = 200, 5, 3
+    x = rnd(n, hidden, scale=2.0)
+    parts = rnd(s, n, hidden, seed=4)
+    gain = rnd(hidden, seed=2) + 1.0
+    x0 = x.clone()
+    out = ops.add_rmsnorm(x, parts, gain, 1e-6, dtype)
+    v = x0 + (parts[0] + parts[1]) + parts[2]
+    close(x, v, torch.float32, "x + partials", f32=1e-6)
+    close(out, F.rms_norm(v.double(), (hidden,), gain.double(), eps=1e-6), dtype, "partials rmsnorm")
+    rows = i32([4, 1])
+    x1 = x.clone()
+    out2 = ops.add_rmsnorm(x, parts, gain, 1e-6, dtype, rows)
+    assert torch.equal(x, x1)
+    close(out2, F.rms_norm((x1 + parts.sum(0))[rows.long()].double(), (hidden,), gain.double(), eps=1e-6), dtype, "rows")
+
+
 def test_gemm_bf16_refuses_unaligned():
     from gibbs_amd import ops
     from gibbs_amd.ops.lib import KernelError
@@ -198,6 +251,30 @@ def test_attention_plain_paged(dtype, nh, nkv, hd, page, window):
         want = attention_reference(q[at:at + len(ps)].view(-1, nh, hd), ks[r], vs[r], ps, scale, window)
         close(out[at:at + len(ps)].view(-1, nh, hd), want, dtype, f"attention request {r}", f32=2e-5, bf16=1e-2)
         at += len(ps)
+
+
+@pytest.mark.parametrize("n_splits", [1, 3, 16, None])
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
+                                                   (32, 8, 64, 16, None), (16, 2, 128, 16, None), (2, 2, 256, 64, 100),
+                                                   (24, 2, 32, 16, None)])
+def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits):
+    """The key-splitting kernel against the float64 reference and against the plain kernel, for
+    rows of different lengths (one key, a page edge, hundreds of keys) in one call."""
+    from gibbs_amd import ops
+    dtype = torch.bfloat16
+    seq_lens = [700, 1, 33, 16]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 120, seed=7)
+    positions = [l - 1 for l in seq_lens]
+    pos, row_req = i32(positions), i32([0, 1, 2, 3])
+    q = rnd(4, nh * hd, dtype=dtype, seed=9)
+    scale = 1 / math.sqrt(hd)
+    out = ops.attention_decode(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window, max_seq=700,
+                               n_splits=n_splits)
+    plain = ops.attention_plain(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window)
+    for r in range(4):
+        want = attention_reference(q[r:r + 1].view(1, nh, hd), ks[r], vs[r], [positions[r]], scale, window)
+        close(out[r].view(1, nh, hd), want, dtype, f"decode attention row {r}", bf16=1e-2)
+    close(out, plain, dtype, "decode vs plain kernel", bf16=1e-2)
 
 
 @pytest.mark.parametrize("dtype", DT)
