@@ -10,7 +10,7 @@
 
 namespace {
 constexpr int MAX_K = 64;
-constexpr int THREADS = 256;
+constexpr int THREADS = 1024;
 
 // Order of candidates: larger value first, then smaller index.  NaN ranks below everything.
 __device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
@@ -41,10 +41,22 @@ __global__ __launch_bounds__(THREADS) void argmax_kernel(const float* __restrict
   const float* row = logits + (size_t)blockIdx.x * ld;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += THREADS) {
-    const float v = row[i];  // NaN fails both comparisons in `better`
-    if (better(v, i, bv, bi)) { bv = v; bi = i; }
+  // 16-byte loads over the aligned middle; NaN fails both comparisons in `better`
+  const int head = min(V, (int)(((16 - ((uintptr_t)row & 15)) & 15) / 4));
+  const int n4 = (V - head) / 4;
+  for (int i = threadIdx.x; i < head; i += THREADS)
+    if (better(row[i], i, bv, bi)) { bv = row[i]; bi = i; }
+  const float4* row4 = (const float4*)(row + head);
+  for (int j = threadIdx.x; j < n4; j += THREADS) {
+    const float4 v = row4[j];
+    const int i = head + 4 * j;
+    if (better(v.x, i, bv, bi)) { bv = v.x; bi = i; }
+    if (better(v.y, i + 1, bv, bi)) { bv = v.y; bi = i + 1; }
+    if (better(v.z, i + 2, bv, bi)) { bv = v.z; bi = i + 2; }
+    if (better(v.w, i + 3, bv, bi)) { bv = v.w; bi = i + 3; }
   }
+  for (int i = head + 4 * n4 + threadIdx.x; i < V; i += THREADS)
+    if (better(row[i], i, bv, bi)) { bv = row[i]; bi = i; }
   block_best(bv, bi, sv, si);
   if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
 }

@@ -2,8 +2,10 @@
 
 Weights come from one SplitMix64 stream in call order (tests/golden/util.rs:18-95);
 the model and its draw order are those of `graphlm_lfm2` (tests/golden/lm.rs:262-309);
-the expected logits are the committed tests/golden/lm_graphlm_lfm2.json of the
-reference, which is read as data.
+the expected logits are the reference's committed tests/golden/lm_graphlm_lfm2.json.  Its numbers
+(float32 logits and the greedy ids) are kept beside this file as golden_lfm2_expected.npz, so
+that the check also runs where the reference is not mounted; when it is mounted, the copy is
+compared with the original.
 """
 from __future__ import annotations
 
@@ -14,6 +16,7 @@ import numpy as np
 
 MASK = (1 << 64) - 1
 GOLDEN_JSON = "/root/reference/tests/golden/lm_graphlm_lfm2.json"
+GOLDEN_NPZ = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden_lfm2_expected.npz")
 
 PROMPT = [5, 17, 42, 99, 133, 200]            # tests/golden/lm.rs:13
 DECODE = [7, 64, 250]                         # tests/golden/lm.rs:15
@@ -109,11 +112,17 @@ def golden_weights() -> dict:
 
 
 def golden_expected():
-    """The reference's committed outputs, or None when the reference is not mounted."""
-    if not os.path.exists(GOLDEN_JSON):
-        return None
-    with open(GOLDEN_JSON) as f:
-        return json.load(f)
+    """The reference's committed outputs: {"f32": {name: logits}, "ids": {"greedy8": [...]}}."""
+    data = np.load(GOLDEN_NPZ, allow_pickle=False)
+    out = {"f32": {k: data[k].astype(np.float64) for k in data.files if k != "greedy8"},
+           "ids": {"greedy8": data["greedy8"].tolist()}}
+    if os.path.exists(GOLDEN_JSON):                     # the copy must be the original's numbers
+        with open(GOLDEN_JSON) as f:
+            orig = json.load(f)
+        assert orig["ids"]["greedy8"] == out["ids"]["greedy8"]
+        for k, v in orig["f32"].items():
+            assert np.array_equal(np.asarray(v, dtype=np.float64), out["f32"][k]), k
+    return out
 
 
 def write_safetensors_f32(path: str, tensors: dict) -> None:

@@ -1,0 +1,242 @@
+"""Generation through the entry points: greedy and seeded temperature sampling against the plain
+implementation, the reference's golden vector through the engine, continuous batching under
+page pressure, the captured decode loop, the replay program and the command line."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+from tests.plain import golden_fixture as G
+from tests.plain import lfm2_plain as P
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def dirs(tmp_path_factory):
+    root = tmp_path_factory.mktemp("gen")
+    out = {n: H.make_model_dir(str(root), n, seed=21 + i) for i, n in enumerate("ABC")}
+    G.write_golden_model(str(root / "golden"))
+    out["golden"] = str(root / "golden")
+    return out
+
+
+def plain_greedy(model_dir, prompt, n):
+    w, cfg = P.load_model_dir(model_dir)
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = P.argmax_first(P.forward(w, cfg, seq)[-1])
+        out.append(t); seq.append(t)
+    return out
+
+
+def acceptable(model_dir, prompt, tokens, dtype):
+    """Every generated token is the plain implementation's choice given the same history, or lies
+    within the precision's error of the best logit."""
+    logits = H.plain_logits(model_dir, list(prompt) + list(tokens))
+    tol = H.tolerance(dtype) * np.abs(logits).max()
+    for i, t in enumerate(tokens):
+        row = logits[len(prompt) - 1 + i]
+        assert row[t] >= row.max() - 2 * tol, f"token {i} = {t}: logit {row[t]:.4f} vs best {row.max():.4f}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_matches_plain(dirs, dtype):
+    from gibbs_amd import Engine, generate
+    for name, lens in (("A", [7, 13]), ("C", [5])):
+        eng = Engine(dirs[name], dtype=dtype, max_tokens=512, max_requests=4)
+        prompts = [H.tokens(40 + i, n, H.TINY[name]["vocab_size"]) for i, n in enumerate(lens)]
+        outs = generate(eng, prompts, max_tokens=16, temperature=0.0, ignore_eos=True)
+        for p, o in zip(prompts, outs):
+            assert o.finish_reason == "length" and len(o.tokens) == 16
+            if dtype == "float32":
+                assert o.tokens == plain_greedy(dirs[name], p, 16)
+            acceptable(dirs[name], p, o.tokens, dtype)
+        eng.cache.check()
+        assert eng.cache.free_slots() == 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_reference_golden_vector_through_the_engine(dirs, dtype):
+    """tests/golden/lm_graphlm_lfm2.json of the reference: tolerance rel-L2 < 1e-3, cos > 0.9999
+    (tests/golden/util.rs:257-260) for the 32-bit path."""
+    from gibbs_amd import Engine, Entry, generate
+    exp = G.golden_expected()
+    eng = Engine(dirs["golden"], dtype=dtype, max_tokens=256, max_requests=2)
+    rel, cos = (1e-3, 0.9999) if dtype == "float32" else (3e-2, 0.999)
+    def last(rid, ids):
+        out = eng.step([Entry(rid, ids, [len(ids) - 1])]).cpu().numpy()[0]
+        return out
+    for name, ids in (("prefill6", G.PROMPT), ("prefill20", G.LONG_PROMPT)):
+        got = last(name, ids)
+        assert G.rel_l2(got, exp["f32"][name]) < rel and G.cosine(got, exp["f32"][name]) > cos, name
+        eng.release(name)
+    last("d", G.PROMPT)
+    for i, t in enumerate(G.DECODE):                                    # cached decode of forced tokens
+        got = last("d", [t])
+        assert G.rel_l2(got, exp["f32"][f"decode{i}"]) < rel and G.cosine(got, exp["f32"][f"decode{i}"]) > cos
+    eng.release("d")
+    if dtype == "float32":
+        out = generate(eng, [G.PROMPT], max_tokens=8, temperature=0.0, ignore_eos=True)[0]
+        assert out.tokens == exp["ids"]["greedy8"]
+
+
+def test_seeded_temperature_sampling(dirs):
+    """BASELINE's Tiny B workload: four requests (5, 11, 17, 29 tokens), prompt portions of 8,
+    temperature 0.8 from a fixed seed.  Every token equals what the plain sampler draws from the
+    plain logits of the same history with the same draw."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    from gibbs_amd.sampling import request_key, uniform
+    d = dirs["B"]
+    prompts = [H.tokens(60 + i, n, 512) for i, n in enumerate([5, 11, 17, 29])]
+    def run(seed):
+        eng = Engine(d, dtype="float32", max_tokens=1024, max_requests=4)
+        gen = Generator(eng, max_batch_tokens=16, chunk=8)
+        rids = [gen.submit(p, SamplingParams(temperature=0.8, max_new_tokens=12, seed=seed, ignore_eos=True)) for p in prompts]
+        res = gen.run()
+        return rids, [res[r].tokens for r in rids]
+    rids, toks = run(7)
+    assert run(7)[1] == toks, "a fixed seed reproduces the tokens"
+    assert run(8)[1] != toks
+    for rid, p, out in zip(rids, prompts, toks):
+        logits = H.plain_logits(d, p + out)
+        for i, t in enumerate(out):
+            cand, probs = P.nucleus(logits[len(p) - 1 + i].astype(np.float32), 0.8, 50, 0.9)
+            assert t == P.draw(cand, probs, uniform(7, request_key(rid), i)), f"request {rid} token {i}"
+
+
+def test_continuous_batching_under_page_pressure(dirs):
+    """A pool so small that running requests collide: the youngest is preempted and recomputed, and
+    every request still gets exactly the tokens it gets alone."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    d = dirs["A"]
+    prompts = [H.tokens(80 + i, n, 256) for i, n in enumerate([20, 24, 18, 30])]
+    params = SamplingParams(temperature=0.0, max_new_tokens=24, ignore_eos=True)
+    alone = []
+    for p in prompts:
+        eng = Engine(d, dtype="float32", max_tokens=256, max_requests=1, page_size=8)
+        g = Generator(eng)
+        r = g.submit(p, params)
+        alone.append(g.run()[r].tokens)
+    eng = Engine(d, dtype="float32", max_tokens=136, max_requests=4, page_size=8)      # 17 pages for ~200 tokens
+    gen = Generator(eng, max_batch_tokens=32)
+    rids = [gen.submit(p, params) for p in prompts]
+    preempted = 0
+    while gen.scheduler.has_work():
+        preempted += len(gen.step().preempted)
+        eng.cache.check()
+    res = gen.results()
+    assert preempted > 0, "the pool was meant to be too small"
+    for r, want in zip(rids, alone):
+        assert res[r].finish_reason == "length" and res[r].tokens == want
+    assert eng.cache.free_pages() == 17 and eng.cache.free_slots() == 4
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_loop_graph_replays_match_eager(dirs, dtype):
+    """The captured decode step, replayed several times with eager work and synchronisations in
+    between, gives on every replay what the eager step function gives."""
+    from gibbs_amd import Engine, Entry, SamplingParams
+    from gibbs_amd.engine.decode import DecodeLoop
+    d = dirs["B"]
+    prompts = [H.tokens(90 + i, n, 512) for i, n in enumerate([9, 30, 17])]
+    def prefill(eng):
+        first = []
+        for i, p in enumerate(prompts):
+            first.append(int(eng.step([Entry(i, p, [len(p) - 1])]).argmax(-1).item()))
+        return first
+    # eager reference through the step function, token by token
+    eng = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+    last, want = prefill(eng), [[] for _ in prompts]
+    for _ in range(40):
+        logits = eng.step([Entry(i, [last[i]], [0]) for i in range(3)])
+        last = logits.argmax(-1).tolist()
+        for i in range(3):
+            want[i].append(last[i])
+    for use_graph in (False, True):
+        eng = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+        loop = DecodeLoop(eng, [0, 1, 2], prefill(eng), use_graph=use_graph)
+        for n in (1, 7, 20, 12):                      # page edges are crossed between and inside runs
+            loop.run(n)
+            torch.cuda.synchronize()
+            eng.step([Entry("other", H.tokens(1, 11, 512), [10])])     # eager work between the replays
+            eng.release("other")
+        assert loop.tokens() == want, f"use_graph={use_graph}"
+        assert [eng.cached_tokens(i) for i in range(3)] == [len(p) + 40 for p in prompts]
+    # sampled decoding in the loop equals sampled decoding through the scheduler's sampler
+    params = [SamplingParams(temperature=0.9, top_p=0.8, top_k=20, seed=3, ignore_eos=True)] * 3
+    eng = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+    loop = DecodeLoop(eng, [0, 1, 2], prefill(eng), params=params, first_index=[1, 1, 1])
+    loop.run(10); loop.run(6)
+    from gibbs_amd.sampling import Draw, Sampler
+    eng2 = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+    last, sampler, got = prefill(eng2), Sampler(eng2.device), [[] for _ in prompts]
+    for s in range(16):
+        logits = eng2.step([Entry(i, [last[i]], [0]) for i in range(3)])
+        last = sampler.sample(logits, [Draw(params[i], i, 1 + s) for i in range(3)])
+        for i in range(3):
+            got[i].append(last[i])
+    assert loop.tokens() == got
+
+
+def trace_lines(steps):
+    return "".join(json.dumps({"step": i, "entries": [{"id": r, "tokens": t, "want": w} for r, t, w in e], "end": end}) + "\n"
+                   for i, (e, end) in enumerate(steps))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(dirs, dtype, tmp_path):
+    """bin/trace_run as a user runs it: a subprocess fed JSON lines, logits read back from files."""
+    d = dirs["A"]
+    a, b = H.tokens(1, 70, 256), H.tokens(2, 40, 256)
+    steps = [([("a", a[:50], list(range(50)))], []),
+             ([("a", a[50:52], [1]), ("b", b[:33], [0, 32])], []),
+             ([("b", b[33:35], [])], []),                                   # nothing wanted: no file
+             ([("a", a[52:53], [0]), ("b", b[35:40], [4])], ["b"]),
+             ([("a", a[53:70], list(range(17)))], ["a"])]
+    out = tmp_path / "logits"
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                           "--out", str(out), "--max-tokens", "192"], input=trace_lines(steps), capture_output=True,
+                          text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    assert not (out / "2.f32").exists()
+    pa, pb = H.plain_logits(d, a), H.plain_logits(d, b)
+    read = lambda i: np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(-1, 256)
+    H.assert_close(read(0), pa[:50], dtype, "step 0")
+    H.assert_close(read(1), np.stack([pa[51], pb[0], pb[32]]), dtype, "step 1")
+    H.assert_close(read(3), np.stack([pa[52], pb[39]]), dtype, "step 3")
+    H.assert_close(read(4), pa[53:70], dtype, "step 4")
+
+
+def test_command_line(dirs, tmp_path):
+    env = dict(os.environ)
+    run = lambda *a: subprocess.run([sys.executable, os.path.join(ROOT, "bin", "gibbs"), *a], capture_output=True,
+                                    text=True, timeout=300, env=env)
+    prompt = H.tokens(5, 9, 256)
+    p = run("--model", dirs["A"], "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0",
+            "--dtype", "float32")
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert "⚡ Prefill: 9 tokens" in p.stdout and "⚡ Decode: 5 tokens" in p.stdout and "📈 Roofline:" in p.stdout
+    line = p.stdout.split("✨ Output:\n")[1].splitlines()[0]
+    assert [int(t) for t in line.split()] == plain_greedy(dirs["A"], prompt, 6)
+    p = run("--model", dirs["B"], "--arch-dump")
+    dump = json.loads(p.stdout)
+    assert dump["architecture"] == "Lfm2ForCausalLM" and dump["unconsumed"] == [] and dump["missing"] == []
+    assert dump["derived"] == {"intermediate_size": 256, "full_attn_idxs": [0, 2, 5]}
+    p = run("--model", dirs["A"], "--probe-top5", "1,2,3", "--dtype", "float32")
+    top = json.loads(p.stdout.strip().splitlines()[-1])
+    want = H.plain_logits(dirs["A"], [1, 2, 3])[-1]
+    assert [t["id"] for t in top] == np.argsort(-want)[:5].tolist()
+    assert run("--model", dirs["A"], "--prompt-ids", "1", "--backend", "cpu").returncode == 2
+    cfgfile = tmp_path / "cfg.json"
+    cfgfile.write_text(json.dumps(H.TINY["C"]))
+    p = run("--model", str(tmp_path / "fresh"), "--random-weights", str(cfgfile), "--seed", "5", "--prompt-ids", "3,4",
+            "--max-tokens", "3")
+    assert p.returncode == 0 and os.path.isfile(tmp_path / "fresh" / "model.safetensors"), p.stderr[-2000:]

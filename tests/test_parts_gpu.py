@@ -1,0 +1,393 @@
+"""Each part alone against the plain implementation; parts chosen layer by layer; a layer order
+that names a layer twice and a layer that reads another layer's cache; a windowed attention
+whose cache group gives pages back; and a toy mixer with state of its own, defined here and
+registered without a change to the framework's files."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from tests import helpers as H
+from tests.plain import lfm2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [("float32", torch.float32), ("bfloat16", torch.bfloat16)]
+
+
+def bf16_exact(a: np.ndarray) -> np.ndarray:
+    """Rounds to values bfloat16 holds exactly, so every precision starts from the same numbers."""
+    return torch.tensor(a, dtype=torch.float32).to(torch.bfloat16).double().numpy()
+
+
+def store(tensors: dict, decls, dtype):
+    from gibbs_amd.weights import WeightStore
+    out = {}
+    for d in decls:
+        out[d.name] = torch.tensor(tensors[d.name]).reshape(d.shape).to(DEV, d.resolved_dtype(dtype)).contiguous()
+    return WeightStore(out, dtype, torch.device(DEV))
+
+
+def run_mixer(mixer, hs, chunks, dtype, page_size=8):
+    """Feeds h (a list of [T_r, hidden] arrays, one per request) through a bound mixer in the given
+    chunks [(request, a, b), ...] per step; returns the concatenated outputs per request."""
+    from gibbs_amd.cache import CacheManager, DeviceCache
+    from gibbs_amd.engine.batch import BatchStager
+    cm = CacheManager([mixer.cache_need()], [tuple(mixer.state_needs())], page_size, 64, 4)
+    dc = DeviceCache(cm, dtype, torch.device(DEV))
+    view = dc.layer_view(0)
+    stager = BatchStager(torch.device(DEV))
+    outs = {r: [] for r in range(len(hs))}
+    for step in chunks:
+        rids = [r for r, _, _ in step]
+        for r, a, b in step:
+            if r not in cm:
+                assert cm.admit(r)
+            assert cm.reserve(r, b - a)
+        dc.clear_fresh_slots()
+        q = np.array([b - a for _, a, b in step], dtype=np.int32)
+        cu = np.concatenate([[0], np.cumsum(q)]).astype(np.int32)
+        ctx = np.array([cm.tokens(r) for r in rids], dtype=np.int32)
+        row_req = np.repeat(np.arange(len(step), dtype=np.int32), q)
+        pos = (np.arange(cu[-1], dtype=np.int32) - cu[:-1][row_req] + ctx[row_req]).astype(np.int32)
+        batch = stager.stage(np.zeros(cu[-1], np.int32), pos, row_req, cu, ctx,
+                             np.array([cm.slot(r) for r in rids], np.int32), np.zeros(0, np.int32),
+                             [cm.block_table(rids, g) for g in range(cm.n_groups)])
+        h = torch.tensor(np.concatenate([hs[r][a:b] for r, a, b in step])).to(DEV, dtype).contiguous()
+        y = mixer.forward(h, batch, view)
+        if y.dim() == 3:
+            y = y.sum(0)
+        y = y.float().cpu().numpy()
+        for i, (r, a, b) in enumerate(step):
+            outs[r].append(y[cu[i]:cu[i + 1]])
+            cm.commit(r, b - a)
+        cm.check()
+    return {r: np.concatenate(v) for r, v in outs.items()}, cm
+
+
+def close(got, want, name, what):
+    tol = {"float32": 1e-5, "bfloat16": 2e-2}[name]
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= tol * scale, f"{what}: {np.abs(got - want).max():.3e} > {tol} x {scale:.3e}"
+
+
+# two requests fed in ragged steps: portions of one beside single tokens of the other
+STEPS = [[(0, 0, 5)], [(0, 5, 7), (1, 0, 9)], [(0, 7, 8), (1, 9, 11)], [(0, 8, 9), (1, 11, 12)], [(0, 9, 26), (1, 12, 13)],
+         [(1, 13, 14), (0, 26, 27)]]
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_norm_part(name, dtype):
+    from gibbs_amd.config import NormSpec
+    from gibbs_amd.parts import Runtime, build_norm
+    rng = np.random.default_rng(0)
+    norm = build_norm(NormSpec("rms", 3e-6, "g"), 72)
+    gain = rng.normal(size=72) + 1
+    norm.bind(store({"g": gain}, norm.tensor_decls(), dtype), Runtime(torch.device(DEV), dtype))
+    x = rng.normal(size=(5, 72)).astype(np.float32)
+    delta = bf16_exact(rng.normal(size=(5, 72)))
+    xt = torch.tensor(x, device=DEV)
+    out = norm.forward(xt, torch.tensor(delta).to(DEV, dtype))
+    close(out.float().cpu().numpy(), P.rms_norm(x.astype(np.float64) + delta, gain, 3e-6), name, "norm")
+    np.testing.assert_allclose(xt.cpu().numpy(), x + delta.astype(np.float32), rtol=1e-6)
+
+
+def test_rope_part_table():
+    from gibbs_amd.config import PositionSpec
+    from gibbs_amd.parts import Runtime, build_position
+    for theta, dim in [(1e4, 16), (1e6, 64), (5e5, 48)]:
+        pos = build_position(PositionSpec("rope", {"theta": theta, "rotary_dim": dim, "precision": "f32"}), dim)
+        pos.bind(None, Runtime(torch.device(DEV), torch.float32))
+        np.testing.assert_array_equal(pos.inv_freq.cpu().numpy(), P.rope_inv_freq(dim, theta))
+    assert build_position(None, 16) is None and build_position(PositionSpec("none"), 16) is None
+    with pytest.raises(ValueError, match="rotary_dim"):
+        build_position(PositionSpec("rope", {"theta": 1e4, "rotary_dim": 18}), 16)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv,hd,hidden,window", [(4, 2, 16, 40, None), (3, 1, 48, 72, None), (4, 4, 32, 64, 6)])
+def test_attention_part(name, dtype, heads, kv, hd, hidden, window):
+    from gibbs_amd.config import MixerSpec, PositionSpec
+    from gibbs_amd.parts import Runtime, build_mixer
+    rng = np.random.default_rng(1)
+    names = {k: k for k in ("q_proj", "k_proj", "v_proj", "out_proj", "q_norm", "k_norm")}
+    spec = MixerSpec("attention", {"heads": heads, "kv_heads": kv, "head_dim": hd, "scale": 1 / math.sqrt(hd),
+                                   "qk_norm": "before", "qk_norm_eps": 1e-6, "window": window}, names,
+                     PositionSpec("rope", {"theta": 1e4, "rotary_dim": hd, "precision": "f32"}))
+    mixer = build_mixer(spec, hidden, 0)
+    w = {"q_proj": bf16_exact(rng.normal(size=(heads * hd, hidden)) * 0.3), "k_proj": bf16_exact(rng.normal(size=(kv * hd, hidden)) * 0.3),
+         "v_proj": bf16_exact(rng.normal(size=(kv * hd, hidden)) * 0.3), "out_proj": bf16_exact(rng.normal(size=(hidden, heads * hd)) * 0.2),
+         "q_norm": rng.normal(size=hd) * 0.1 + 1, "k_norm": rng.normal(size=hd) * 0.1 + 1}
+    mixer.bind(store(w, mixer.tensor_decls(), dtype), Runtime(torch.device(DEV), dtype))
+    hs = [bf16_exact(rng.normal(size=(27, hidden))), bf16_exact(rng.normal(size=(14, hidden)))]
+    got, cm = run_mixer(mixer, hs, STEPS, dtype)
+    for r, h in enumerate(hs):
+        want = P.attention_mixer(h, w["q_proj"], w["k_proj"], w["v_proj"], w["out_proj"], w["q_norm"], w["k_norm"],
+                                 heads=heads, kv_heads=kv, head_dim=hd, eps=1e-6, inv_freq=P.rope_inv_freq(hd, 1e4),
+                                 positions=list(range(len(h))), scale=1 / math.sqrt(hd), window=window)
+        close(got[r], want, name, f"attention part request {r}")
+    if window is not None:
+        # pages of 8 tokens behind a window of 6: request 0 (27 tokens) holds at most 2 pages at the end
+        table = cm.block_table([0], 0)[0]
+        assert (table >= 0).sum() <= 2 and (table[:2] == -1).all(), table
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("width,kernel,bias", [(40, 3, False), (72, 4, True), (16, 2, True)])
+def test_shortconv_part(name, dtype, width, kernel, bias):
+    from gibbs_amd.config import MixerSpec
+    from gibbs_amd.parts import Runtime, build_mixer
+    rng = np.random.default_rng(2)
+    names = {"in_proj": "in", "conv": "taps", "out_proj": "out", "conv_bias": "b"}
+    mixer = build_mixer(MixerSpec("short_conv", {"width": width, "kernel": kernel, "bias": bias}, names), width, 0)
+    w = {"in": bf16_exact(rng.normal(size=(3 * width, width)) * 0.3), "taps": rng.normal(size=(width, 1, kernel)),
+         "out": bf16_exact(rng.normal(size=(width, width)) * 0.3), "b": rng.normal(size=width) * 0.1}
+    mixer.bind(store(w, mixer.tensor_decls(), dtype), Runtime(torch.device(DEV), dtype))
+    hs = [bf16_exact(rng.normal(size=(27, width))), bf16_exact(rng.normal(size=(14, width)))]
+    got, _ = run_mixer(mixer, hs, STEPS, dtype)
+    taps32 = w["taps"].astype(np.float32).astype(np.float64)
+    for r, h in enumerate(hs):
+        want = P.short_conv_mixer(h, w["in"], taps32, w["out"], w["b"].astype(np.float32) if bias else None)
+        close(got[r], want, name, f"short conv part request {r}")
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_glu_part(name, dtype):
+    from gibbs_amd.config import FeedForwardSpec
+    from gibbs_amd.parts import Runtime, build_feed_forward
+    rng = np.random.default_rng(3)
+    ffn = build_feed_forward(FeedForwardSpec("glu", {"inter": 200, "activation": "silu"},
+                                             {"gate": "w1", "up": "w3", "down": "w2"}), 72)
+    w = {"w1": bf16_exact(rng.normal(size=(200, 72)) * 0.2), "w3": bf16_exact(rng.normal(size=(200, 72)) * 0.2),
+         "w2": bf16_exact(rng.normal(size=(72, 200)) * 0.2)}
+    ffn.bind(store(w, ffn.tensor_decls(), dtype), Runtime(torch.device(DEV), dtype))
+    h = bf16_exact(rng.normal(size=(9, 72)))
+    y = ffn.forward(torch.tensor(h).to(DEV, dtype), None)
+    y = y.sum(0) if y.dim() == 3 else y
+    close(y.float().cpu().numpy(), P.swiglu_ffn(h, w["w1"], w["w3"], w["w2"]), name, "glu part")
+    with pytest.raises(ValueError, match="activation"):
+        build_feed_forward(FeedForwardSpec("glu", {"inter": 8, "activation": "relu"}, {}), 8)
+    with pytest.raises(KeyError, match="no feed-forward of kind"):
+        build_feed_forward(FeedForwardSpec("experts", {}, {}), 8)
+
+
+# --------------------------------------------------------------------------- whole specs built by hand
+def plain_spec_forward(spec, weights, ids):
+    """Plain forward of a hand-built ModelSpec from the plain part functions: handles a run order
+    that repeats layers and attention layers that read an earlier run's keys and values."""
+    T = len(ids)
+    x = P.embedding(weights[spec.embedding], ids)
+    kv_of_layer = {}
+    for i in spec.order:
+        L = spec.layers[i]
+        h = P.rms_norm(x, weights[L.mixer_norm.weight], L.mixer_norm.eps)
+        m, t = L.mixer, L.mixer.tensors
+        if m.kind == "short_conv":
+            a = P.short_conv_mixer(h, weights[t["in_proj"]], weights[t["conv"]], weights[t["out_proj"]],
+                                   weights.get(t.get("conv_bias", "")))
+        else:
+            p = m.params
+            nh, nkv, hd = p["heads"], p["kv_heads"], p["head_dim"]
+            inv = P.rope_inv_freq(hd, m.position.params["theta"])
+            q = P.rope_half_split(P.rms_norm(P.linear(h, weights[t["q_proj"]]).reshape(T, nh, hd), weights[t["q_norm"]], p["qk_norm_eps"]), range(T), inv)
+            if p.get("kv_source") is None:
+                k = P.rope_half_split(P.rms_norm(P.linear(h, weights[t["k_proj"]]).reshape(T, nkv, hd), weights[t["k_norm"]], p["qk_norm_eps"]), range(T), inv)
+                v = P.linear(h, weights[t["v_proj"]]).reshape(T, nkv, hd)
+                kv_of_layer[i] = (k, v)
+            else:
+                k, v = kv_of_layer[p["kv_source"]]
+            a = P.linear(P.causal_attention(q, k, v, p["scale"], p.get("window")).reshape(T, nh * hd), weights[t["out_proj"]])
+        x = x + a
+        h = P.rms_norm(x, weights[L.ffn_norm.weight], L.ffn_norm.eps)
+        f = L.ffn.tensors
+        x = x + P.swiglu_ffn(h, weights[f["gate"]], weights[f["up"]], weights[f["down"]])
+    x = P.rms_norm(x, weights[spec.final_norm.weight], spec.final_norm.eps)
+    return P.linear(x, weights[spec.head or spec.embedding])
+
+
+def hand_spec(hidden=48, vocab=97):
+    """Layer 0 attention (owns a cache), layer 1 short conv, layer 2 attention that reads layer 0's
+    cache, run order 0, 1, 2, 1: layer 1 runs twice with the same weights and a state per run."""
+    from gibbs_amd.config import FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec
+    rope = PositionSpec("rope", {"theta": 1e4, "rotary_dim": 16, "precision": "f32"})
+    layers = []
+    for i, kind in enumerate(["attention", "short_conv", "shared"]):
+        p = f"l{i}"
+        if kind == "short_conv":
+            mixer = MixerSpec("short_conv", {"width": hidden, "kernel": 3, "bias": False},
+                              {"in_proj": f"{p}.in", "conv": f"{p}.taps", "out_proj": f"{p}.out"})
+        else:
+            params = {"heads": 3, "kv_heads": 1, "head_dim": 16, "scale": 0.25, "qk_norm": "before", "qk_norm_eps": 1e-5,
+                      "window": None}
+            tensors = {"q_proj": f"{p}.q", "out_proj": f"{p}.o", "q_norm": f"{p}.qn"}
+            if kind == "shared":
+                params["kv_source"] = 0
+            else:
+                tensors.update({"k_proj": f"{p}.k", "v_proj": f"{p}.v", "k_norm": f"{p}.kn"})
+            mixer = MixerSpec("attention", params, tensors, rope)
+        ffn = FeedForwardSpec("glu", {"inter": 64, "activation": "silu"}, {"gate": f"{p}.w1", "up": f"{p}.w3", "down": f"{p}.w2"})
+        layers.append(LayerSpec(p, "pre_norm", NormSpec("rms", 1e-5, f"{p}.n1"), mixer, NormSpec("rms", 1e-5, f"{p}.n2"), ffn))
+    return ModelSpec("Hand", hidden, vocab, tuple(layers), (0, 1, 2, 1), "emb", NormSpec("rms", 1e-5, "fn"), "head", 256)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_layer_order_and_shared_cache(name, dtype, tmp_path):
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import random_tensor
+    spec = hand_spec()
+    decls = DecoderModel(spec).tensor_decls()
+    assert not any(d.name in ("l2.k", "l2.v", "l2.kn") for d in decls), "a layer that reads a cache projects no k, v"
+    tensors = {d.name: random_tensor(d, 5, torch.bfloat16, std=0.15, gain_std=0.1) for d in decls}
+
+    class Hand(ArchConfig):
+        def model_spec(self):
+            return spec
+    ws = store({k: v.float().numpy() for k, v in tensors.items()}, decls, dtype)
+    eng = Engine(config=Hand(), weights=ws, dtype=name, max_tokens=256, max_requests=2, page_size=8)
+    assert eng.cache.group_layers == [[0]] and len(eng.cache.state_layout) == 2, "one cache, one state per run of layer 1"
+    ids = H.tokens(4, 40, spec.vocab)
+    want = plain_spec_forward(spec, {k: v.double().numpy() for k, v in tensors.items()}, ids)
+    got = []
+    for a, b in [(0, 9), (9, 11), (11, 12), (12, 13), (13, 40)]:
+        got.append(eng.step([Entry("r", ids[a:b], list(range(b - a)))]).cpu().numpy())
+    H.assert_close(np.concatenate(got), want, name, "hand-built spec")
+
+
+# --------------------------------------------------------------------------- a toy mixer with its own state
+def register_toy():
+    """An exponential moving average over time of a projection of the input: state [hidden] per
+    request.  Written with framework operations and plain tensor code; nothing in the framework
+    knows about it."""
+    from gibbs_amd.cache import StateNeed
+    from gibbs_amd.ops.linear import linear
+    from gibbs_amd.parts import Mixer, register_mixer
+    from gibbs_amd.weights import TensorDecl
+
+    @register_mixer("toy_ema")
+    class ToyEma(Mixer):
+        def state_needs(self):
+            return (StateNeed("ema", (self.hidden,)),)
+
+        def tensor_decls(self):
+            return [TensorDecl(self.spec.tensors["proj"], (self.hidden, self.hidden))]
+
+        def bind(self, weights, rt):
+            self.rt, self.w = rt, weights[self.spec.tensors["proj"]]
+
+        def forward(self, h, batch, cache):
+            u = linear(h, self.w).float()
+            decay = self.spec.params["decay"]
+            state = cache.states["ema"]
+            out = torch.empty_like(u)
+            row = 0
+            for q, slot in zip(batch.q_lens, batch.slots):
+                s = state[slot].clone()
+                for t in range(q):
+                    s = decay * s + u[row + t]
+                    out[row + t] = s
+                state[slot] = s
+                row += q
+            return out.to(self.rt.act_dtype)
+    return ToyEma
+
+
+def toy_config_class():
+    from gibbs_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                  register_architecture)
+    from gibbs_amd.config.base import ArchConfig
+
+    class ToyConfig(ArchConfig):
+        architecture = "ToyEmaForCausalLM"
+
+        def __init__(self, cfg):
+            self.cfg = dict(cfg)
+
+        @classmethod
+        def from_dict(cls, cfg, tensors=None):
+            return cls(cfg)
+
+        def to_dict(self):
+            return dict(self.cfg)
+
+        def model_spec(self):
+            c, layers = self.cfg, []
+            H_, hd = c["width"], c["head_size"]
+            for i, kind in enumerate(c["mixers"]):
+                p = f"blocks.{i}"
+                if kind == "ema":
+                    mixer = MixerSpec("toy_ema", {"decay": c["decay"]}, {"proj": f"{p}.ema.proj"})
+                else:
+                    mixer = MixerSpec("attention", {"heads": c["heads"], "kv_heads": c["heads"], "head_dim": hd,
+                                                    "scale": hd ** -0.5, "qk_norm": None, "window": None},
+                                      {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o"},
+                                      PositionSpec("rope", {"theta": c["theta"], "rotary_dim": hd, "precision": "f32"}))
+                ffn = FeedForwardSpec("glu", {"inter": c["ff"], "activation": "silu"},
+                                      {"gate": f"{p}.g", "up": f"{p}.u", "down": f"{p}.d"})
+                layers.append(LayerSpec(p, "pre_norm", NormSpec("rms", c["eps"], f"{p}.n1"), mixer,
+                                        NormSpec("rms", c["eps"], f"{p}.n2"), ffn))
+            return ModelSpec(self.architecture, H_, c["vocab"], tuple(layers), tuple(range(len(layers))), "tok",
+                             NormSpec("rms", c["eps"], "out_norm"), None, c["max_len"])
+    register_architecture("ToyEmaForCausalLM", ToyConfig, aliases=("toy_ema",))
+    return ToyConfig
+
+
+def toy_plain(cfg, w, ids):
+    T, hd, nh = len(ids), cfg["head_size"], cfg["heads"]
+    x = P.embedding(w["tok"], ids)
+    for i, kind in enumerate(cfg["mixers"]):
+        p = f"blocks.{i}"
+        h = P.rms_norm(x, w[f"{p}.n1"], cfg["eps"])
+        if kind == "ema":
+            u, s, a = P.linear(h, w[f"{p}.ema.proj"]), np.zeros(cfg["width"]), []
+            for t in range(T):
+                s = cfg["decay"] * s + u[t]
+                a.append(s)
+            a = np.stack(a)
+        else:
+            inv = P.rope_inv_freq(hd, cfg["theta"])
+            q = P.rope_half_split(P.linear(h, w[f"{p}.q"]).reshape(T, nh, hd), range(T), inv)
+            k = P.rope_half_split(P.linear(h, w[f"{p}.k"]).reshape(T, nh, hd), range(T), inv)
+            v = P.linear(h, w[f"{p}.v"]).reshape(T, nh, hd)
+            a = P.linear(P.causal_attention(q, k, v, hd ** -0.5).reshape(T, nh * hd), w[f"{p}.o"])
+        x = x + a
+        x = x + P.swiglu_ffn(P.rms_norm(x, w[f"{p}.n2"], cfg["eps"]), w[f"{p}.g"], w[f"{p}.u"], w[f"{p}.d"])
+    return P.linear(P.rms_norm(x, w["out_norm"], cfg["eps"]), w["tok"])
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_toy_mixer_with_state_registers_builds_and_steps(name, dtype, tmp_path):
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import write_random_model
+    register_toy()
+    Toy = toy_config_class()
+    cfg = {"architectures": ["ToyEmaForCausalLM"], "width": 40, "heads": 2, "head_size": 16, "ff": 56, "vocab": 83,
+           "mixers": ["ema", "attn", "ema"], "decay": 0.75, "theta": 1e4, "eps": 1e-5, "max_len": 128}
+    folder = str(tmp_path / "toy")
+    config = Toy.from_dict(cfg)
+    write_random_model(folder, config, DecoderModel(config.model_spec()).tensor_decls(), seed=2, std=0.15, gain_std=0.1)
+    assert json.load(open(os.path.join(folder, "config.json")))["mixers"] == ["ema", "attn", "ema"]
+    eng = Engine(folder, dtype=name, max_tokens=128, max_requests=2, page_size=8)     # the class is chosen by config.json
+    assert [type(b.mixer).__name__ for b in eng.model.blocks] == ["ToyEma", "AttentionMixer", "ToyEma"]
+    assert set(eng.cache.state_layout) == {(0, "ema"), (2, "ema")}
+    weights, _ = P.load_model_dir(folder)
+    seqs = {"a": H.tokens(1, 30, 83), "b": H.tokens(2, 17, 83)}
+    got = {}
+    # a (portions) beside b (tokens one by one), b ends first and c takes its slot: the state must be cleared
+    plan = [[("a", 0, 6), ("b", 0, 4)], [("a", 6, 8), ("b", 4, 5)], [("a", 8, 9), ("b", 5, 17)], [("a", 9, 30)]]
+    for step in plan:
+        out = eng.step([Entry(r, seqs[r][a:b], list(range(b - a))) for r, a, b in step]).cpu().numpy()
+        at = 0
+        for r, a, b in step:
+            got.setdefault(r, []).append(out[at:at + b - a]); at += b - a
+    eng.release("b")
+    seqs["c"] = H.tokens(3, 9, 83)
+    got["c"] = [eng.step([Entry("c", seqs["c"], list(range(9)))]).cpu().numpy()]
+    assert eng.cache.slot("c") != eng.cache.slot("a")
+    for r, ids in seqs.items():
+        H.assert_close(np.concatenate(got[r]), toy_plain(cfg, weights, ids), name, f"toy model request {r}")

@@ -157,7 +157,6 @@ def test_tail_tied_equals_untied_copy():
     np.testing.assert_allclose(P.forward(w, cfg, G.PROMPT[:4]), a[:4], atol=1e-12)
 
 
-@pytest.mark.skipif(G.golden_expected() is None, reason="reference golden JSON not mounted")
 def test_whole_model_golden_vector():
     """tests/golden/lm_graphlm_lfm2.json of the reference; tolerance of tests/golden/util.rs:257-260."""
     w, cfg, exp = G.golden_weights(), G.golden_config(), G.golden_expected()
