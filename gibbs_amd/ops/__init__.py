@@ -274,6 +274,31 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     return out
 
 
+def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
+                      vpages: torch.Tensor, table: torch.Tensor, n_req: int, cu: torch.Tensor, ctx: torch.Tensor,
+                      scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """bfloat16 paged causal attention for prompt portions on the matrix cores: rows cu[r] .. cu[r+1]
+    of request r sit at positions ctx[r] ..; same result as `attention_plain`.  Head sizes: multiples
+    of 16 up to 128."""
+    require_cuda(q, kpages, vpages, table, cu, ctx)
+    if q.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill is the bfloat16 kernel; the float32 path uses attention_plain")
+    if hd % 16 or not 16 <= hd <= 128:
+        raise KernelError(f"attention_prefill: head size {hd} must be a multiple of 16 up to 128")
+    assert q.dim() == 2 and q.shape[0] == n_rows and q.stride(1) == 1 and q.shape[1] >= nh * hd
+    num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
+    assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
+    assert table.dim() == 2 and table.shape[0] >= n_req
+    _i32(table, n_req, "block table"); _i32(cu, n_req + 1, "cu"); _i32(ctx, n_req, "ctx")
+    if out is None:
+        out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
+    assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
+    call("gibbs_attention_prefill", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(cu), ptr(ctx), ptr(table), n_req,
+         table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd, q.stride(0) if n_rows > 1 else q.shape[1], nh * hd,
+         float(scale), int(window or 0), stream())
+    return out
+
+
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Index of the first largest value of each row (NaN never wins), int32 [M]."""
     require_cuda(logits)

@@ -101,9 +101,15 @@ class AttentionMixer(Mixer):
         return linear(a, self.w_out, partial_ok=True)
 
     def attend(self, qkv, batch, cache, table) -> torch.Tensor:
-        """Attention of the step's rows over the cache.  bfloat16 rows that are all single decoded
-        tokens take the kernel that splits the keys; everything else the plain kernel."""
-        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1:
+        """Attention of the step's rows over the cache.  bfloat16: rows that are all single decoded
+        tokens take the kernel that splits the keys, steps with prompt portions the matrix-core
+        kernel (head sizes up to 128).  float32, and whatever the fast kernels do not take: the
+        plain kernel."""
+        bf16 = self.rt.act_dtype == torch.bfloat16
+        if bf16 and batch.max_q > 1 and self.head_dim % 16 == 0 and self.head_dim <= 128:
+            return ops.attention_prefill(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
+                                         cache.vpages, table, batch.n_req, batch.cu, batch.ctx, self.scale, self.window)
+        if bf16 and batch.max_q == 1 and self.head_dim % 8 == 0:
             return ops.attention_decode(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
                                         cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
                                         self.window, max_seq=batch.max_seq)

@@ -94,9 +94,14 @@ def tolerance(dtype: str) -> float:
 
 def consistency(dtype: str) -> float:
     """Largest allowed difference, as a fraction of the scale, between the logits that two ways of
-    cutting or batching the same tokens give in the same precision.  The ways differ only in the
-    order of float32 additions, and in bfloat16 in the few values that then round the other way."""
-    return {"float32": 2e-6, "bfloat16": 1e-2}[dtype]
+    cutting or batching the same tokens give in the same precision.  32-bit: the ways differ only
+    in the order of float32 additions.  bfloat16: prompt portions and decoded tokens take different
+    attention kernels (the matrix-core kernel rounds the softmax weights to bfloat16 for its second
+    product, the decode kernel keeps them in float32) and different matrix-product kernels, so the
+    ways differ by rounding noise of the same kind as each differs from the plain implementation,
+    amplified through the layers in the same way (measured up to 1.6 % for the 6-layer model);
+    what pins the fast kernels' indexing tightly is their own tests against exact references."""
+    return {"float32": 2e-6, "bfloat16": 4e-2}[dtype]
 
 
 def assert_close(got: np.ndarray, want: np.ndarray, dtype: str, what: str = "", tol: float | None = None) -> None:

@@ -277,6 +277,34 @@ def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits):
     close(out, plain, dtype, "decode vs plain kernel", bf16=1e-2)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
+                                                   (32, 8, 64, 16, None), (4, 2, 128, 16, None), (2, 2, 96, 64, 100),
+                                                   (3, 1, 32, 16, 5)])
+def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window):
+    """Prompt portions on the matrix cores: a long portion after a cached context that ends off a
+    tile edge, a whole short prompt, a 2-token portion, a single decoded row and a 65-row portion
+    that starts at position 0, all in one call."""
+    from gibbs_amd import ops
+    dtype = torch.bfloat16
+    seq_lens = [333, 9, 130, 77, 65]
+    q_lens = [150, 9, 2, 1, 65]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 120, seed=11)
+    ctx = [s - q for s, q in zip(seq_lens, q_lens)]
+    cu = np.concatenate([[0], np.cumsum(q_lens)])
+    n = int(cu[-1])
+    q = rnd(n, nh * hd, dtype=dtype, seed=9)
+    scale = 1 / math.sqrt(hd)
+    out = ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window)
+    pos = i32([c + t for c, ql in zip(ctx, q_lens) for t in range(ql)])
+    row_req = i32([r for r, ql in enumerate(q_lens) for _ in range(ql)])
+    plain = ops.attention_plain(q, n, nh, nkv, hd, kp, vp, table, 5, pos, row_req, scale, window)
+    for r in range(5):
+        rows = slice(int(cu[r]), int(cu[r + 1]))
+        want = attention_reference(q[rows].view(-1, nh, hd), ks[r], vs[r], list(range(ctx[r], seq_lens[r])), scale, window)
+        close(out[rows].view(-1, nh, hd), want, dtype, f"prefill attention request {r}", bf16=1e-2)
+    close(out, plain, dtype, "prefill vs plain kernel", bf16=1e-2)
+
+
 @pytest.mark.parametrize("dtype", DT)
 def test_attention_far_key_stands_out(dtype):
     """One key far back among hundreds gets a large score: its value must dominate the output."""
@@ -292,6 +320,14 @@ def test_attention_far_key_stands_out(dtype):
     want = attention_reference(q.view(1, 1, hd), ks[0], vs[0], [L - 1], 1 / math.sqrt(hd), None)
     close(out.view(1, 1, hd), want, dtype, "far key", f32=2e-5, bf16=1e-2)
     assert (out.float() - vs[0][far, 0].float()).abs().max() < 0.05 * vs[0][far, 0].float().abs().max() + 0.05
+    if dtype == torch.bfloat16:
+        # the same through the fast kernels: split keys (the far key lies in the first slice), and
+        # the matrix-core kernel with the row as the last of a 2-row portion
+        split = ops.attention_decode(q, 1, nh, nkv, hd, kp, vp, table, 1, i32([L - 1]), i32([0]), 1 / math.sqrt(hd), n_splits=8)
+        close(split.view(1, 1, hd), want, dtype, "far key, split keys", bf16=1e-2)
+        q2 = torch.cat([rnd(1, hd, dtype=dtype, seed=2), q])
+        pre = ops.attention_prefill(q2, 2, nh, nkv, hd, kp, vp, table, 1, i32([0, 2]), i32([L - 2]), 1 / math.sqrt(hd))
+        close(pre[1].view(1, 1, hd), want, dtype, "far key, matrix cores", bf16=1e-2)
 
 
 @pytest.mark.parametrize("dtype", DT)
