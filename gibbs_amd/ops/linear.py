@@ -1,12 +1,15 @@
 """y = x @ W^T for weights stored [out, in], in the precision of the run.
 
 float32: the hand-written plain-FMA kernel (a true 32-bit product whose per-row result does not
-depend on the batch).  bfloat16: matrix cores with float32 accumulation; up to 64 rows take the
-kernel that streams W once (decode), more rows the tiled kernel (prefill).  The output is
-bfloat16, or float32 where the caller asks for it (logits).
+depend on the batch).  bfloat16, float32 accumulation throughout: up to 64 rows take the
+hand-written kernel that streams W once (decode); more rows take a matrix product on the matrix
+cores, by default the library's (hipBLASLt through `torch.matmul`, as the reference's engine
+uses a library product for its prefill), or the hand-written tiled kernel (`GIBBS_GEMM=own`),
+which also serves what the library does not give: float32 output (logits of many rows).
 """
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -15,6 +18,7 @@ from . import gemm_bf16, gemm_f32, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
 SKINNY_ROWS = 64
+USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -34,5 +38,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         if 1 <= x.shape[0] <= SKINNY_ROWS:
             splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
             return gemm_skinny(x, w, out_dtype, splits)
+        if USE_LIBRARY_GEMM and out_dtype == torch.bfloat16:
+            return torch.matmul(x, w.t())
         return gemm_bf16(x, w, out_dtype)
     raise KernelError(f"linear: unsupported dtype {x.dtype}")
