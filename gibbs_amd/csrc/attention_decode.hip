@@ -183,25 +183,45 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
 }
 
 // Merges the slices of one (row, head): out = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s.
+// One wave per (row, head): lanes first fetch the slices' (max, sum) side by side, then each lane
+// sums its elements over the slices, four loads in flight at a time.
 __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int nh, int hd,
                                        int n_splits, long ldo) {
   const int row = blockIdx.x, head = blockIdx.y * (blockDim.x / WAVE) + threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
   if (head >= nh) return;
-  const float* ps = partial + ((size_t)row * nh + head) * n_splits * (hd + 2);
+  const size_t stride = hd + 2;
+  const float* ps = partial + ((size_t)row * nh + head) * n_splits * stride;
   float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, ps[(size_t)s * (hd + 2)]);
+  for (int s0 = 0; s0 < n_splits; s0 += WAVE) {
+    const int s = s0 + lane;
+    M = fmaxf(M, wave_max(s < n_splits ? ps[s * stride] : -INFINITY));
+  }
   float L = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float ms = ps[(size_t)s * (hd + 2)];
-    if (ms != -INFINITY) L += __expf(ms - M) * ps[(size_t)s * (hd + 2) + 1];
+  for (int s0 = 0; s0 < n_splits; s0 += WAVE) {
+    const int s = s0 + lane;
+    float term = 0.f;
+    if (s < n_splits) {
+      const float ms = ps[s * stride];
+      if (ms != -INFINITY) term = __expf(ms - M) * ps[s * stride + 1];
+    }
+    L += wave_sum(term);
   }
   const float inv = 1.0f / L;
   for (int e = lane; e < hd; e += WAVE) {
     float v = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float ms = ps[(size_t)s * (hd + 2)];
-      if (ms != -INFINITY) v += __expf(ms - M) * ps[(size_t)s * (hd + 2) + 2 + e];
+    int s = 0;
+    for (; s + 4 <= n_splits; s += 4) {
+      float ms[4], av[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { ms[j] = ps[(s + j) * stride]; av[j] = ps[(s + j) * stride + 2 + e]; }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (ms[j] != -INFINITY) v = fmaf(__expf(ms[j] - M), av[j], v);
+    }
+    for (; s < n_splits; ++s) {
+      const float m1 = ps[s * stride];
+      if (m1 != -INFINITY) v = fmaf(__expf(m1 - M), ps[s * stride + 2 + e], v);
     }
     out[(size_t)row * ldo + (size_t)head * hd + e] = (bf16)(v * inv);
   }
@@ -259,4 +279,316 @@ GIBBS_EXPORT int gibbs_attention_decode(const void* q, const void* kpages, const
     attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, (bf16*)out, nh, hd, n_splits, ldo);
   }
   GIBBS_LAUNCH_STATUS("attention_decode");
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same attention for a step of decoded tokens only, with what surrounds it fused in: the rows
+// arrive as the raw fused projection qkv[N, (nh + 2 nkv) hd]; the kernel norms and rotates q on the
+// fly (every slice's workgroup does, it is a few hundred operations), norms and rotates the row's
+// own new key, writes it and the new value to their page (the workgroup of head chunk 0 whose key
+// slice holds the row's position does) and uses them from LDS instead of reading them back.
+// The slices are merged by the separate merge kernel: letting the last workgroup to arrive merge
+// them in place needs device-scope fences, and on this chip (one L2 per XCD) each such fence
+// writes back and invalidates an L2, which cost 130 us a call when it was tried.
+namespace {
+struct FusedDecodeArgs {
+  DecodeArgs d;
+  const float* q_gain;    // [hd] or null
+  const float* k_gain;    // [hd] or null
+  float eps;
+  const float* inv_freq;  // [rot/2] or null
+  int rot, variant;       // 0 half split, 1 interleaved
+  long ld;                // row stride of qkv
+};
+
+// Rotation factors of this lane's 8 elements at position `pos` (the same for every head).
+struct Rot8 {
+  float c[EPL], s[EPL];
+};
+
+__device__ __forceinline__ Rot8 rotation8(int e0, const float* inv_freq, int rot, int variant, int pos) {
+  Rot8 r;
+  const int half = rot / 2;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = e0 + i;
+    r.c[i] = 1.f;
+    r.s[i] = 0.f;
+    if (inv_freq && e < rot) {
+      const int j = variant == 1 ? e / 2 : (e < half ? e : e - half);
+      sincosf((float)pos * inv_freq[j], &r.s[i], &r.c[i]);
+    }
+  }
+  return r;
+}
+
+// Norm (optional) and rotation of one head held 8 elements per lane by LPK neighbouring lanes.
+// `v` are this lane's elements e0 .. e0+7 of the head; returns them normed and rotated.
+template <int LPK>
+__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
+                                           const Rot8& rt, int rot, int variant, int lane) {
+  const bool active = e0 < hd;
+  if (gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
+#pragma unroll
+    for (int o = 1; o < LPK; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
+  }
+  if (!rotate) return;
+  const int half = rot / 2;
+  if (variant == 1) {  // pairs (2j, 2j+1) lie in one lane
+#pragma unroll
+    for (int i = 0; i < EPL; i += 2) {
+      if (e0 + i + 1 < rot) {
+        const float x0 = v[i], x1 = v[i + 1];
+        v[i] = x0 * rt.c[i] - x1 * rt.s[i];
+        v[i + 1] = x0 * rt.s[i] + x1 * rt.c[i];
+      }
+    }
+    return;
+  }
+  // half split: element e pairs with e + half (e < half) or e - half; the partner lies half/8 lanes away
+  const int shift = half / EPL;  // half is a multiple of 8 (rotary sizes in steps of 16)
+  const int base = lane - lane % LPK;
+  const int sub = lane % LPK;
+  const bool low = e0 < half;
+  const int partner = base + (low ? sub + shift : sub - shift);
+  const int src = (partner >= base && partner < base + LPK) ? partner : lane;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const float other = __shfl(v[i], src, WAVE);
+    if (e0 + i < rot) v[i] = low ? v[i] * rt.c[i] - other * rt.s[i] : other * rt.s[i] + v[i] * rt.c[i];
+  }
+}
+
+template <int LPK, int GT>
+__global__ __launch_bounds__(256) void attention_decode_fused_kernel(const bf16* __restrict__ qkv,
+                                                                     bf16* __restrict__ kpages, bf16* __restrict__ vpages,
+                                                                     float* __restrict__ partial, bf16* __restrict__ out,
+                                                                     FusedDecodeArgs fa) {
+  constexpr int KPW = WAVE / LPK;
+  constexpr int MAX_HD = LPK * EPL;
+  __shared__ float s_ml[4][GT][2];
+  __shared__ float s_acc[4][GT][MAX_HD];
+  __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
+  const DecodeArgs& a = fa.d;
+
+  const int row = blockIdx.x;
+  const int kvh = blockIdx.y / a.head_chunks, hc = blockIdx.y % a.head_chunks;
+  const int split = blockIdx.z;
+  const int G = a.nh / a.nkv;
+  const int g0 = hc * GT;
+  const int gcount = min(GT, G - g0);
+  const int hd = a.hd;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int grp = lane / LPK, sub = lane % LPK;
+  const int e0 = sub * EPL;
+  const bool active = e0 < hd;
+
+  const int p = a.pos[row];
+  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+  const int len = p + 1 - lo;
+  int per = (len + a.n_splits - 1) / a.n_splits;
+  per = (per + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+  const int k0 = lo + split * per;
+  const int k1 = min(k0 + per, p + 1);
+  const int* table = a.table + (size_t)a.row_req[row] * a.max_pages;
+  const bf16* qrow = qkv + (size_t)row * fa.ld;
+
+  const Rot8 rt = rotation8(e0, fa.inv_freq, fa.rot, fa.variant, p);
+  const bool rotate = fa.inv_freq != nullptr;
+  // the row's own key and value: wave 0's first LPK lanes prepare them for everyone
+  const bool has_new = p >= k0 && p < k1;
+  if (has_new && wave == 0 && grp == 0) {
+    float kf[EPL], vf[EPL];
+    if (active) {
+      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0), kf);
+      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0), vf);
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
+    }
+    norm_rope8<LPK>(kf, e0, hd, fa.k_gain, fa.eps, rotate, rt, fa.rot, fa.variant, lane);
+    if (active) {
+      // what later steps read from the page is the bfloat16 value: use the same value now
+      uint32_t kw[4], vw[4];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const bf16 kb = (bf16)kf[i];
+        kf[i] = (float)kb;
+        s_knew[e0 + i] = kf[i];
+        s_vnew[e0 + i] = vf[i];
+        const uint32_t kbits = __float_as_uint(kf[i]) >> 16, vbits = __float_as_uint(vf[i]) >> 16;
+        if (i % 2 == 0) { kw[i / 2] = kbits; vw[i / 2] = vbits; }
+        else { kw[i / 2] |= kbits << 16; vw[i / 2] |= vbits << 16; }
+      }
+      if (hc == 0) {
+        const int page = table[p / a.page_size];
+        if (page >= 0 && page < a.num_pages) {
+          const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + p % a.page_size) * hd + e0;
+          *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
+          *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+        }
+      }
+    }
+  }
+
+  float qf[GT][EPL];
+  float m[GT], l[GT], acc[GT][EPL];
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    m[g] = -INFINITY;
+    l[g] = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) { acc[g][i] = 0.f; qf[g][i] = 0.f; }
+    if (g < gcount) {
+      if (active) unpack8(*(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0), qf[g]);
+      norm_rope8<LPK>(qf[g], e0, hd, fa.q_gain, fa.eps, rotate, rt, fa.rot, fa.variant, lane);
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) qf[g][i] = (float)(bf16)qf[g][i] * a.scale;   // q is bfloat16 where it is stored
+    }
+  }
+  __syncthreads();  // s_knew, s_vnew
+
+  for (int key = k0 + wave * KPW + grp; key < k1; key += 4 * KPW) {
+    float kf[EPL], vf[EPL];
+    if (key == p) {
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) { kf[i] = active ? s_knew[e0 + i] : 0.f; vf[i] = active ? s_vnew[e0 + i] : 0.f; }
+    } else if (active) {
+      int page = table[key / a.page_size];
+      page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);
+      const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + key % a.page_size) * hd + e0;
+      unpack8(*(const uint4*)(kpages + off), kf);
+      unpack8(*(const uint4*)(vpages + off), vf);
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
+    }
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (g >= gcount) break;
+      float d = 0.f;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
+#pragma unroll
+      for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
+      const float m_new = fmaxf(m[g], d);
+      const float keep = __expf(m[g] - m_new);
+      const float w = __expf(d - m_new);
+      l[g] = l[g] * keep + w;
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
+      m[g] = m_new;
+    }
+  }
+
+#pragma unroll
+  for (int g = 0; g < GT; ++g) {
+    if (g >= gcount) break;
+#pragma unroll
+    for (int o = LPK; o < WAVE; o <<= 1) {
+      const float mb = __shfl_xor(m[g], o, WAVE), lb = __shfl_xor(l[g], o, WAVE);
+      float ab[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) ab[i] = __shfl_xor(acc[g][i], o, WAVE);
+      fold<EPL>(m[g], l[g], acc[g], mb, lb, ab);
+    }
+    if (grp == 0) {
+      if (sub == 0) { s_ml[wave][g][0] = m[g]; s_ml[wave][g][1] = l[g]; }
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) s_acc[wave][g][e0 + i] = acc[g][i];
+    }
+  }
+  __syncthreads();
+  if (wave == 0 && grp == 0) {
+#pragma unroll
+    for (int g = 0; g < GT; ++g) {
+      if (g >= gcount) break;
+      float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
+      for (int w = 1; w < 4; ++w) {
+        float ab[EPL];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
+        fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
+      }
+      const int head = kvh * G + g0 + g;
+      if (a.n_splits == 1) {
+        if (active) {
+          const float inv = 1.0f / ll;
+          bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
+#pragma unroll
+          for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
+        }
+      } else {
+        float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
+        if (sub == 0) { ps[0] = mm; ps[1] = ll; }
+        if (active) {
+#pragma unroll
+          for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
+        }
+      }
+    }
+  }
+}
+
+template <int LPK>
+void launch_decode_fused(int gt, dim3 grid, hipStream_t stream, const bf16* qkv, bf16* k, bf16* v, float* partial,
+                         bf16* out, const FusedDecodeArgs& a) {
+  switch (gt) {
+    case 1: attention_decode_fused_kernel<LPK, 1><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
+    case 2: attention_decode_fused_kernel<LPK, 2><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
+    case 4: attention_decode_fused_kernel<LPK, 4><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
+    default: attention_decode_fused_kernel<LPK, 8><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
+  }
+}
+}  // namespace
+
+// qkv: [N, ld] bfloat16, raw projection (q heads, k heads, v heads) of N decoded tokens, one per request.
+GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, void* vpages, void* out, float* partial,
+                                              const float* q_gain, const float* k_gain, float eps,
+                                              const float* inv_freq, int rot, int variant, const int* pos,
+                                              const int* row_req, const int* table, int max_pages, int page_size,
+                                              int num_pages, int n_rows, int nh, int nkv, int hd, long ld, long ldo,
+                                              float scale, int window, int n_splits, hipStream_t stream) {
+  GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_decode_fused: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
+  GIBBS_REQUIRE(nh % nkv == 0, "attention_decode_fused: %d heads are not a multiple of %d kv heads", nh, nkv);
+  GIBBS_REQUIRE(hd % 16 == 0 && hd <= 256, "attention_decode_fused: head size %d must be a multiple of 16 up to 256", hd);
+  GIBBS_REQUIRE(ld % 8 == 0 && ((uintptr_t)qkv % 16) == 0 && ld >= (long)(nh + 2 * nkv) * hd, "attention_decode_fused: qkv rows must be 16-byte aligned and hold q, k and v");
+  GIBBS_REQUIRE(ldo >= (long)nh * hd, "attention_decode_fused: output rows shorter than heads * hd");
+  GIBBS_REQUIRE(!inv_freq || (rot > 0 && rot % 16 == 0 && rot <= hd), "attention_decode_fused: rotary_dim %d must be a multiple of 16 within the head size %d", rot, hd);
+  GIBBS_REQUIRE(variant == 0 || variant == 1, "attention_decode_fused: unknown rotation variant %d", variant);
+  GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_decode_fused: bad cache geometry");
+  GIBBS_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || partial), "attention_decode_fused: %d key slices need a workspace", n_splits);
+  if (n_rows == 0) return 0;
+  const int G = nh / nkv;
+  const int gt = G >= 8 ? 8 : (G > 2 ? 4 : G);
+  const int head_chunks = ceil_div(G, gt);
+  GIBBS_REQUIRE((long)nkv * head_chunks <= 65535, "attention_decode_fused: too many heads");
+  FusedDecodeArgs fa{};
+  fa.d = DecodeArgs{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ld, ldo, scale, window, n_splits, head_chunks};
+  fa.q_gain = q_gain; fa.k_gain = k_gain; fa.eps = eps; fa.inv_freq = inv_freq; fa.rot = rot; fa.variant = variant;
+  fa.ld = ld;
+  dim3 grid(n_rows, nkv * head_chunks, n_splits);
+  const bf16* qq = (const bf16*)qkv;
+  bf16 *kk = (bf16*)kpages, *vv = (bf16*)vpages, *oo = (bf16*)out;
+  const int lanes = hd / EPL;
+  if (lanes <= 2) launch_decode_fused<2>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
+  else if (lanes <= 4) launch_decode_fused<4>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
+  else if (lanes <= 8) launch_decode_fused<8>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
+  else if (lanes <= 16) launch_decode_fused<16>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
+  else launch_decode_fused<32>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return gibbs_fail("attention_decode_fused: %s", hipGetErrorString(e));
+  if (n_splits > 1) {
+    dim3 mgrid(n_rows, ceil_div(nh, 4));
+    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, oo, nh, hd, n_splits, ldo);
+  }
+  GIBBS_LAUNCH_STATUS("attention_decode_fused");
 }

@@ -1,0 +1,296 @@
+// Decode-step matrix products with the neighbouring operations fused in, so that a layer is a
+// handful of kernels instead of a dozen (no kernel on this chip is shorter than about 4 us, and
+// a decode step at small batch is a chain of products that each stream a few megabytes).
+//
+//   Y = X W^T for at most 64 rows of X (bfloat16), W streamed once straight into the A operand of
+//   v_mfma_f32_16x16x32_bf16, the workgroup's waves splitting k and meeting in LDS, as in
+//   gemm_skinny.  On top of that:
+//
+//   prologue RMS   the rows of X are the bfloat16 mirror of the residual stream; the workgroup sums
+//                  their squares from the B operands it loads anyway and scales its outputs by
+//                  1/sqrt(mean(x^2) + eps).  The norm's gain is folded into W when weights are bound.
+//   row groups     a workgroup computes the same ROWS features of up to 3 row ranges of W (offsets
+//                  0, group_stride, 2 group_stride) so that an epilogue finds its operands in one lane:
+//                  gate and up of a GLU; B, C, x of the short convolution.
+//   epilogues      STORE     y = acc (bfloat16)
+//                  RESIDUAL  x += acc (float32 stream, each element owned by one workgroup);
+//                            xb = bfloat16(x), the mirror the next product reads
+//                  GLU       out = silu(gate) * up
+//                  CONV      bx = B * x;  cv = bias + taps . [state, bx];  y = C * cv;  state shifts
+//                            (every row is one decoded token of a different request)
+#include "common.h"
+#include <stdlib.h>
+
+namespace {
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+
+enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_GLU = 2, EPI_CONV = 3 };
+constexpr int MAX_TAPS = 8;
+
+struct FusedArgs {
+  const bf16* W;
+  const bf16* X;   // [N, I] bfloat16 (the mirror of the residual stream when rms)
+  int N, O, I;     // O: features per row group
+  long ldw, ldx;
+  long group_stride;  // rows of W between row groups
+  float eps;          // rms prologue
+  // STORE / GLU / CONV: bfloat16 output [N, ldy]
+  bf16* Y;
+  long ldy;
+  // RESIDUAL
+  float* x;   // [N, O] float32, updated in place
+  bf16* xb;   // [N, O] mirror
+  // CONV
+  const float* taps;  // [O, K]
+  const float* bias;  // [O] or null
+  float* state;       // [slots, K-1, O]
+  long slot_stride;
+  const int* slot;  // [N]
+  const int* ctx;   // [N] cached length of each row's request (history rows before position 0 are zero)
+  int K;
+};
+
+template <int NT, int RG, int ROWS, int WAVES, bool RMS, int EPI>
+__global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
+  __shared__ floatx4 red[WAVES / 2][RG][NT][WAVE];
+  __shared__ float red_ss[WAVES][NT][16];
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int r = lane % 16, g = lane / 16;
+  const int o0 = blockIdx.x * ROWS;
+  // the wave's share of k, in whole MFMA steps of 32
+  const int steps = (a.I + 31) / 32;
+  const int per_wave = (steps + WAVES - 1) / WAVES;
+  const int k_begin = wave * per_wave * 32;
+  const int k_end = min(a.I, k_begin + per_wave * 32);
+
+  const bool row_ok = r < ROWS && o0 + r < a.O;
+  const bf16* wrow[RG];
+#pragma unroll
+  for (int q = 0; q < RG; ++q) wrow[q] = a.W + ((size_t)q * a.group_stride + (row_ok ? o0 + r : 0)) * a.ldw + g * 8;
+  const bf16* xrow[NT];
+  bool x_ok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    x_ok[t] = t * 16 + r < a.N;
+    xrow[t] = a.X + (size_t)(x_ok[t] ? t * 16 + r : 0) * a.ldx + g * 8;
+  }
+  floatx4 acc[RG][NT];
+  float ss[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    ss[t] = 0.f;
+#pragma unroll
+    for (int q = 0; q < RG; ++q) acc[q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  constexpr int U = (RG * NT >= 6) ? 2 : 4;  // MFMA steps per iteration
+  for (int k = k_begin; k < k_end; k += 32 * U) {
+    bf16x8 av[U][RG], bv[U][NT];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kk = k + u * 32;
+      const bool k_ok = kk + g * 8 < k_end;
+#pragma unroll
+      for (int q = 0; q < RG; ++q) av[u][q] = (row_ok && k_ok) ? *(const bf16x8*)(wrow[q] + kk) : zero;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        if (RMS) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float v = (float)bv[u][t][e];
+            ss[t] = fmaf(v, v, ss[t]);
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < RG; ++q)
+          acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][q], bv[u][t], acc[q][t], 0, 0, 0);
+      }
+  }
+
+  // sum of squares of row n = t*16 + r: over the 4 lane groups, then over the waves
+  if (RMS) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      ss[t] += __shfl_xor(ss[t], 16, WAVE);
+      ss[t] += __shfl_xor(ss[t], 32, WAVE);
+      if (g == 0) red_ss[wave][t][r] = ss[t];
+    }
+  }
+  // the waves' partial products meet in a tree (fixed order of additions)
+#pragma unroll
+  for (int stride = WAVES / 2; stride >= 1; stride /= 2) {
+    if (wave >= stride && wave < 2 * stride) {
+#pragma unroll
+      for (int q = 0; q < RG; ++q)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) red[wave - stride][q][t][lane] = acc[q][t];
+    }
+    __syncthreads();
+    if (wave < stride) {
+#pragma unroll
+      for (int q = 0; q < RG; ++q)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) acc[q][t] += red[wave][q][t][lane];
+    }
+    __syncthreads();
+  }
+  if (wave != 0) return;
+
+  // D[feature g*4 + i][row r] of tile t: lane holds 4 consecutive features of one row
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int n = t * 16 + r;
+    const int o = o0 + g * 4;
+    if (n >= a.N || g * 4 >= ROWS || o >= a.O) continue;
+    float scale = 1.f;
+    if (RMS) {
+      float tot = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) tot += red_ss[w][t][r];
+      scale = 1.0f / sqrtf(tot / (float)a.I + a.eps);
+    }
+    const bool full = o + 3 < a.O;
+    if (EPI == EPI_STORE) {
+      bf16* y = a.Y + (size_t)n * a.ldy + o;
+      if (full && a.ldy % 4 == 0) {
+        *(bf16x4*)y = bf16x4{(bf16)(acc[0][t][0] * scale), (bf16)(acc[0][t][1] * scale), (bf16)(acc[0][t][2] * scale),
+                             (bf16)(acc[0][t][3] * scale)};
+      } else {
+        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = (bf16)(acc[0][t][i] * scale);
+      }
+    } else if (EPI == EPI_RESIDUAL) {
+      float* xp = a.x + (size_t)n * a.O + o;
+      bf16* bp = a.xb + (size_t)n * a.O + o;
+      for (int i = 0; i < 4 && o + i < a.O; ++i) {
+        const float v = xp[i] + acc[0][t][i] * scale;
+        xp[i] = v;
+        bp[i] = (bf16)v;
+      }
+    } else if (EPI == EPI_GLU) {
+      bf16* y = a.Y + (size_t)n * a.ldy + o;
+      for (int i = 0; i < 4 && o + i < a.O; ++i) {
+        const float gt = acc[0][t][i] * scale, up = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        y[i] = (bf16)(gt * (1.0f / (1.0f + expf(-gt))) * up);
+      }
+    } else {  // EPI_CONV
+      const int K = a.K;
+      float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
+      const int before = a.ctx[n];
+      bf16* y = a.Y + (size_t)n * a.ldy + o;
+      for (int i = 0; i < 4 && o + i < a.O; ++i) {
+        const int c = o + i;
+        const float bx = (acc[0][t][i] * scale) * (acc[RG > 2 ? 2 : 0][t][i] * scale);
+        const float cg = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        float hist[MAX_TAPS - 1];
+        float cv = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAX_TAPS - 1; ++j) {
+          hist[j] = 0.f;
+          if (j < K - 1) {
+            // history row j is position before - (K-1) + j; rows before the sequence start are zero
+            if (before - (K - 1) + j >= 0) hist[j] = st[(size_t)j * a.O + c];
+            cv = fmaf(a.taps[(size_t)c * K + j], hist[j], cv);
+          }
+        }
+        cv = fmaf(a.taps[(size_t)c * K + K - 1], bx, cv);
+        if (a.bias) cv += a.bias[c];
+        y[i] = (bf16)(cg * cv);
+#pragma unroll
+        for (int j = 0; j < MAX_TAPS - 2; ++j)
+          if (j + 1 < K - 1) st[(size_t)j * a.O + c] = hist[j + 1];
+        st[(size_t)(K - 2) * a.O + c] = bx;
+      }
+    }
+  }
+}
+
+template <int NT, int RG, bool RMS, int EPI>
+void launch_rows(const FusedArgs& a, hipStream_t s) {
+  // few features: halve the rows per workgroup so that every compute unit gets one
+  static const int rows8_below = getenv("GIBBS_SKINNY_ROWS8_BELOW") ? atoi(getenv("GIBBS_SKINNY_ROWS8_BELOW")) : 256;
+  if (a.O / 16 < rows8_below) {
+    gemm_skinny_fused_kernel<NT, RG, 8, 8, RMS, EPI><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+  } else {
+    gemm_skinny_fused_kernel<NT, RG, 16, 8, RMS, EPI><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+  }
+}
+
+template <int RG, bool RMS, int EPI>
+void launch_nt(const FusedArgs& a, hipStream_t s) {
+  const int nt = ceil_div(a.N, 16);
+  if (nt == 1) launch_rows<1, RG, RMS, EPI>(a, s);
+  else if (nt == 2) launch_rows<2, RG, RMS, EPI>(a, s);
+  else if (nt == 3) launch_rows<3, RG, RMS, EPI>(a, s);
+  else launch_rows<4, RG, RMS, EPI>(a, s);
+}
+
+int check_common(const char* what, const void* X, const void* W, int N, int O, int I, long ldx, long ldw) {
+  GIBBS_REQUIRE(N > 0 && N <= 64 && O > 0 && I > 0, "%s: bad sizes N=%d O=%d I=%d (N up to 64)", what, N, O, I);
+  GIBBS_REQUIRE(I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "%s: inner size %d and row strides (%ld, %ld) must be multiples of 8", what, I, ldx, ldw);
+  GIBBS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "%s: operands must be 16-byte aligned", what);
+  GIBBS_REQUIRE(ldx >= I && ldw >= I, "%s: row strides shorter than rows", what);
+  return 0;
+}
+}  // namespace
+
+// Y[n, o] = scale_n * sum_k X[n, k] W[o, k], bfloat16 out; scale_n = 1/sqrt(mean_k X[n,k]^2 + eps) if rms.
+GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N, int O, int I, long ldx, long ldw,
+                                    long ldy, int rms, float eps, hipStream_t stream) {
+  if (check_common("skinny_store", X, W, N, O, I, ldx, ldw)) return 1;
+  GIBBS_REQUIRE(ldy >= O, "skinny_store: output rows shorter than %d", O);
+  FusedArgs a{};
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.Y = (bf16*)Y; a.ldy = ldy;
+  if (rms) launch_nt<1, true, EPI_STORE>(a, stream);
+  else launch_nt<1, false, EPI_STORE>(a, stream);
+  GIBBS_LAUNCH_STATUS("skinny_store");
+}
+
+// x[n, o] += sum_k X[n, k] W[o, k];  xb[n, o] = bfloat16(x[n, o]).  x: [N, O] float32, xb: [N, O] bfloat16.
+GIBBS_EXPORT int gibbs_skinny_residual(const void* X, const void* W, float* x, void* xb, int N, int O, int I, long ldx,
+                                       long ldw, hipStream_t stream) {
+  if (check_common("skinny_residual", X, W, N, O, I, ldx, ldw)) return 1;
+  FusedArgs a{};
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx;
+  a.x = x; a.xb = (bf16*)xb;
+  launch_nt<1, false, EPI_RESIDUAL>(a, stream);
+  GIBBS_LAUNCH_STATUS("skinny_residual");
+}
+
+// out[n, f] = silu(s_n gate_f . X_n) * (s_n up_f . X_n); W = [gate rows (F); up rows (F)], rms prologue.
+GIBBS_EXPORT int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw,
+                                  long ldy, int rms, float eps, hipStream_t stream) {
+  if (check_common("skinny_glu", X, W, N, F, I, ldx, ldw)) return 1;
+  GIBBS_REQUIRE(ldy >= F, "skinny_glu: output rows shorter than %d", F);
+  FusedArgs a{};
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy;
+  if (rms) launch_nt<2, true, EPI_GLU>(a, stream);
+  else launch_nt<2, false, EPI_GLU>(a, stream);
+  GIBBS_LAUNCH_STATUS("skinny_glu");
+}
+
+// In-projection and gated short convolution of N decoded tokens of N different requests:
+// W = [B rows (C); C rows (C); x rows (C)]; y[n, c] = Cg * (bias + taps . [state, B*x]); state shifts.
+GIBBS_EXPORT int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N, int C, int I, long ldx, long ldw,
+                                   int rms, float eps, const float* taps, const float* bias, float* state,
+                                   long slot_stride, const int* slot, const int* ctx, int K, hipStream_t stream) {
+  if (check_common("skinny_conv", X, W, N, C, I, ldx, ldw)) return 1;
+  GIBBS_REQUIRE(K >= 2 && K <= MAX_TAPS, "skinny_conv: kernel length %d outside 2..%d", K, MAX_TAPS);
+  GIBBS_REQUIRE(slot_stride >= (long)(K - 1) * C, "skinny_conv: state slot stride %ld shorter than (K-1)*C", slot_stride);
+  FusedArgs a{};
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = C; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.group_stride = C; a.Y = (bf16*)Y; a.ldy = C;
+  a.taps = taps; a.bias = bias; a.state = state; a.slot_stride = slot_stride; a.slot = slot; a.ctx = ctx; a.K = K;
+  if (rms) launch_nt<3, true, EPI_CONV>(a, stream);
+  else launch_nt<3, false, EPI_CONV>(a, stream);
+  GIBBS_LAUNCH_STATUS("skinny_conv");
+}

@@ -28,7 +28,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ x, const T* __restrict__ 
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = xr[i];
     if (dr && !write_x) v += to_float(dr[i]);
-    o[i] = from_float<T>(v * scale * gain[i]);
+    o[i] = from_float<T>(gain ? v * scale * gain[i] : v * scale);
   }
 }
 
@@ -79,7 +79,7 @@ __global__ void add_partials_rmsnorm_kernel(float* __restrict__ x, const float* 
       for (int s = 0; s < n_partials; ++s) d += pr[(size_t)s * partial_stride + i];
       v += d;
     }
-    o[i] = from_float<T>(v * scale * gain[i]);
+    o[i] = from_float<T>(gain ? v * scale * gain[i] : v * scale);
   }
 }
 
@@ -103,19 +103,26 @@ GIBBS_EXPORT int gibbs_add_partials_rmsnorm(float* x, const float* partials, int
 // x[r] += delta[r] alone (the last residual add of a model whose tail norms only some rows
 // still has to leave x whole for callers that read it).
 template <typename T>
-__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, size_t count) {
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, bf16* __restrict__ mirror,
+                                    size_t count) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < count) x[i] += to_float(delta[i]);
+  if (i < count) {
+    const float v = delta ? x[i] + to_float(delta[i]) : x[i];
+    x[i] = v;
+    if (mirror) mirror[i] = (bf16)v;
+  }
 }
 
-GIBBS_EXPORT int gibbs_residual_add(float* x, const void* delta, int dtype, long count, hipStream_t stream) {
+// x += delta (delta may be null); mirror (optional) = bfloat16(x).
+GIBBS_EXPORT int gibbs_residual_add(float* x, const void* delta, int dtype, void* mirror, long count,
+                                    hipStream_t stream) {
   GIBBS_REQUIRE(count >= 0, "residual_add: bad count");
   if (count == 0) return 0;
   const int blocks = ceil_div(count, 256);
   if (dtype == GIBBS_F32)
-    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)count);
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (bf16*)mirror, (size_t)count);
   else if (dtype == GIBBS_BF16)
-    residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (size_t)count);
+    residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (bf16*)mirror, (size_t)count);
   else
     return gibbs_fail("residual_add: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("residual_add");

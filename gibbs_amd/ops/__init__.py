@@ -17,8 +17,9 @@ def _i32(t: torch.Tensor, n: int, what: str) -> None:
         raise KernelError(f"{what} must be a contiguous int32 tensor of at least {n} elements")
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, n: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """x[n, :] = float32(table[ids[n], :])."""
+def embed(table: torch.Tensor, ids: torch.Tensor, n: int, out: Optional[torch.Tensor] = None,
+          mirror: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x[n, :] = float32(table[ids[n], :]); `mirror` (optional, bfloat16 [n, hidden]) gets the same rows."""
     require_cuda(table, ids)
     vocab, hidden = table.shape
     _i32(ids, n, "ids")
@@ -26,11 +27,13 @@ def embed(table: torch.Tensor, ids: torch.Tensor, n: int, out: Optional[torch.Te
         out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
     assert out.dtype == torch.float32 and out.is_contiguous() and out.shape == (n, hidden)
     assert table.is_contiguous()
-    call("gibbs_embed", ptr(table), dtype_code(table.dtype), ptr(ids), ptr(out), n, hidden, vocab, stream())
+    if mirror is not None:
+        assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, hidden) and mirror.is_contiguous()
+    call("gibbs_embed", ptr(table), dtype_code(table.dtype), ptr(ids), ptr(out), ptr(mirror), n, hidden, vocab, stream())
     return out
 
 
-def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tensor, eps: float,
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[torch.Tensor], eps: float,
                 out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None, n_out: Optional[int] = None,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """v = x (+ delta); x <- v when all rows are normed; out = v * rsqrt(mean(v^2) + eps) * gain.
@@ -39,7 +42,7 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
     require_cuda(x, delta, gain, rows)
     n, hidden = x.shape
     assert x.dtype == torch.float32 and x.is_contiguous()
-    assert gain.dtype == torch.float32 and gain.shape == (hidden,) and gain.is_contiguous()
+    assert gain is None or (gain.dtype == torch.float32 and gain.shape == (hidden,) and gain.is_contiguous())
     partials = delta is not None and delta.dim() == 3
     if partials:
         assert delta.dtype == torch.float32 and delta.shape[1:] == x.shape and delta.is_contiguous()
@@ -62,10 +65,19 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: torch.Tens
     return out
 
 
-def residual_add(x: torch.Tensor, delta: torch.Tensor) -> None:
-    require_cuda(x, delta)
-    assert x.dtype == torch.float32 and x.is_contiguous() and delta.is_contiguous() and delta.shape == x.shape
-    call("gibbs_residual_add", ptr(x), ptr(delta), dtype_code(delta.dtype), x.numel(), stream())
+def residual_add(x: torch.Tensor, delta: Optional[torch.Tensor], mirror: Optional[torch.Tensor] = None) -> None:
+    """x += delta (if given; float32 parts [S, N, H] are summed first); `mirror` (optional, bfloat16,
+    same shape as x) = bfloat16(x)."""
+    require_cuda(x, delta, mirror)
+    assert x.dtype == torch.float32 and x.is_contiguous()
+    if delta is not None:
+        if delta.dim() == 3:
+            delta = delta.sum(0)
+        assert delta.is_contiguous() and delta.shape == x.shape
+    if mirror is not None:
+        assert mirror.dtype == torch.bfloat16 and mirror.shape == x.shape and mirror.is_contiguous()
+    call("gibbs_residual_add", ptr(x), ptr(delta), dtype_code(delta.dtype) if delta is not None else 0, ptr(mirror),
+         x.numel(), stream())
 
 
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -139,6 +151,120 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
     call("gibbs_gemm_skinny", ptr(x), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i, ldx, w.stride(0), o, k_splits,
          stream())
+    return out
+
+
+def _skinny_check(x: torch.Tensor, w: torch.Tensor, what: str) -> tuple[int, int, int]:
+    require_cuda(x, w)
+    assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2
+    assert x.shape[1] == w.shape[1] and x.stride(1) == 1 and w.stride(1) == 1, (x.shape, w.shape)
+    n, i = x.shape
+    if not 1 <= n <= 64:
+        raise KernelError(f"{what} takes 1..64 rows, not {n}")
+    ldx = x.stride(0) if n > 1 else i
+    if i % 8 or ldx % 8 or w.stride(0) % 8:
+        raise KernelError(f"{what}: inner size {i} and row strides must be multiples of 8")
+    return n, i, ldx
+
+
+def skinny_store(x: torch.Tensor, w: torch.Tensor, rms_eps: Optional[float] = None,
+                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = s * (x @ w^T), bfloat16, for at most 64 rows; with `rms_eps` the rows of x are the raw
+    residual stream and s_n = 1/sqrt(mean(x_n^2) + eps) (the norm's gain being folded into w)."""
+    n, i, ldx = _skinny_check(x, w, "skinny_store")
+    o = w.shape[0]
+    if out is None:
+        out = torch.empty((n, o), dtype=torch.bfloat16, device=x.device)
+    assert out.shape == (n, o) and out.dtype == torch.bfloat16 and out.is_contiguous()
+    call("gibbs_skinny_store", ptr(x), ptr(w), ptr(out), n, o, i, ldx, w.stride(0), o, int(rms_eps is not None),
+         float(rms_eps or 0.0), stream())
+    return out
+
+
+def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor, mirror: torch.Tensor) -> None:
+    """stream_x += x_in @ w^T (float32 residual stream, in place); mirror = bfloat16(stream_x)."""
+    n, i, ldx = _skinny_check(x_in, w, "skinny_residual")
+    o = w.shape[0]
+    assert stream_x.dtype == torch.float32 and stream_x.shape == (n, o) and stream_x.is_contiguous()
+    assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, o) and mirror.is_contiguous()
+    call("gibbs_skinny_residual", ptr(x_in), ptr(w), ptr(stream_x), ptr(mirror), n, o, i, ldx, w.stride(0), stream())
+
+
+def skinny_glu(x: torch.Tensor, w_gate_up: torch.Tensor, rms_eps: Optional[float] = None,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = silu(s x @ gate^T) * (s x @ up^T) with w_gate_up = [gate rows; up rows]."""
+    n, i, ldx = _skinny_check(x, w_gate_up, "skinny_glu")
+    assert w_gate_up.shape[0] % 2 == 0 and w_gate_up.is_contiguous()
+    f = w_gate_up.shape[0] // 2
+    if out is None:
+        out = torch.empty((n, f), dtype=torch.bfloat16, device=x.device)
+    assert out.shape == (n, f) and out.dtype == torch.bfloat16 and out.is_contiguous()
+    call("gibbs_skinny_glu", ptr(x), ptr(w_gate_up), ptr(out), n, f, i, ldx, w_gate_up.stride(0), f,
+         int(rms_eps is not None), float(rms_eps or 0.0), stream())
+    return out
+
+
+def skinny_conv(x: torch.Tensor, w_in: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor],
+                state: torch.Tensor, slot: torch.Tensor, ctx: torch.Tensor, rms_eps: Optional[float] = None,
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """In-projection and gated short convolution for a step of decoded tokens (row n is one token of
+    the request in slot[n] with ctx[n] cached positions): w_in = [B rows; C rows; x rows]."""
+    n, i, ldx = _skinny_check(x, w_in, "skinny_conv")
+    require_cuda(taps, bias, state, slot, ctx)
+    c, k = taps.shape
+    assert w_in.shape[0] == 3 * c and w_in.is_contiguous()
+    assert taps.dtype == torch.float32 and taps.is_contiguous()
+    assert bias is None or (bias.dtype == torch.float32 and bias.shape == (c,) and bias.is_contiguous())
+    assert state.dtype == torch.float32 and state.shape[1:] == (k - 1, c) and state.stride(2) == 1 and state.stride(1) == c
+    _i32(slot, n, "slot"); _i32(ctx, n, "ctx")
+    if not 2 <= k <= 8:
+        raise KernelError(f"skinny_conv: kernel length {k} outside 2..8")
+    if out is None:
+        out = torch.empty((n, c), dtype=torch.bfloat16, device=x.device)
+    assert out.shape == (n, c) and out.dtype == torch.bfloat16 and out.is_contiguous()
+    call("gibbs_skinny_conv", ptr(x), ptr(w_in), ptr(out), n, c, i, ldx, w_in.stride(0), int(rms_eps is not None),
+         float(rms_eps or 0.0), ptr(taps), ptr(bias), ptr(state), state.stride(0), ptr(slot), ptr(ctx), k, stream())
+    return out
+
+
+def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
+                           vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor,
+                           row_req: torch.Tensor, scale: float, *, q_gain: Optional[torch.Tensor],
+                           k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
+                           rotary_dim: int, variant: str, window: Optional[int] = None,
+                           max_seq: int = 0, n_splits: Optional[int] = None,
+                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Decode attention straight from the raw fused projection qkv[N, (nh + 2 nkv) hd] of N decoded
+    tokens: q/k norm and rotation, the write of the new key and value to their pages, attention over
+    split keys in one kernel (followed by the merge of the slices)."""
+    require_cuda(qkv, kpages, vpages, table, pos, row_req, q_gain, k_gain, inv_freq)
+    if qkv.dtype != torch.bfloat16:
+        raise KernelError("attention_decode_fused is a bfloat16 kernel")
+    if hd % 16 or hd > 256:
+        raise KernelError(f"attention_decode_fused: head size {hd} must be a multiple of 16 up to 256")
+    assert qkv.dim() == 2 and qkv.shape[0] == n_rows and qkv.stride(1) == 1 and qkv.shape[1] >= (nh + 2 * nkv) * hd
+    num_pages, page_size = _check_pages(kpages, nkv, hd, qkv.dtype)
+    assert _check_pages(vpages, nkv, hd, qkv.dtype) == (num_pages, page_size)
+    assert table.dim() == 2 and table.shape[0] >= n_req
+    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    for g in (q_gain, k_gain):
+        assert g is None or (g.dtype == torch.float32 and g.shape == (hd,) and g.is_contiguous())
+    if inv_freq is not None:
+        assert inv_freq.dtype == torch.float32 and inv_freq.shape == (rotary_dim // 2,) and inv_freq.is_contiguous()
+        if rotary_dim % 16:
+            raise KernelError(f"attention_decode_fused: rotary_dim {rotary_dim} must be a multiple of 16")
+    if n_splits is None:
+        n_splits = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+    partial = None
+    if n_splits > 1:
+        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=qkv.device)
+    if out is None:
+        out = torch.empty((n_rows, nh * hd), dtype=qkv.dtype, device=qkv.device)
+    assert out.shape == (n_rows, nh * hd) and out.dtype == qkv.dtype and out.is_contiguous()
+    call("gibbs_attention_decode_fused", ptr(qkv), ptr(kpages), ptr(vpages), ptr(out), ptr(partial),
+         ptr(q_gain), ptr(k_gain), float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(pos),
+         ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
+         qkv.stride(0) if n_rows > 1 else qkv.shape[1], nh * hd, float(scale), int(window or 0), n_splits, stream())
     return out
 
 

@@ -23,15 +23,25 @@ class KernelError(RuntimeError):
 
 
 _SIGNATURES = {
-    "gibbs_embed": [c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
+    "gibbs_embed": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "gibbs_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "gibbs_residual_add": [c_void_p, c_void_p, c_int, c_long, c_void_p],
+    "gibbs_residual_add": [c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
     "gibbs_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_gemm_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_int,
                           c_void_p],
     "gibbs_add_partials_rmsnorm": [c_void_p, c_void_p, c_int, c_long, c_void_p, c_float, c_void_p, c_int, c_void_p,
                                    c_int, c_int, c_void_p],
+    "gibbs_skinny_store": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_int, c_float,
+                           c_void_p],
+    "gibbs_skinny_residual": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_void_p],
+    "gibbs_skinny_glu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_int, c_float,
+                         c_void_p],
+    "gibbs_skinny_conv": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_int, c_float, c_void_p,
+                          c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p],
+    "gibbs_attention_decode_fused": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_void_p],
     "gibbs_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_shortconv": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                         c_int, c_int, c_int, c_int, c_int, c_void_p],

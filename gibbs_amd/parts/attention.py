@@ -82,6 +82,28 @@ class AttentionMixer(Mixer):
         return [t for t in (self.q_gain, self.k_gain, None if self.position is None else self.position.inv_freq)
                 if t is not None]
 
+    def fold_input_gain(self, gain: torch.Tensor) -> None:
+        """The preceding norm's gain, multiplied into the columns of the q, k, v projections."""
+        self.w_qkv = (self.w_qkv.float() * gain[None, :]).to(self.w_qkv.dtype)
+
+    def can_decode_fused(self, batch) -> bool:
+        rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
+        return (self.source is None and self.hidden % 8 == 0 and self.head_dim % 16 == 0 and self.head_dim <= 256
+                and rot_ok)
+
+    def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
+        """norm -> q, k, v in one kernel; q/k norm, rotation, the write of the new key and value,
+        attention over split keys in a second (and the merge of the slices); out_proj + residual add in a third."""
+        qkv = ops.skinny_store(stream.mirror, self.w_qkv, rms_eps=norm_eps)
+        pos = self.position
+        a = ops.attention_decode_fused(
+            qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages, cache.vpages,
+            batch.tables[cache.group], batch.n_req, batch.pos, batch.row_req, self.scale, q_gain=self.q_gain,
+            k_gain=self.k_gain, eps=self.qk_norm_eps, inv_freq=None if pos is None else pos.inv_freq,
+            rotary_dim=0 if pos is None else pos.rotary_dim, variant="half_split" if pos is None else pos.variant,
+            window=self.window, max_seq=batch.max_seq)
+        ops.skinny_residual(a, self.w_out, stream.x, stream.mirror)
+
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         n = batch.n_rows

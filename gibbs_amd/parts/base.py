@@ -12,7 +12,12 @@ model it is in.  To add a part: subclass the interface, decorate the class with 
                   that the next norm adds in order); may ask for cache pages
                   (`cache_need`) and per-request state of fixed size (`state_needs`)
   FeedForward     forward(h, batch) -> delta [N, hidden]
-  Block           forward(x, pending, batch, cache) -> pending delta (arrangement of the above)
+  Block           forward(stream, batch, cache) -> stream (arrangement of the above)
+
+Optional fast-path hooks (a part without them simply takes the general path): a norm may offer
+`fold_gain()` (hand its gain over to be multiplied into the following matrices), a mixer or
+feed-forward `fold_input_gain(gain)` and `decode_fused(stream, norm_eps, batch[, cache])`, which
+runs norm + part + residual add for a step of single decoded tokens in a few fused kernels.
 """
 from __future__ import annotations
 
@@ -31,6 +36,16 @@ class Runtime:
     """What a part needs to know about the run it is bound into."""
     device: torch.device
     act_dtype: torch.dtype          # activations and cache pages: bfloat16, or float32 for the 32-bit path
+
+
+@dataclass
+class Stream:
+    """The residual stream between blocks.  `x` is float32 [N, hidden].  `pending` is a delta that
+    has not been added yet (the next norm adds it as it reads x).  `mirror`, when kept, is
+    bfloat16(x) with nothing pending: what the fused decode products read as their input."""
+    x: torch.Tensor
+    pending: Optional[torch.Tensor] = None
+    mirror: Optional[torch.Tensor] = None
 
 
 class Part:
@@ -123,9 +138,9 @@ class Block(Part):
     def small_tensors(self) -> List[torch.Tensor]:
         return [m for p in self.parts() for m in p.small_tensors()]
 
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], batch, cache) -> torch.Tensor:
-        """x: float32 residual stream, updated in place; `pending`: the previous block's last delta,
-        not yet added.  Returns this block's last delta, for the next norm to add."""
+    def forward(self, stream: Stream, batch, cache) -> Stream:
+        """Runs the block on the residual stream (updated in place) and returns it, with the
+        block's last delta either added or left pending for the next norm."""
         raise NotImplementedError
 
 

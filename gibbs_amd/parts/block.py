@@ -2,22 +2,63 @@
 
 `pre_norm` is LFM2's (/root/reference/arch/families/lfm2.json5:77-88):
     x = x + mixer(norm(x));   x = x + ffn(norm(x))
-The residual stream x is float32.  Each residual add is fused into the norm that follows it, so
-a block hands its last delta on to the next block's (or the tail's) norm instead of adding it.
+The residual stream x is float32.  On the general path each residual add is fused into the norm
+that follows it, so a block hands its last delta on instead of adding it.
+
+In bfloat16 the block folds each norm's gain into the matrices that read the normed rows (the
+reference's graph passes fold norm gains into weights too, /root/reference/src/graph/passes/mod.rs).
+A step of single decoded tokens (at most 64 rows) then takes the parts' fused decode kernels: the
+product itself computes 1/rms of its input rows, and the last product of each half adds its result
+into the stream, so a half of a layer is two or three kernels.
 """
 from __future__ import annotations
 
-from typing import Optional
-
 import torch
 
-from .base import Block, register_arrangement
+from .. import ops
+from .base import Block, Runtime, Stream, register_arrangement
+
+FUSED_DECODE_ROWS = 64
 
 
 @register_arrangement("pre_norm")
 class PreNormBlock(Block):
-    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], batch, cache) -> torch.Tensor:
-        h = self.mixer_norm.forward(x, pending)           # x += pending; h = norm(x)
-        a = self.mixer.forward(h, batch, cache)
-        h = self.ffn_norm.forward(x, a)                   # x += a; h = norm(x)
-        return self.ffn.forward(h, batch)
+    def bind(self, weights, rt: Runtime) -> None:
+        super().bind(weights, rt)
+        self.mixer_folded = self._fold(self.mixer_norm, self.mixer)
+        self.ffn_folded = self._fold(self.ffn_norm, self.ffn)
+
+    def _fold(self, norm, part) -> bool:
+        if self.rt.act_dtype != torch.bfloat16:
+            return False
+        if not (hasattr(norm, "fold_gain") and hasattr(part, "fold_input_gain")):
+            return False
+        part.fold_input_gain(norm.fold_gain())
+        return True
+
+    @staticmethod
+    def _with_mirror(stream: Stream) -> Stream:
+        """Adds what is pending and makes sure the bfloat16 mirror of x exists."""
+        if stream.pending is not None or stream.mirror is None:
+            mirror = torch.empty(stream.x.shape, dtype=torch.bfloat16, device=stream.x.device)
+            ops.residual_add(stream.x, stream.pending, mirror)
+            stream.pending, stream.mirror = None, mirror
+        return stream
+
+    def _fused(self, part, folded: bool, batch, cache=None) -> bool:
+        return (folded and self.rt.act_dtype == torch.bfloat16 and batch is not None and batch.max_q == 1
+                and batch.n_rows <= FUSED_DECODE_ROWS and hasattr(part, "decode_fused")
+                and part.can_decode_fused(batch))
+
+    def forward(self, stream: Stream, batch, cache) -> Stream:
+        if self._fused(self.mixer, self.mixer_folded, batch):
+            self.mixer.decode_fused(self._with_mirror(stream), self.mixer_norm.spec.eps, batch, cache)
+        else:
+            h = self.mixer_norm.forward(stream.x, stream.pending)       # x += pending; h = norm(x)
+            stream.pending, stream.mirror = self.mixer.forward(h, batch, cache), None
+        if self._fused(self.ffn, self.ffn_folded, batch):
+            self.ffn.decode_fused(self._with_mirror(stream), self.ffn_norm.spec.eps, batch)
+        else:
+            h = self.ffn_norm.forward(stream.x, stream.pending)
+            stream.pending, stream.mirror = self.ffn.forward(h, batch), None
+        return stream

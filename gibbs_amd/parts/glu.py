@@ -36,6 +36,18 @@ class GluFeedForward(FeedForward):
     def matrices(self):
         return [self.w_gate_up, self.w_down]
 
+    def fold_input_gain(self, gain: torch.Tensor) -> None:
+        """The preceding norm's gain, multiplied into the columns of the gate and up matrices."""
+        self.w_gate_up = (self.w_gate_up.float() * gain[None, :]).to(self.w_gate_up.dtype)
+
+    def can_decode_fused(self, batch) -> bool:
+        return self.hidden % 8 == 0 and self.inter % 8 == 0
+
+    def decode_fused(self, stream, norm_eps: float, batch) -> None:
+        """norm -> gate/up -> activation in one kernel, down + residual add in another."""
+        act = ops.skinny_glu(stream.mirror, self.w_gate_up, rms_eps=norm_eps)
+        ops.skinny_residual(act, self.w_down, stream.x, stream.mirror)
+
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         gu = linear(h, self.w_gate_up)
         return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True)

@@ -16,7 +16,7 @@ from ..cache.needs import CacheNeed, StateNeed
 from ..config.spec import ModelSpec
 from ..ops.linear import linear
 from ..weights.loader import TensorDecl, WeightStore
-from .base import Block, Part, Runtime, build_block, build_norm
+from .base import Block, Part, Runtime, Stream, build_block, build_norm
 
 
 class DecoderModel(Part):
@@ -78,11 +78,14 @@ class DecoderModel(Part):
         """Runs the batch's rows through every layer from the cache (`caches[run]` is the view of
         run number `run` of the layer order); returns float32 logits [len(logit_rows), vocab]
         (None if no logits are wanted)."""
-        x = ops.embed(self.table, batch.ids, batch.n_rows)
-        pending = None
+        mirror = None
+        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and batch.n_rows <= 64:
+            # a step of decoded tokens: the fused kernels read the stream's bfloat16 mirror
+            mirror = torch.empty((batch.n_rows, self.spec.hidden), dtype=torch.bfloat16, device=self.rt.device)
+        stream = Stream(ops.embed(self.table, batch.ids, batch.n_rows, mirror=mirror), None, mirror)
         for run, i in enumerate(self.spec.order):
-            pending = self.blocks[i].forward(x, pending, batch, caches[run])
+            stream = self.blocks[i].forward(stream, batch, caches[run])
         if batch.n_logits == 0:
             return None
-        h = self.final_norm.forward(x, pending, batch.logit_rows, batch.n_logits)
+        h = self.final_norm.forward(stream.x, stream.pending, batch.logit_rows, batch.n_logits)
         return linear(h, self.head, out_dtype=torch.float32)

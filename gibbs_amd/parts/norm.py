@@ -21,8 +21,14 @@ class RMSNorm(Norm):
         self.rt = rt
         self.gain = weights[self.spec.weight]
 
+    def fold_gain(self) -> torch.Tensor:
+        """Hands the gain over to whoever multiplies it into the matrices that read the normed
+        rows; from then on this norm only divides by the root mean square."""
+        gain, self.gain = self.gain, None
+        return gain
+
     def forward(self, x, delta, rows=None, n_rows=None):
         return ops.add_rmsnorm(x, delta, self.gain, self.spec.eps, self.rt.act_dtype, rows, n_rows)
 
     def small_tensors(self):
-        return [self.gain]
+        return [] if self.gain is None else [self.gain]

@@ -57,6 +57,20 @@ class ShortConvMixer(Mixer):
     def small_tensors(self):
         return [self.taps] + ([self.conv_bias] if self.bias else [])
 
+    def fold_input_gain(self, gain: torch.Tensor) -> None:
+        """The preceding norm's gain, multiplied into the columns of the in-projection."""
+        self.w_in = (self.w_in.float() * gain[None, :]).to(self.w_in.dtype)
+
+    def can_decode_fused(self, batch) -> bool:
+        return self.hidden % 8 == 0 and self.width % 8 == 0 and self.kernel <= 8
+
+    def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
+        """norm -> in_proj -> gated convolution with its state in one kernel, out_proj + residual
+        add in another."""
+        y = ops.skinny_conv(stream.mirror, self.w_in, self.taps, self.conv_bias, cache.states[STATE], batch.slot,
+                            batch.ctx, rms_eps=norm_eps)
+        ops.skinny_residual(y, self.w_out, stream.x, stream.mirror)
+
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         bcx = linear(h, self.w_in)
         y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,

@@ -401,3 +401,111 @@ def test_sample_against_plain():
     # temperature <= 1e-4 is greedy
     g = ops.sample(logits, torch.zeros(M, device=DEV), torch.tensor(top_p, device=DEV), i32(top_k), torch.tensor(u, device=DEV))
     assert g.tolist() == logits.argmax(-1).tolist()
+
+
+# --------------------------------------------------------------------------- fused decode kernels
+def rms_scale(x, eps):
+    return 1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
+
+
+@pytest.mark.parametrize("n,o,i", [(1, 64, 128), (8, 3072, 2048), (16, 331 * 8, 1000), (17, 200, 512), (64, 96, 4096), (5, 40, 72)])
+def test_skinny_store_with_rms_prologue(n, o, i):
+    from gibbs_amd import ops
+    x, w = rnd(n, i, dtype=torch.bfloat16, scale=3.0), rnd(o, i, dtype=torch.bfloat16, seed=1)
+    plain = x.double() @ w.double().t()
+    close(ops.skinny_store(x, w), plain, torch.bfloat16, "skinny_store", bf16=4e-3)
+    close(ops.skinny_store(x, w, rms_eps=1e-5), plain * rms_scale(x, 1e-5), torch.bfloat16, "skinny_store rms", bf16=4e-3)
+
+
+@pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96)])
+def test_skinny_residual(n, o, i):
+    from gibbs_amd import ops
+    y, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
+    x = rnd(n, o, scale=2.0, seed=2)
+    want = x.double() + y.double() @ w.double().t()
+    mirror = torch.zeros(n, o, dtype=torch.bfloat16, device=DEV)
+    ops.skinny_residual(y, w, x, mirror)
+    close(x, want, torch.float32, "skinny_residual", f32=2e-5)
+    assert torch.equal(mirror, x.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024)])
+def test_skinny_glu(n, f, i):
+    from gibbs_amd import ops
+    x, w = rnd(n, i, dtype=torch.bfloat16, scale=2.0), rnd(2 * f, i, dtype=torch.bfloat16, scale=0.05, seed=1)
+    gu = (x.double() @ w.double().t()) * rms_scale(x, 1e-6)
+    want = F.silu(gu[:, :f]) * gu[:, f:]
+    close(ops.skinny_glu(x, w, rms_eps=1e-6), want, torch.bfloat16, "skinny_glu", bf16=6e-3)
+
+
+@pytest.mark.parametrize("n,c,i,k,bias", [(1, 2048, 2048, 3, False), (8, 72, 96, 4, True), (20, 40, 64, 2, True), (64, 96, 128, 3, False)])
+def test_skinny_conv(n, c, i, k, bias):
+    """In-projection + convolution of decoded tokens against the unfused kernels and the reference."""
+    from gibbs_amd import ops
+    x = rnd(n, i, dtype=torch.bfloat16, scale=2.0)
+    w = rnd(3 * c, i, dtype=torch.bfloat16, scale=0.1, seed=1)
+    taps, b = rnd(c, k, seed=4), (rnd(c, seed=5) if bias else None)
+    slots = torch.randperm(n + 3)[:n].to(torch.int32).to(DEV)
+    ctx = i32([j % (k + 1) for j in range(n)])             # 0 (fresh), shorter than the history, longer
+    state = rnd(n + 3, k - 1, c, seed=6)
+    state2 = state.clone()
+    y = ops.skinny_conv(x, w, taps, b, state, slots, ctx, rms_eps=1e-5)
+    bcx = (x.double() @ w.double().t()) * rms_scale(x, 1e-5)
+    B, C, X = bcx[:, :c], bcx[:, c:2 * c], bcx[:, 2 * c:]
+    bx = B * X
+    for r in range(n):
+        hist = state2[slots[r]].double().clone()
+        for j in range(k - 1):
+            if int(ctx[r]) - (k - 1) + j < 0:
+                hist[j] = 0
+        window = torch.cat([hist, bx[r:r + 1]])
+        cv = (window * taps.double().t()).sum(0) + (b.double() if bias else 0)
+        close(y[r], C[r] * cv, torch.bfloat16, f"skinny_conv row {r}", bf16=8e-3)
+        close(state[slots[r]], window[1:], torch.float32, "state", f32=2e-5)
+    untouched = [s for s in range(n + 3) if s not in slots.tolist()]
+    assert torch.equal(state[untouched], state2[untouched])
+
+
+def test_embed_and_residual_mirror():
+    from gibbs_amd import ops
+    table = rnd(50, 72, dtype=torch.bfloat16)
+    mirror = torch.zeros(4, 72, dtype=torch.bfloat16, device=DEV)
+    x = ops.embed(table, i32([3, 49, 0, 3]), 4, mirror=mirror)
+    assert torch.equal(mirror.float(), x)
+    d = rnd(4, 72, dtype=torch.bfloat16, seed=3)
+    x0 = x.clone()
+    ops.residual_add(x, d, mirror)
+    assert torch.equal(x, x0 + d.float()) and torch.equal(mirror, x.to(torch.bfloat16))
+    out = ops.add_rmsnorm(x, None, None, 1e-5, torch.bfloat16)       # no gain
+    close(out, F.rms_norm(x.double(), (72,), None, 1e-5), torch.bfloat16, "gain-free norm")
+
+
+@pytest.mark.parametrize("n_splits", [1, 4, None])
+@pytest.mark.parametrize("variant", ["half_split", "interleaved"])
+@pytest.mark.parametrize("nh,nkv,hd,rot,page,window", [(4, 2, 16, 16, 16, None), (32, 8, 64, 64, 16, None), (6, 1, 48, 32, 8, None),
+                                                       (5, 5, 80, 80, 32, 37), (16, 2, 128, 128, 16, None), (24, 2, 32, 32, 16, None)])
+def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_splits):
+    """The fused decode attention against the separate kernels: same pages afterwards, same output,
+    for rows at a page's first slot, its last slot, position 0 and far into the cache."""
+    from gibbs_amd import ops
+    from gibbs_amd.parts.rope import rope_inv_freq
+    dtype = torch.bfloat16
+    seq_lens = [700, 1, 33, 16, 17]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 120, seed=7)
+    n = len(seq_lens)
+    pos, row_req = i32([l - 1 for l in seq_lens]), i32(list(range(n)))
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=9)
+    qg, kg = rnd(hd, seed=1) * 0.1 + 1, rnd(hd, seed=2) * 0.1 + 1
+    inv = torch.from_numpy(rope_inv_freq(rot, 10000.0, "f32")).to(DEV)
+    scale = 1 / math.sqrt(hd)
+    kp2, vp2, qkv2 = kp.clone(), vp.clone(), qkv.clone()
+    ops.qk_rope_kv(qkv2, n, nh, nkv, hd, q_gain=qg, k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
+                   pos=pos, row_req=row_req, kpages=kp2, vpages=vp2, table=table, n_req=n)
+    want = ops.attention_decode(qkv2, n, nh, nkv, hd, kp2, vp2, table, n, pos, row_req, scale, window, max_seq=700, n_splits=3)
+    kp1, vp1 = kp.clone(), vp.clone()
+    got = ops.attention_decode_fused(qkv, n, nh, nkv, hd, kp1, vp1, table, n, pos, row_req, scale, q_gain=qg,
+                                     k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
+                                     window=window, max_seq=700, n_splits=n_splits)
+    close(kp1, kp2, dtype, "new keys in the pages", bf16=8e-3)
+    assert torch.equal(vp1, vp2)
+    close(got, want, dtype, "fused decode attention", bf16=8e-3)
