@@ -16,6 +16,7 @@
 
 namespace {
 constexpr int EPL = 8;  // head-dim elements per lane (16 bytes of bfloat16)
+constexpr int SEG_PAGES = 512;  // page ids of a key slice kept in LDS at a time
 
 struct DecodeArgs {
   const int* pos;
@@ -37,6 +38,24 @@ __device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
     f[2 * i] = __uint_as_float(w[i] << 16);
     f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
   }
+}
+
+// Sum over the LPK neighbouring lanes that share a key, every one of them getting the total.
+// Data-parallel-primitive moves (a few cycles each) instead of LDS permutes (tens of cycles each,
+// and this sum sits on the critical path of every key): swap within pairs, within quads, then
+// mirror the half row (lane i <-> 7 - i: the other quad) and the row (i <-> 15 - i: the other half).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int LPK>
+__device__ __forceinline__ float group_sum(float v) {
+  if (LPK >= 2) v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (LPK >= 4) v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (LPK >= 8) v += dpp_move<0x141>(v);  // row_half_mirror
+  if (LPK >= 16) v += dpp_move<0x140>(v); // row_mirror
+  if (LPK >= 32) v += __shfl_xor(v, 16, WAVE);
+  return v;
 }
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -117,8 +136,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
       float d = 0.f;
 #pragma unroll
       for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
-#pragma unroll
-      for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
+      d = group_sum<LPK>(d);
       const float m_new = fmaxf(m[g], d);
       const float keep = __expf(m[g] - m_new);  // 0 at the stream's first key
       const float w = __expf(d - m_new);
@@ -332,8 +350,7 @@ __device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
-#pragma unroll
-    for (int o = 1; o < LPK; o <<= 1) ss += __shfl_xor(ss, o, WAVE);
+    ss = group_sum<LPK>(ss);
     const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
 #pragma unroll
     for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
@@ -375,6 +392,7 @@ __global__ __launch_bounds__(256) void attention_decode_fused_kernel(const bf16*
   __shared__ float s_ml[4][GT][2];
   __shared__ float s_acc[4][GT][MAX_HD];
   __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
+  __shared__ int s_pages[SEG_PAGES];
   const DecodeArgs& a = fa.d;
 
   const int row = blockIdx.x;
@@ -454,36 +472,60 @@ __global__ __launch_bounds__(256) void attention_decode_fused_kernel(const bf16*
   }
   __syncthreads();  // s_knew, s_vnew
 
-  for (int key = k0 + wave * KPW + grp; key < k1; key += 4 * KPW) {
-    float kf[EPL], vf[EPL];
-    if (key == p) {
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) { kf[i] = active ? s_knew[e0 + i] : 0.f; vf[i] = active ? s_vnew[e0 + i] : 0.f; }
-    } else if (active) {
-      int page = table[key / a.page_size];
-      page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);
-      const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + key % a.page_size) * hd + e0;
-      unpack8(*(const uint4*)(kpages + off), kf);
-      unpack8(*(const uint4*)(vpages + off), vf);
-    } else {
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
+  // The slice's page ids go to LDS first (one round trip for all of them, instead of a dependent
+  // table load in front of every key's loads); the loads of the next two keys are issued before the
+  // current key is worked on, so that memory latency overlaps the arithmetic.
+  for (int seg0 = k0; seg0 < k1; seg0 += SEG_PAGES * a.page_size) {
+    const int first_page = seg0 / a.page_size;
+    const int seg1 = min(k1, (first_page + SEG_PAGES) * a.page_size);
+    __syncthreads();  // the previous segment's ids are no longer read
+    for (int j = threadIdx.x; j < SEG_PAGES && (first_page + j) * a.page_size < seg1; j += 256) {
+      int page = table[first_page + j];
+      s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
     }
+    __syncthreads();
+    auto fetch = [&](int key, uint4& kr, uint4& vr) {
+      kr = vr = make_uint4(0, 0, 0, 0);
+      if (key < seg1 && key != p && active) {
+        const int lp = key / a.page_size;
+        const size_t off = (((size_t)s_pages[lp - first_page] * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
+        kr = *(const uint4*)(kpages + off);
+        vr = *(const uint4*)(vpages + off);
+      }
+    };
+    uint4 kraw[3], vraw[3];
+    // the wave's first key of this segment keeps the global stride pattern k0 + (4 it + wave) KPW + grp
+    int key = k0 + wave * KPW + grp;
+    if (key < seg0) key += (seg0 - key + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    fetch(key, kraw[0], vraw[0]);
+    fetch(key + 4 * KPW, kraw[1], vraw[1]);
+    for (; key < seg1; key += 4 * KPW) {
+      fetch(key + 8 * KPW, kraw[2], vraw[2]);
+      float kf[EPL], vf[EPL];
+      if (key == p) {
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      if (g >= gcount) break;
-      float d = 0.f;
+        for (int i = 0; i < EPL; ++i) { kf[i] = active ? s_knew[e0 + i] : 0.f; vf[i] = active ? s_vnew[e0 + i] : 0.f; }
+      } else {
+        unpack8(kraw[0], kf);
+        unpack8(vraw[0], vf);
+      }
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
+      for (int g = 0; g < GT; ++g) {
+        if (g >= gcount) break;
+        float d = 0.f;
 #pragma unroll
-      for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
-      const float m_new = fmaxf(m[g], d);
-      const float keep = __expf(m[g] - m_new);
-      const float w = __expf(d - m_new);
-      l[g] = l[g] * keep + w;
+        for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
+        d = group_sum<LPK>(d);
+        const float m_new = fmaxf(m[g], d);
+        const float keep = __expf(m[g] - m_new);
+        const float w = __expf(d - m_new);
+        l[g] = l[g] * keep + w;
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
-      m[g] = m_new;
+        for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
+        m[g] = m_new;
+      }
+      kraw[0] = kraw[1]; vraw[0] = vraw[1];
+      kraw[1] = kraw[2]; vraw[1] = vraw[2];
     }
   }
 

@@ -17,7 +17,9 @@ import torch
 from . import gemm_bf16, gemm_f32, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
-SKINNY_ROWS = 64
+# rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
+# output features, which stops paying beyond one or two MFMA tiles of rows)
+SKINNY_ROWS = int(os.environ.get("GIBBS_SKINNY_ROWS", "32"))
 USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 
 

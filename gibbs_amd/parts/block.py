@@ -7,7 +7,7 @@ that follows it, so a block hands its last delta on instead of adding it.
 
 In bfloat16 the block folds each norm's gain into the matrices that read the normed rows (the
 reference's graph passes fold norm gains into weights too, /root/reference/src/graph/passes/mod.rs).
-A step of single decoded tokens (at most 64 rows) then takes the parts' fused decode kernels: the
+A step of single decoded tokens (up to `FUSED_DECODE_ROWS` rows) then takes the parts' fused decode kernels: the
 product itself computes 1/rms of its input rows, and the last product of each half adds its result
 into the stream, so a half of a layer is two or three kernels.
 """
@@ -16,9 +16,10 @@ from __future__ import annotations
 import torch
 
 from .. import ops
+from ..ops.linear import SKINNY_ROWS
 from .base import Block, Runtime, Stream, register_arrangement
 
-FUSED_DECODE_ROWS = 64
+FUSED_DECODE_ROWS = SKINNY_ROWS
 
 
 @register_arrangement("pre_norm")

@@ -17,6 +17,7 @@ from ..config.spec import ModelSpec
 from ..ops.linear import linear
 from ..weights.loader import TensorDecl, WeightStore
 from .base import Block, Part, Runtime, Stream, build_block, build_norm
+from .block import FUSED_DECODE_ROWS
 
 
 class DecoderModel(Part):
@@ -79,7 +80,7 @@ class DecoderModel(Part):
         run number `run` of the layer order); returns float32 logits [len(logit_rows), vocab]
         (None if no logits are wanted)."""
         mirror = None
-        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and batch.n_rows <= 64:
+        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and batch.n_rows <= FUSED_DECODE_ROWS:
             # a step of decoded tokens: the fused kernels read the stream's bfloat16 mirror
             mirror = torch.empty((batch.n_rows, self.spec.hidden), dtype=torch.bfloat16, device=self.rt.device)
         stream = Stream(ops.embed(self.table, batch.ids, batch.n_rows, mirror=mirror), None, mirror)
