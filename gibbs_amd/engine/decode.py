@@ -23,31 +23,63 @@ from .engine import Engine, OutOfPages, StepError
 class DecodeLoop:
     def __init__(self, engine: Engine, rids: Sequence[Hashable], last_tokens: Sequence[int],
                  params: Optional[Sequence[SamplingParams]] = None, use_graph: bool = True,
-                 max_steps: int = 4096, first_index: Optional[Sequence[int]] = None):
+                 max_steps: int = 2048, first_index: Optional[Sequence[int]] = None):
         """`rids`: live requests whose prompts are cached; `last_tokens`: the token each one feeds
         next (sampled from its last logits).  `params`: per-request sampling (default greedy);
         `first_index`: for sampled requests, the output index of their next token (for the draws)."""
-        self.engine, self.rids = engine, list(rids)
-        b = self.n = len(self.rids)
-        if b == 0 or len(last_tokens) != b:
-            raise StepError("a decode loop needs one last token per request")
-        for rid in self.rids:
-            if rid not in engine.cache:
-                raise StepError(f"request {rid!r} is not live")
-        self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * b
-        self.greedy = all(p.greedy for p in self.params)
-        self.index = list(first_index) if first_index is not None else [0] * b
+        self.engine = engine
+        self.n = len(rids)
+        if self.n == 0:
+            raise StepError("a decode loop needs at least one request")
         self.use_graph = use_graph
         self.capacity = max_steps
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._allocate(params)
+        self.rebind(rids, last_tokens, params, first_index)
+
+    def _allocate(self, params) -> None:
+        """Static device buffers of a loop for `n` requests; the captured graph replays over them."""
+        engine, b = self.engine, self.n
         cm, dev = engine.cache, engine.device
+        self.greedy = params is None or all(p.greedy for p in params)
         self.width = [cm.pages_for(engine.ctx_limit) for _ in range(cm.n_groups)]
         # static metadata: ids pos row_req cu ctx slot logit_rows tables...
         sizes = [b, b, b, b + 1, b, b, b] + [b * w for w in self.width]
         offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])
         self._host = np.zeros(int(offs[-1]), dtype=np.int32)
         self._dev = torch.zeros(int(offs[-1]), dtype=torch.int32, device=dev)
-        sec = lambda i: slice(int(offs[i]), int(offs[i]) + sizes[i])
-        self._sec = [sec(i) for i in range(len(sizes))]
+        self._sec = [slice(int(offs[i]), int(offs[i]) + sizes[i]) for i in range(len(sizes))]
+        d = self._dev
+        self.batch = StepBatch(
+            n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
+            cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
+            tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
+            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=engine.ctx_limit, decode_graph=True)
+        self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
+        self.counter = torch.zeros(1, dtype=torch.int32, device=dev)
+        if not self.greedy:
+            self.temperature = torch.zeros(b, dtype=torch.float32, device=dev)
+            self.top_p = torch.zeros(b, dtype=torch.float32, device=dev)
+            self.top_k = torch.zeros(b, dtype=torch.int32, device=dev)
+            self.u_all = torch.zeros((self.capacity, b), dtype=torch.float32, device=dev)
+            self.u = torch.zeros(b, dtype=torch.float32, device=dev)
+
+    def rebind(self, rids: Sequence[Hashable], last_tokens: Sequence[int],
+               params: Optional[Sequence[SamplingParams]] = None, first_index: Optional[Sequence[int]] = None) -> None:
+        """Points the loop (and its captured graph, which only knows the static buffers) at another
+        set of as many live requests; greedy loops take greedy requests only."""
+        engine, b = self.engine, self.n
+        cm = engine.cache
+        if len(rids) != b or len(last_tokens) != b:
+            raise StepError(f"this decode loop was made for {b} requests with one last token each")
+        for rid in rids:
+            if rid not in cm:
+                raise StepError(f"request {rid!r} is not live")
+        self.rids = list(rids)
+        self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * b
+        if self.greedy != all(p.greedy for p in self.params):
+            raise StepError("a decode loop is captured either for greedy or for sampled requests")
+        self.index = list(first_index) if first_index is not None else [0] * b
         h = self._host
         h[self._sec[0]] = np.asarray(last_tokens, dtype=np.int32)
         lens = np.array([cm.tokens(r) for r in self.rids], dtype=np.int32)
@@ -59,23 +91,15 @@ class DecodeLoop:
         h[self._sec[6]] = np.arange(b)
         self._fill_tables()
         self._dev.copy_(torch.from_numpy(h))
-        d = self._dev
-        self.batch = StepBatch(
-            n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
-            cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
-            tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
-            q_lens=[1] * b, ctx_lens=lens.tolist(), slots=h[self._sec[5]].tolist(), max_q=1,
-            max_seq=engine.ctx_limit, decode_graph=True)
-        self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
-        self.counter = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.batch.ctx_lens, self.batch.slots = lens.tolist(), h[self._sec[5]].tolist()
+        self.counter.zero_()
         self.steps_done = 0
+        self.pending = 0
         if not self.greedy:
-            self.temperature = torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32, device=dev)
-            self.top_p = torch.tensor([p.resolved_top_p for p in self.params], dtype=torch.float32, device=dev)
-            self.top_k = torch.tensor([p.top_k for p in self.params], dtype=torch.int32, device=dev)
-            self.u_all = torch.zeros((self.capacity, b), dtype=torch.float32, device=dev)
-            self.u = torch.zeros(b, dtype=torch.float32, device=dev)
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
+            dev = engine.device
+            self.temperature.copy_(torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32))
+            self.top_p.copy_(torch.tensor([p.resolved_top_p for p in self.params], dtype=torch.float32))
+            self.top_k.copy_(torch.tensor([p.top_k for p in self.params], dtype=torch.int32))
 
     # ------------------------------------------------------------------ host side
     def _fill_tables(self) -> None:
@@ -159,6 +183,8 @@ class DecodeLoop:
             self.engine.cache.commit(rid, self.pending)
         self.pending = 0
 
-    def tokens(self) -> List[List[int]]:
-        """Tokens sampled so far, per request (row s of the log is what step s sampled)."""
-        return self.log[:self.steps_done].cpu().numpy().T.tolist()
+    def tokens(self, last: Optional[int] = None) -> List[List[int]]:
+        """Tokens sampled since the loop was bound (or only by the last `last` steps), per request
+        (row s of the log is what step s sampled)."""
+        first = 0 if last is None else self.steps_done - last
+        return self.log[first:self.steps_done].cpu().numpy().T.tolist()

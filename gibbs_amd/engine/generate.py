@@ -14,7 +14,8 @@ import torch
 
 from ..sampling.sampler import Draw, Sampler, SamplingParams
 from .batch import Entry
-from .engine import Engine
+from .decode import DecodeLoop
+from .engine import Engine, OutOfPages
 from .scheduler import MAX_PREFILL_CHUNK, ContinuousBatchScheduler, FinishReason, StepOutput
 
 
@@ -47,8 +48,13 @@ class GenerationStats:
 
 class Generator:
     def __init__(self, engine: Engine, *, max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
-                 eos_token_ids: Optional[Sequence[int]] = None):
+                 eos_token_ids: Optional[Sequence[int]] = None, decode_burst: int = 16):
+        """`decode_burst`: while nothing waits and every running request decodes, up to this many
+        decode steps run back to back as captured graphs (0: every step goes through the host)."""
         self.engine = engine
+        self.decode_burst = decode_burst
+        self._loops: Dict[tuple, DecodeLoop] = {}
+        self._stepped = True        # a host-driven step ran since the last burst: the loops' device state is stale
         self.sampler = Sampler(engine.device)
         eos = engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids
         self.scheduler = ContinuousBatchScheduler(engine.cache, self._run, context_len=engine.ctx_limit,
@@ -65,12 +71,42 @@ class Generator:
                rid: Optional[Hashable] = None) -> Hashable:
         return self.scheduler.submit(prompt_tokens, params, rid)
 
+    def _burst(self) -> Optional[StepOutput]:
+        plan = self.scheduler.burst_plan(self.decode_burst) if self.decode_burst > 0 else None
+        if plan is None:
+            return None
+        seqs, n = plan
+        rids = [s.id for s in seqs]
+        params = [s.params for s in seqs]
+        greedy = all(p.greedy for p in params)
+        if not greedy and not all(not p.greedy for p in params):
+            return None                                     # mixed greedy and sampled: step by step
+        last = [s.output_tokens[-1] for s in seqs]
+        index = [len(s.output_tokens) for s in seqs]
+        key = (len(seqs), greedy)
+        try:
+            loop = self._loops.get(key)
+            if loop is None:
+                loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index)
+            elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:
+                loop.rebind(rids, last, params, index)
+            else:
+                loop.params, loop.index = params, [i - loop.steps_done for i in index]
+            self._stepped = False
+            loop.run(n)
+        except OutOfPages:
+            return None                                     # let the scheduler make room
+        return self.scheduler.apply_burst(seqs, loop.tokens(last=n))
+
     def step(self) -> StepOutput:
-        """One scheduler step, timed: a step that holds prompt tokens counts as prefill (with its
-        decoded tokens riding along), any other as decode."""
+        """One scheduler step (or one burst of decode steps), timed: a step that holds prompt tokens
+        counts as prefill (with its decoded tokens riding along), any other as decode."""
         torch.cuda.synchronize(self.engine.device)
         t0 = time.perf_counter()
-        out = self.scheduler.step()
+        out = self._burst()
+        if out is None:
+            out = self.scheduler.step()
+            self._stepped = True
         torch.cuda.synchronize(self.engine.device)
         dt = time.perf_counter() - t0
         self.stats.steps += 1
@@ -96,9 +132,9 @@ class Generator:
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_tokens: int = 64,
              temperature: Optional[float] = None, top_p: Optional[float] = None, top_k: int = 50, seed: int = 0,
              ignore_eos: bool = False, max_batch_tokens: int = MAX_PREFILL_CHUNK,
-             chunk: Optional[int] = None) -> List[Generation]:
+             chunk: Optional[int] = None, decode_burst: int = 16) -> List[Generation]:
     """Generates a continuation of every prompt (lists of token ids), batched continuously."""
-    gen = Generator(engine, max_batch_tokens=max_batch_tokens, chunk=chunk)
+    gen = Generator(engine, max_batch_tokens=max_batch_tokens, chunk=chunk, decode_burst=decode_burst)
     params = SamplingParams(temperature, top_p, top_k, max_tokens, seed, ignore_eos)
     rids = [gen.submit(p, params) for p in prompts]
     results = gen.run()

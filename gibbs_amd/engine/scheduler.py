@@ -297,6 +297,42 @@ class ContinuousBatchScheduler:
         return StepOutput(entries, emitted, finished, preempted, prefill_tokens, decode_tokens,
                           len(self.active), len(self.waiting))
 
+    # ------------------------------------------------------------------ bursts of decode steps
+    def burst_plan(self, cap: int) -> Optional[Tuple[List[Sequence], int]]:
+        """When nothing waits and every running request decodes, several decode steps may run back to
+        back on the device without the host in between (a captured graph per step).  Returns the
+        requests (oldest first) and how many steps all of them can still take, at most `cap`; None
+        when a step has anything else to do."""
+        if self.waiting or not self.active:
+            return None
+        if any(s.state != SequenceState.DECODING or self._remaining(s) != 1 for s in self.active):
+            return None
+        seqs = sorted(self.active, key=lambda s: s.submitted)
+        n = min(cap, min(min(s.params.max_new_tokens - len(s.output_tokens), self.context_len - len(s.tokens))
+                         for s in seqs))
+        return (seqs, n) if n >= 1 else None
+
+    def apply_burst(self, seqs: List[Sequence], tokens: List[List[int]]) -> StepOutput:
+        """Books the tokens that a burst sampled (tokens[i]: those of seqs[i], all already cached):
+        the same emitting and finishing rules as a step, token by token."""
+        self.steps += len(tokens[0]) if tokens else 0
+        emitted: List[Tuple[Hashable, int]] = []
+        finished: List[Hashable] = []
+        for seq, toks in zip(seqs, tokens):
+            for tok in toks:
+                if tok in self.eos and not seq.params.ignore_eos:
+                    self._finish(seq, FinishReason.STOP)
+                    finished.append(seq.id)
+                    break
+                seq.output_tokens.append(int(tok))
+                emitted.append((seq.id, int(tok)))
+                if (len(seq.output_tokens) >= seq.params.max_new_tokens
+                        or len(seq.tokens) >= self.context_len):
+                    self._finish(seq, FinishReason.LENGTH)
+                    finished.append(seq.id)
+                    break
+        return StepOutput([], emitted, finished, [], 0, len(emitted), len(self.active), len(self.waiting))
+
     def run(self, on_step: Optional[Callable[[StepOutput], None]] = None) -> Dict[Hashable, Sequence]:
         """Steps until every submitted request has finished."""
         while self.has_work():

@@ -63,6 +63,43 @@ def test_greedy_generation_matches_plain(dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_bursts_change_nothing(dirs, dtype):
+    """Generation with bursts of captured decode steps gives the tokens that stepping through the
+    host gives: greedy and sampled, requests of different lengths that finish at different times,
+    an end-of-sequence token inside a burst."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    d = dirs["B"]
+    prompts = [H.tokens(70 + i, n, 512) for i, n in enumerate([9, 21, 5])]
+    for temperature in (0.0, 0.9):
+        runs = []
+        for burst in (0, 5, 16):
+            eng = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+            gen = Generator(eng, decode_burst=burst, eos_token_ids=())
+            rids = [gen.submit(p, SamplingParams(temperature=temperature, max_new_tokens=n, seed=4), rid=f"r{i}")
+                    for i, (p, n) in enumerate(zip(prompts, [37, 20, 9]))]
+            res = gen.run()
+            runs.append([res[r].tokens for r in rids])
+            assert [len(t) for t in runs[-1]] == [37, 20, 9]
+            eng.cache.check()
+            assert eng.cache.free_slots() == 4
+        assert runs[0] == runs[1] == runs[2], f"temperature {temperature}"
+    # a token that the first request produces mid-way becomes the end token: what follows it is dropped
+    # (the same three requests again, so that every kernel sees the batch it saw before)
+    stop = runs[0][0][11]
+    eng = Engine(d, dtype=dtype, max_tokens=1024, max_requests=4)
+    gen = Generator(eng, decode_burst=16, eos_token_ids=(stop,))
+    rids = [gen.submit(p, SamplingParams(temperature=0.9, max_new_tokens=n, seed=4), rid=f"r{i}")
+            for i, (p, n) in enumerate(zip(prompts, [37, 20, 9]))]
+    res = gen.run()
+    for i, (rid, full) in enumerate(zip(rids, runs[0])):
+        want = full[:full.index(stop)] if stop in full else full
+        # (in bfloat16 the others go on in a smaller batch once r0 has stopped, which may round otherwise)
+        if i == 0 or dtype == "float32":
+            assert res[rid].tokens == want
+            assert res[rid].finish_reason == ("stop" if stop in full else "length")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_reference_golden_vector_through_the_engine(dirs, dtype):
     """tests/golden/lm_graphlm_lfm2.json of the reference.  32-bit path: the reference's own golden
     tolerance, rel-L2 < 1e-3 and cos > 0.9999 (tests/golden/util.rs:257-260).  bfloat16 path (the
