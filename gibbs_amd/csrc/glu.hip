@@ -16,6 +16,26 @@ __global__ void glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int F,
   out[(size_t)n * F + f] = from_float<T>(a * u);
 }
 
+// 8 elements (16 bytes of bfloat16) per thread: the pass is bound by memory traffic.
+__global__ void glu_bf16x8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int F) {
+  const int n = blockIdx.x;
+  const int f = (blockIdx.y * blockDim.x + threadIdx.x) * 8;
+  if (f >= F) return;
+  const uint4 gr = *(const uint4*)(gu + (size_t)n * 2 * F + f);
+  const uint4 ur = *(const uint4*)(gu + (size_t)n * 2 * F + F + f);
+  const uint32_t gw[4] = {gr.x, gr.y, gr.z, gr.w}, uw[4] = {ur.x, ur.y, ur.z, ur.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+    const bf16 a0 = (bf16)(g0 * (1.0f / (1.0f + expf(-g0))) * u0);
+    const bf16 a1 = (bf16)(g1 * (1.0f / (1.0f + expf(-g1))) * u1);
+    ow[i] = (uint32_t)__builtin_bit_cast(unsigned short, a0) | ((uint32_t)__builtin_bit_cast(unsigned short, a1) << 16);
+  }
+  *(uint4*)(out + (size_t)n * F + f) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 GIBBS_EXPORT int gibbs_glu(const void* gu, void* out, int dtype, int n, int F, int act, hipStream_t stream) {
   GIBBS_REQUIRE(n >= 0 && F > 0, "glu: bad sizes n=%d F=%d", n, F);
   GIBBS_REQUIRE(act == ACT_SILU, "glu: unknown activation %d", act);
@@ -24,6 +44,8 @@ GIBBS_EXPORT int gibbs_glu(const void* gu, void* out, int dtype, int n, int F, i
   dim3 grid(n, ceil_div(F, 256));
   if (dtype == GIBBS_F32)
     glu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu, (float*)out, F, act);
+  else if (dtype == GIBBS_BF16 && F % 8 == 0 && ((uintptr_t)gu % 16) == 0 && ((uintptr_t)out % 16) == 0)
+    glu_bf16x8_kernel<<<dim3(n, ceil_div(F, 8 * 256)), 256, 0, stream>>>((const bf16*)gu, (bf16*)out, F);
   else if (dtype == GIBBS_BF16)
     glu_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (bf16*)out, F, act);
   else

@@ -61,6 +61,95 @@ __global__ __launch_bounds__(256) void shortconv_kernel(
     }
   }
 }
+// The same for bfloat16 with 8 channels (16 bytes) per thread and the window kept in registers:
+// a prompt portion is a pass over 3 + 1 values per (row, channel), bound by memory traffic.
+// K is a template parameter (2..4, what LFM2 checkpoints use); other lengths take the kernel above.
+constexpr int TLV = 16;  // rows per tile (>= K - 1)
+
+__device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+template <int K>
+__global__ __launch_bounds__(64) void shortconv_bf16x8_kernel(
+    const bf16* __restrict__ bcx, const float* __restrict__ taps, const float* __restrict__ bias,
+    float* __restrict__ state, long slot_stride, const int* __restrict__ cu, const int* __restrict__ ctx,
+    const int* __restrict__ slot, bf16* __restrict__ y, int n_req, int C) {
+  int tile = blockIdx.y, r = 0, q = 0;
+  for (; r < n_req; ++r) {
+    q = cu[r + 1] - cu[r];
+    const int t = (q + TLV - 1) / TLV;
+    if (tile < t) break;
+    tile -= t;
+  }
+  if (r >= n_req) return;
+  const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+  if (c0 >= C) return;
+  const int row0 = cu[r], before = ctx[r];
+  float* st = state + (size_t)slot[r] * slot_stride;
+  const size_t ld = (size_t)3 * C;
+  float w[8][K], b[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    b[i] = bias ? bias[c0 + i] : 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) w[i][j] = taps[(size_t)(c0 + i) * K + j];
+  }
+  // B * x of row tp of this step's chunk (tp may be negative: the request's state, or zero before its start)
+  auto bx_at = [&](int tp, float* out) {
+    if (tp >= 0) {
+      const bf16* row = bcx + (size_t)(row0 + tp) * ld + c0;
+      float bv[8], xv[8];
+      unpack8(*(const uint4*)row, bv);
+      unpack8(*(const uint4*)(row + 2 * C), xv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[i] = bv[i] * xv[i];
+    } else {
+      const bool have = before + tp >= 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) out[i] = have ? st[(size_t)(K - 1 + tp) * C + c0 + i] : 0.f;
+    }
+  };
+  const int t0 = tile * TLV, t_end = min(q, t0 + TLV);
+  float win[K][8];  // win[j]: B * x of row t - (K-1) + j
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) bx_at(t0 - (K - 1) + j, win[j + 1]);
+  for (int t = t0; t < t_end; ++t) {
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) win[j][i] = win[j + 1][i];
+    bx_at(t, win[K - 1]);
+    float cg[8];
+    unpack8(*(const uint4*)(bcx + (size_t)(row0 + t) * ld + C + c0), cg);
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < K; ++j) acc = fmaf(w[i][j], win[j][i], acc);
+      acc += b[i];
+      const uint32_t bits = (uint32_t)__builtin_bit_cast(unsigned short, (bf16)(cg[i] * acc));
+      if (i % 2 == 0) ow[i / 2] = bits;
+      else ow[i / 2] |= bits << 16;
+    }
+    *(uint4*)(y + (size_t)(row0 + t) * C + c0) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+  if (tile == 0) {
+    // new[s] = window[q + s] reads old[q + s] (an index above s), so ascending s is safe
+    for (int s2 = 0; s2 < K - 1; ++s2) {
+      float v[8];
+      bx_at(q - (K - 1) + s2, v);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) st[(size_t)s2 * C + c0 + i] = v[i];
+    }
+  }
+}
 }  // namespace
 
 GIBBS_EXPORT int gibbs_shortconv(const void* bcx, const float* taps, const float* bias, float* state,
@@ -75,7 +164,15 @@ GIBBS_EXPORT int gibbs_shortconv(const void* bcx, const float* taps, const float
   if (dtype == GIBBS_F32)
     shortconv_kernel<float><<<grid, 256, 0, stream>>>((const float*)bcx, taps, bias, state, slot_stride, cu, ctx,
                                                       slot, (float*)y, n_req, C, K);
-  else if (dtype == GIBBS_BF16)
+  else if (dtype == GIBBS_BF16 && C % 8 == 0 && K >= 2 && K <= 4 && ((uintptr_t)bcx % 16) == 0 && ((uintptr_t)y % 16) == 0) {
+    dim3 vgrid(ceil_div(C, 8 * 64), ceil_div(n_rows, TLV) + n_req);
+    GIBBS_REQUIRE(vgrid.y <= 65535, "shortconv: too many row tiles (%d)", (int)vgrid.y);
+    const bf16* in = (const bf16*)bcx;
+    bf16* out = (bf16*)y;
+    if (K == 2) shortconv_bf16x8_kernel<2><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
+    else if (K == 3) shortconv_bf16x8_kernel<3><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
+    else shortconv_bf16x8_kernel<4><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
+  } else if (dtype == GIBBS_BF16)
     shortconv_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)bcx, taps, bias, state, slot_stride, cu, ctx,
                                                      slot, (bf16*)y, n_req, C, K);
   else

@@ -96,6 +96,20 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
     return out
 
 
+def gemm_bf16_plain(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """The bfloat16 product for shapes the matrix-core kernels refuse (inner size or row strides
+    that are no multiple of 8): plain FMA, float32 accumulation."""
+    require_cuda(a, w)
+    assert a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1] and a.stride(1) == 1 and w.stride(1) == 1
+    n, i = a.shape
+    o = w.shape[0]
+    out = torch.empty((n, o), dtype=out_dtype, device=a.device)
+    call("gibbs_gemm_bf16_plain", ptr(a), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i,
+         a.stride(0) if n > 1 else i, w.stride(0), o, stream())
+    return out
+
+
 def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16,
               out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[n, o] = sum_k a[n, k] * w[o, k]: bfloat16 operands on the matrix cores, float32

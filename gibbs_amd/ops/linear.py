@@ -14,7 +14,7 @@ from typing import Optional
 
 import torch
 
-from . import gemm_bf16, gemm_f32, gemm_skinny, skinny_splits
+from . import gemm_bf16, gemm_bf16_plain, gemm_f32, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
 # rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
@@ -37,6 +37,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
             raise KernelError("linear: the float32 path writes float32")
         return gemm_f32(x, w)
     if x.dtype == torch.bfloat16:
+        n, i = x.shape
+        if i % 8 or w.stride(0) % 8 or (n > 1 and x.stride(0) % 8) or x.data_ptr() % 16 or w.data_ptr() % 16:
+            return gemm_bf16_plain(x, w, out_dtype)             # what the matrix-core kernels refuse
         if 1 <= x.shape[0] <= SKINNY_ROWS:
             splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
             return gemm_skinny(x, w, out_dtype, splits)

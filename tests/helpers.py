@@ -40,8 +40,19 @@ TINY_C = {
     "conv_L_cache": 2, "conv_bias": True, "rope_theta": 500000.0, "norm_eps": 1e-6,
     "max_position_embeddings": 2048,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-GAIN_STD = {"A": 0.0, "B": 0.1, "C": 0.1}
+# Tiny D: sizes that the fast kernels refuse, so that every fallback runs: a width of 100 and a
+# feed-forward width of 150 (no multiples of 8; 226 auto-adjusted to two thirds without rounding),
+# heads of 24 (no multiple of 16), an odd vocabulary, K 5.
+TINY_D = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "num_hidden_layers": 3, "layer_types": ["conv", "full_attention", "conv"],
+    "hidden_size": 100, "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 24,
+    "block_ff_dim": 226, "block_auto_adjust_ff_dim": True, "vocab_size": 131, "tie_embedding": True,
+    "conv_L_cache": 5, "conv_bias": False, "rope_theta": 10000.0, "norm_eps": 1e-5,
+    "max_position_embeddings": 512,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
+GAIN_STD = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1}
 
 
 def make_model_dir(folder: str, name: str, seed: int = 0, std: float = 0.1, dtype: str = "bfloat16") -> str:

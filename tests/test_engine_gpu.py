@@ -10,9 +10,9 @@ from tests import helpers as H
 
 pytestmark = pytest.mark.gpu
 
-NAMES = ["A", "B", "C"]
+NAMES = ["A", "B", "C", "D"]
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 150, "B": 200, "C": 130}
+LENGTHS = {"A": 150, "B": 200, "C": 130, "D": 90}
 
 
 @pytest.fixture(scope="module")
