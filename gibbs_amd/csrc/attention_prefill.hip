@@ -21,12 +21,34 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 constexpr int BM = 64;   // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
 constexpr int LDP = BN + 8;
+constexpr int SEG_PAGES = 1024;  // page ids kept in LDS at a time (a segment of the request's block table)
+
+// Maximum / sum over the 16 lanes of a row (the lanes that hold one query row's scores), every lane
+// getting the result: data-parallel-primitive moves (swap in pairs, in quads, mirror the half row,
+// mirror the row) instead of LDS permutes, which sit on the critical path of every key tile.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_move<0xB1>(v));
+  v = fmaxf(v, dpp_move<0x4E>(v));
+  v = fmaxf(v, dpp_move<0x141>(v));
+  return fmaxf(v, dpp_move<0x140>(v));
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  v += dpp_move<0x141>(v);
+  return v + dpp_move<0x140>(v);
+}
 
 struct PrefillArgs {
   const int* cu;
   const int* ctx;
   const int* table;
   int n_req, max_pages, page_size, num_pages;
+  int page_shift;  // log2(page_size) if it is a power of two, else -1
   int nh, nkv, hd;
   long ldq, ldo;
   float scale;
@@ -44,13 +66,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   __shared__ bf16 sK[BN][LDK];
   __shared__ bf16 sVT[HD][LDP];
   __shared__ bf16 sP[4][16][LDP];
+  __shared__ int s_pages[SEG_PAGES];
 
   // which request and which 64 rows of it
   int tile = blockIdx.x, r = 0, qlen = 0;
   for (; r < a.n_req; ++r) {
     qlen = a.cu[r + 1] - a.cu[r];
     const int t = (qlen + BM - 1) / BM;
-    if (tile < t) break;
+    if (tile < t) {
+      tile = t - 1 - tile;  // a request's last rows see the most keys: those workgroups start first
+      break;
+    }
     tile -= t;
   }
   if (r >= a.n_req) return;
@@ -63,6 +89,15 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   const int p0 = a.ctx[r] + row_in_req0;             // its absolute position
   const int rows_here = min(BM, qlen - row_in_req0);
   const int* table = a.table + (size_t)r * a.max_pages;
+  // (page, slot) of a key: shifts when the page size is a power of two (integer division costs
+  // dozens of instructions, several times per thread and tile); page ids come from a segment of
+  // the block table held in LDS, so that a tile's loads do not wait for a table load first
+  int seg_first_page = 0;
+  auto logical_page = [&](int ak) -> int { return a.page_shift >= 0 ? ak >> a.page_shift : ak / a.page_size; };
+  auto page_row = [&](const bf16* pages, int ak) -> const bf16* {
+    const int lp = logical_page(ak);
+    return pages + (((size_t)s_pages[lp - seg_first_page] * a.nkv + kvh) * a.page_size + (ak - lp * a.page_size)) * HD;
+  };
 
   // Q fragments: A operand, lane holds row lr of the wave's 16 rows, d = s*32 + g*8 .. +8
   const int my_row = wave * 16 + lr;                 // row inside the tile this lane loads
@@ -83,56 +118,91 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   float m[4], l[4];
   floatx4 o[DT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) { m[i] = -INFINITY; l[i] = 0.f; }
+  // a finite stand-in for 'no key seen yet': exp2(x - m) is then 0 for masked scores and for the
+  // first rescale, with no special cases on the path of every score
+  for (int i = 0; i < 4; ++i) { m[i] = -1e30f; l[i] = 0.f; }
 #pragma unroll
   for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
+  const float scale2 = a.scale * 1.44269504088896340736f;
   const int last_pos = p0 + rows_here - 1;
   const int first_key = a.window > 0 ? max(0, p0 - a.window + 1) : 0;
   const int wave_last = p0 + min(wave * 16 + 15, rows_here - 1);
   const int wave_first_key = a.window > 0 ? max(0, p0 + wave * 16 - a.window + 1) : 0;
 
-  for (int kt = first_key / BN; kt * BN <= last_pos; ++kt) {
-    const int key0 = kt * BN;
-    __syncthreads();  // everyone is done with the previous tile
-    // K tile: 64 keys x HD, 16-byte chunks
-    for (int c = tid; c < BN * (HD / 8); c += 256) {
+  // One tile ahead: the next tile's keys and values travel from memory to registers while the
+  // matrix cores work on the current tile, and go to LDS once everyone is done with it.
+  constexpr int KCH = (BN * (HD / 8) + 255) / 256;        // 16-byte chunks of K per thread and tile
+  constexpr int VCH = ((BN / 2) * (HD / 8) + 255) / 256;  // pairs of V chunks per thread and tile
+  uint4 kreg[KCH], vreg0[VCH], vreg1[VCH];
+  auto load_tile = [&](int key0) {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * 256;
       const int key = c / (HD / 8), d = (c % (HD / 8)) * 8;
-      const int ak = key0 + key;
-      uint4 v = make_uint4(0, 0, 0, 0);
-      if (ak <= last_pos) {
-        int page = table[ak / a.page_size];
-        page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);
-        v = *(const uint4*)(kpages + (((size_t)page * a.nkv + kvh) * a.page_size + ak % a.page_size) * HD + d);
-      }
-      *(uint4*)&sK[key][d] = v;
+      kreg[i] = make_uint4(0, 0, 0, 0);
+      if (c < BN * (HD / 8) && key0 + key <= last_pos) kreg[i] = *(const uint4*)(page_row(kpages, key0 + key) + d);
     }
-    // V tile transposed: a thread takes two neighbouring keys x 8 d and writes 8 packed pairs
-    for (int c = tid; c < (BN / 2) * (HD / 8); c += 256) {
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int c = tid + i * 256;
       const int kp = c % (BN / 2), d = (c / (BN / 2)) * 8;
-      uint4 v0 = make_uint4(0, 0, 0, 0), v1 = v0;
       const int ak = key0 + 2 * kp;
-      if (ak <= last_pos) {
-        int page = table[ak / a.page_size];
-        page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);
-        v0 = *(const uint4*)(vpages + (((size_t)page * a.nkv + kvh) * a.page_size + ak % a.page_size) * HD + d);
+      vreg0[i] = vreg1[i] = make_uint4(0, 0, 0, 0);
+      if (c < (BN / 2) * (HD / 8)) {
+        if (ak <= last_pos) vreg0[i] = *(const uint4*)(page_row(vpages, ak) + d);
+        if (ak + 1 <= last_pos) vreg1[i] = *(const uint4*)(page_row(vpages, ak + 1) + d);
       }
-      if (ak + 1 <= last_pos) {
-        int page = table[(ak + 1) / a.page_size];
-        page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);
-        v1 = *(const uint4*)(vpages + (((size_t)page * a.nkv + kvh) * a.page_size + (ak + 1) % a.page_size) * HD + d);
-      }
-      const uint32_t w0[4] = {v0.x, v0.y, v0.z, v0.w}, w1[4] = {v1.x, v1.y, v1.z, v1.w};
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < KCH; ++i) {
+      const int c = tid + i * 256;
+      if (c < BN * (HD / 8)) *(uint4*)&sK[c / (HD / 8)][(c % (HD / 8)) * 8] = kreg[i];
+    }
+    // V transposed: a thread holds two neighbouring keys x 8 d and writes 8 packed pairs
+#pragma unroll
+    for (int i = 0; i < VCH; ++i) {
+      const int c = tid + i * 256;
+      if (c >= (BN / 2) * (HD / 8)) continue;
+      const int kp = c % (BN / 2), d = (c / (BN / 2)) * 8;
+      const uint32_t w0[4] = {vreg0[i].x, vreg0[i].y, vreg0[i].z, vreg0[i].w};
+      const uint32_t w1[4] = {vreg1[i].x, vreg1[i].y, vreg1[i].z, vreg1[i].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // elements d+2j and d+2j+1 of both keys
-        const uint32_t lo = (w0[j] & 0xffffu) | (w1[j] << 16);
-        const uint32_t hi = (w0[j] >> 16) | (w1[j] & 0xffff0000u);
-        *(uint32_t*)&sVT[d + 2 * j][2 * kp] = lo;
-        *(uint32_t*)&sVT[d + 2 * j + 1][2 * kp] = hi;
+        *(uint32_t*)&sVT[d + 2 * j][2 * kp] = (w0[j] & 0xffffu) | (w1[j] << 16);
+        *(uint32_t*)&sVT[d + 2 * j + 1][2 * kp] = (w0[j] >> 16) | (w1[j] & 0xffff0000u);
       }
     }
+  };
+  // the block-table segment that holds the pages of tile `key0` (tiles and segments are aligned)
+  const int seg_keys = SEG_PAGES * a.page_size / BN * BN;   // keys per segment, whole tiles
+  auto load_segment = [&](int key0) {
+    seg_first_page = logical_page(key0 / seg_keys * seg_keys);
+    const int last_page = logical_page(last_pos);
+    for (int j = tid; j < SEG_PAGES && seg_first_page + j <= last_page; j += 256) {
+      const int page = table[seg_first_page + j];
+      s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
+    }
     __syncthreads();
+  };
+
+  const int kt_first = first_key / BN;
+  load_segment(kt_first * BN);
+  load_tile(kt_first * BN);
+  for (int kt = kt_first; kt * BN <= last_pos; ++kt) {
+    const int key0 = kt * BN;
+    __syncthreads();  // everyone is done with the previous tile
+    store_tile();
+    __syncthreads();
+    if ((kt + 1) * BN <= last_pos) {
+      if (((kt + 1) * BN) % seg_keys == 0) load_segment((kt + 1) * BN);  // (uniform: everyone takes it)
+      load_tile((kt + 1) * BN);
+    }
+    // the loads above are to be in flight during the arithmetic below, not sunk to their use
+    __builtin_amdgcn_sched_barrier(0);
     // a wave whose rows see none of this tile's keys has nothing to do (it still takes part in the barriers)
     if (key0 > wave_last || key0 + BN <= wave_first_key) continue;
 
@@ -156,7 +226,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
       const int key = key0 + c * 16 + lr;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = s4[c][i] * a.scale;
+        float v = s4[c][i] * scale2;  // scores in units of log2: exp(s) = exp2(s * log2 e)
         if (need_mask) {
           const bool vis = key <= pos_i[i] && (a.window == 0 || key > pos_i[i] - a.window);
           v = vis ? v : -INFINITY;
@@ -168,11 +238,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     float keep[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-#pragma unroll
-      for (int off = 1; off < 16; off <<= 1) mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], off, WAVE));
+      mx[i] = row16_max(mx[i]);
       const float m_new = fmaxf(m[i], mx[i]);
-      // a row that has seen no key yet keeps m = -inf: exp(-inf - -inf) must not be taken
-      keep[i] = (m_new == -INFINITY) ? 1.f : __expf(m[i] - m_new);
+      keep[i] = __builtin_amdgcn_exp2f(m[i] - m_new);
       m[i] = m_new;
       l[i] *= keep[i];
     }
@@ -181,7 +249,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     for (int c = 0; c < 4; ++c)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = (m[i] == -INFINITY) ? 0.f : __expf(s4[c][i] - m[i]);
+        const float p = __builtin_amdgcn_exp2f(s4[c][i] - m[i]);
         l[i] += p;
         sP[wave][g * 4 + i][c * 16 + lr] = (bf16)p;
       }
@@ -206,8 +274,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   // row sums over the 16 lanes that share the rows; store
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-#pragma unroll
-    for (int off = 1; off < 16; off <<= 1) l[i] += __shfl_xor(l[i], off, WAVE);
+    l[i] = row16_sum(l[i]);
     const int row = wave * 16 + g * 4 + i;
     if (row >= rows_here) continue;
     const float inv = 1.0f / l[i];
@@ -232,7 +299,8 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_prefill: bad cache geometry");
   GIBBS_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
   if (n_rows == 0 || n_req == 0) return 0;
-  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window};
+  const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
+  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window};
   dim3 grid(ceil_div(n_rows, BM) + n_req, nh);
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;

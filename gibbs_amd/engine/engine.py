@@ -93,15 +93,18 @@ class Engine:
             raise StepError("a step needs at least one entry")
         seen = set()
         vocab = self.spec.vocab
+        token_arrays = []
         for e in entries:
             if e.rid in seen:
                 raise StepError(f"request {e.rid!r} appears twice in one step")
             seen.add(e.rid)
             if len(e.tokens) == 0:
                 raise StepError(f"request {e.rid!r}: no tokens")
-            bad = [t for t in e.tokens if not 0 <= int(t) < vocab]
-            if bad:
-                raise StepError(f"request {e.rid!r}: token id {bad[0]} outside the vocabulary (0..{vocab - 1})")
+            toks = np.asarray(e.tokens, dtype=np.int64)
+            token_arrays.append(toks)
+            if toks.min() < 0 or toks.max() >= vocab:
+                bad = int(toks[(toks < 0) | (toks >= vocab)][0])
+                raise StepError(f"request {e.rid!r}: token id {bad} outside the vocabulary (0..{vocab - 1})")
             if any(not 0 <= w < len(e.tokens) for w in e.want):
                 raise StepError(f"request {e.rid!r}: wanted place outside its {len(e.tokens)} tokens")
             before = self.cache.tokens(e.rid) if e.rid in self.cache else 0
@@ -135,7 +138,7 @@ class Engine:
         np.cumsum(q_lens, out=cu[1:])
         ctx = np.array([self.cache.tokens(r) for r in rids], dtype=np.int32)
         slot = np.array([self.cache.slot(r) for r in rids], dtype=np.int32)
-        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int32) for e in entries])
+        ids = np.concatenate(token_arrays).astype(np.int32)
         row_req = np.repeat(np.arange(len(entries), dtype=np.int32), q_lens)
         pos = (np.arange(ids.size, dtype=np.int32) - cu[:-1][row_req]) + ctx[row_req]
         logit_rows = np.array([cu[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)

@@ -509,3 +509,41 @@ def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_split
     close(kp1, kp2, dtype, "new keys in the pages", bf16=8e-3)
     assert torch.equal(vp1, vp2)
     close(got, want, dtype, "fused decode attention", bf16=8e-3)
+
+
+def test_attention_block_table_segments():
+    """Requests with more pages than the kernels keep in LDS at a time (pages of 2 tokens, 2,300
+    keys): the fast kernels cross from one segment of the block table to the next."""
+    from gibbs_amd import ops
+    from gibbs_amd.parts.rope import rope_inv_freq
+    dtype, nh, nkv, hd, page = torch.bfloat16, 2, 1, 32, 2
+    seq_lens = [2300, 1100]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 1800, seed=5)
+    scale = 1 / math.sqrt(hd)
+    # prompt portions ending at the last key of each request
+    q_lens = [130, 70]
+    ctx = [s - q for s, q in zip(seq_lens, q_lens)]
+    cu = np.concatenate([[0], np.cumsum(q_lens)])
+    n = int(cu[-1])
+    q = rnd(n, nh * hd, dtype=dtype, seed=9)
+    out = ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 2, i32(cu), i32(ctx), scale)
+    for r in range(2):
+        rows = slice(int(cu[r]), int(cu[r + 1]))
+        want = attention_reference(q[rows].view(-1, nh, hd), ks[r], vs[r], list(range(ctx[r], seq_lens[r])), scale, None)
+        close(out[rows].view(-1, nh, hd), want, dtype, f"prefill over segments, request {r}", bf16=1e-2)
+    # decoded rows at the last positions, one key slice and several
+    pos, row_req = i32([l - 1 for l in seq_lens]), i32([0, 1])
+    qd = rnd(2, nh * hd, dtype=dtype, seed=3)
+    want = ops.attention_plain(qd, 2, nh, nkv, hd, kp, vp, table, 2, pos, row_req, scale)
+    for ns in (1, 3):
+        close(ops.attention_decode(qd, 2, nh, nkv, hd, kp, vp, table, 2, pos, row_req, scale, n_splits=ns), want, dtype,
+              f"decode over segments, {ns} slices", bf16=1e-2)
+        qkv = torch.cat([qd, rnd(2, 2 * nkv * hd, dtype=dtype, seed=4)], dim=1).contiguous()
+        kp1, vp1, kp2, vp2, qkv2 = kp.clone(), vp.clone(), kp.clone(), vp.clone(), qkv.clone()
+        ops.qk_rope_kv(qkv2, 2, nh, nkv, hd, q_gain=None, k_gain=None, eps=0.0, inv_freq=None, rotary_dim=0,
+                       variant="half_split", pos=pos, row_req=row_req, kpages=kp2, vpages=vp2, table=table, n_req=2)
+        ref = ops.attention_plain(qkv2, 2, nh, nkv, hd, kp2, vp2, table, 2, pos, row_req, scale)
+        got = ops.attention_decode_fused(qkv, 2, nh, nkv, hd, kp1, vp1, table, 2, pos, row_req, scale, q_gain=None,
+                                         k_gain=None, eps=0.0, inv_freq=None, rotary_dim=0, variant="half_split",
+                                         n_splits=ns)
+        close(got, ref, dtype, f"fused decode over segments, {ns} slices", bf16=1e-2)
