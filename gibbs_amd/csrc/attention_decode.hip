@@ -501,6 +501,7 @@ __global__ __launch_bounds__(256) void attention_decode_fused_kernel(const bf16*
     fetch(key + 4 * KPW, kraw[1], vraw[1]);
     for (; key < seg1; key += 4 * KPW) {
       fetch(key + 8 * KPW, kraw[2], vraw[2]);
+      __builtin_amdgcn_sched_barrier(0);  // the loads above stay ahead of the arithmetic below
       float kf[EPL], vf[EPL];
       if (key == p) {
 #pragma unroll

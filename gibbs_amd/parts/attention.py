@@ -89,20 +89,25 @@ class AttentionMixer(Mixer):
     def can_decode_fused(self, batch) -> bool:
         rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
         return (self.source is None and self.hidden % 8 == 0 and self.head_dim % 16 == 0 and self.head_dim <= 256
-                and rot_ok)
+                and rot_ok and (self.heads * self.head_dim) % 8 == 0)
 
     def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
-        """norm -> q, k, v in one kernel; q/k norm, rotation, the write of the new key and value,
-        attention over split keys in a second (and the merge of the slices); out_proj + residual add in a third."""
+        """norm -> q, k, v in one kernel; q/k norm, rotation, the write of the new key and value and
+        attention over split keys in a second (and the merge of the slices); out_proj + residual
+        add in a third."""
         qkv = ops.skinny_store(stream.mirror, self.w_qkv, rms_eps=norm_eps)
+        ops.skinny_residual(self._attend_decoded(qkv, batch, cache), self.w_out, stream.x, stream.mirror)
+
+    def _attend_decoded(self, qkv, batch, cache) -> torch.Tensor:
+        """A step of single decoded tokens, from the raw projection: one kernel norms and rotates q and
+        the new key, writes key and value to their pages and attends."""
         pos = self.position
-        a = ops.attention_decode_fused(
+        return ops.attention_decode_fused(
             qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages, cache.vpages,
             batch.tables[cache.group], batch.n_req, batch.pos, batch.row_req, self.scale, q_gain=self.q_gain,
             k_gain=self.k_gain, eps=self.qk_norm_eps, inv_freq=None if pos is None else pos.inv_freq,
             rotary_dim=0 if pos is None else pos.rotary_dim, variant="half_split" if pos is None else pos.variant,
             window=self.window, max_seq=batch.max_seq)
-        ops.skinny_residual(a, self.w_out, stream.x, stream.mirror)
 
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
@@ -110,6 +115,10 @@ class AttentionMixer(Mixer):
         qkv = linear(h, self.w_qkv)
         table = batch.tables[cache.group]
         owns = self.source is None
+        rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
+        if (owns and self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and self.head_dim % 16 == 0
+                and self.head_dim <= 256 and rot_ok):
+            return linear(self._attend_decoded(qkv, batch, cache), self.w_out, partial_ok=True)
         pos = self.position
         ops.qk_rope_kv(qkv, n, self.heads, self.kv_heads if owns else 0, self.head_dim,
                        q_gain=self.q_gain, k_gain=self.k_gain, eps=self.qk_norm_eps,
