@@ -8,7 +8,20 @@
 // reads 1 KB of contiguous cache per instruction) and keep an online-softmax stream of their own
 // (max, sum, weighted values); the streams are merged at the end, first across the wave by
 // shuffles, then across the 4 waves through LDS.  With more than one slice the workgroup writes a
-// partial (max, sum, values) and a second kernel merges the slices.
+// partial (max, sum, values) and a second kernel merges the slices.  The slice's page ids are
+// staged in LDS, and the loads of the next two keys are in flight while a key is worked on.
+//
+// Two entry points share the kernel.  `attention_decode` takes q as it is (already normed and
+// rotated; the row's key and value already in their pages).  `attention_decode_fused` takes a step
+// of decoded tokens as the raw fused projection qkv[N, (nh + 2 nkv) hd]: the kernel norms and
+// rotates q on the fly (every slice's workgroup does, it is a few hundred operations), norms and
+// rotates the row's own new key, writes it and the new value to their page (the workgroup of head
+// chunk 0 whose key slice holds the row's position does) and uses them from LDS instead of
+// reading them back.
+//
+// The slices are merged by a separate kernel: letting the last workgroup to arrive merge them in
+// place needs device-scope fences, and on this chip (one L2 per XCD) each such fence writes back
+// and invalidates an L2, which cost 130 us a call when it was tried.
 //
 // Visibility is by position only: row n sees keys lo .. pos[n] of its request
 // (lo = max(0, pos - window + 1), window 0 = all).
@@ -23,12 +36,19 @@ struct DecodeArgs {
   const int* row_req;
   const int* table;
   int max_pages, page_size, num_pages;
+  int page_shift;  // log2(page_size) if it is a power of two, else -1
   int nh, nkv, hd;
-  long ldq, ldo;
+  long ldq, ldo;   // row strides of q (or of the raw qkv rows) and of the output
   float scale;
   int window;
   int n_splits;
   int head_chunks;  // workgroups per kv head along the group's query heads
+  // raw rows only: what to do to q and to the new key before they are used
+  const float* q_gain;    // [hd] or null
+  const float* k_gain;    // [hd] or null
+  float eps;
+  const float* inv_freq;  // [rot/2] or null
+  int rot, variant;       // 0 half split, 1 interleaved
 };
 
 __device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
@@ -70,16 +90,79 @@ __device__ __forceinline__ void fold(float& ma, float& la, float* aa, float mb, 
   ma = m;
 }
 
-template <int LPK, int GT>
-__global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __restrict__ q,
-                                                               const bf16* __restrict__ kpages,
-                                                               const bf16* __restrict__ vpages,
-                                                               float* __restrict__ partial, bf16* __restrict__ out,
-                                                               DecodeArgs a) {
-  constexpr int KPW = WAVE / LPK;  // keys per wave and iteration
+// Rotation factors of this lane's 8 elements at position `pos` (the same for every head).
+struct Rot8 {
+  float c[EPL], s[EPL];
+};
+
+__device__ __forceinline__ Rot8 rotation8(int e0, const float* inv_freq, int rot, int variant, int pos) {
+  Rot8 r;
+  const int half = rot / 2;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const int e = e0 + i;
+    r.c[i] = 1.f;
+    r.s[i] = 0.f;
+    if (inv_freq && e < rot) {
+      const int j = variant == 1 ? e / 2 : (e < half ? e : e - half);
+      sincosf((float)pos * inv_freq[j], &r.s[i], &r.c[i]);
+    }
+  }
+  return r;
+}
+
+// Norm (optional) and rotation of one head held 8 elements per lane by LPK neighbouring lanes.
+// `v` are this lane's elements e0 .. e0+7 of the head; returns them normed and rotated.
+template <int LPK>
+__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
+                                           const Rot8& rt, int rot, int variant, int lane) {
+  const bool active = e0 < hd;
+  if (gain) {
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
+    ss = group_sum<LPK>(ss);
+    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
+#pragma unroll
+    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
+  }
+  if (!rotate) return;
+  const int half = rot / 2;
+  if (variant == 1) {  // pairs (2j, 2j+1) lie in one lane
+#pragma unroll
+    for (int i = 0; i < EPL; i += 2) {
+      if (e0 + i + 1 < rot) {
+        const float x0 = v[i], x1 = v[i + 1];
+        v[i] = x0 * rt.c[i] - x1 * rt.s[i];
+        v[i + 1] = x0 * rt.s[i] + x1 * rt.c[i];
+      }
+    }
+    return;
+  }
+  // half split: element e pairs with e + half (e < half) or e - half; the partner lies half/8 lanes away
+  const int shift = half / EPL;  // half is a multiple of 8 (rotary sizes in steps of 16)
+  const int base = lane - lane % LPK;
+  const int sub = lane % LPK;
+  const bool low = e0 < half;
+  const int partner = base + (low ? sub + shift : sub - shift);
+  const int src = (partner >= base && partner < base + LPK) ? partner : lane;
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) {
+    const float other = __shfl(v[i], src, WAVE);
+    if (e0 + i < rot) v[i] = low ? v[i] * rt.c[i] - other * rt.s[i] : other * rt.s[i] + v[i] * rt.c[i];
+  }
+}
+
+template <int LPK, int GT, bool RAW>
+__global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
+                                                               bf16* __restrict__ vpages, float* __restrict__ partial,
+                                                               bf16* __restrict__ out, DecodeArgs a) {
+  constexpr int KPW = WAVE / LPK;
   constexpr int MAX_HD = LPK * EPL;
   __shared__ float s_ml[4][GT][2];
   __shared__ float s_acc[4][GT][MAX_HD];
+  __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
+  __shared__ int s_pages[SEG_PAGES];
 
   const int row = blockIdx.x;
   const int kvh = blockIdx.y / a.head_chunks, hc = blockIdx.y % a.head_chunks;
@@ -101,6 +184,46 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
   const int k0 = lo + split * per;
   const int k1 = min(k0 + per, p + 1);
   const int* table = a.table + (size_t)a.row_req[row] * a.max_pages;
+  const bf16* qrow = qkv + (size_t)row * a.ldq;
+
+  Rot8 rt;
+  if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p);
+  const bool rotate = a.inv_freq != nullptr;
+  // raw rows: the row's own key and value; wave 0's first LPK lanes prepare them for everyone
+  const bool has_new = RAW && p >= k0 && p < k1;
+  if (has_new && wave == 0 && grp == 0) {
+    float kf[EPL], vf[EPL];
+    if (active) {
+      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0), kf);
+      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0), vf);
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
+    }
+    norm_rope8<LPK>(kf, e0, hd, a.k_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
+    if (active) {
+      // what later steps read from the page is the bfloat16 value: use the same value now
+      uint32_t kw[4], vw[4];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) {
+        const bf16 kb = (bf16)kf[i];
+        kf[i] = (float)kb;
+        s_knew[e0 + i] = kf[i];
+        s_vnew[e0 + i] = vf[i];
+        const uint32_t kbits = __float_as_uint(kf[i]) >> 16, vbits = __float_as_uint(vf[i]) >> 16;
+        if (i % 2 == 0) { kw[i / 2] = kbits; vw[i / 2] = vbits; }
+        else { kw[i / 2] |= kbits << 16; vw[i / 2] |= vbits << 16; }
+      }
+      if (hc == 0) {
+        const int page = table[p / a.page_size];
+        if (page >= 0 && page < a.num_pages) {
+          const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + p % a.page_size) * hd + e0;
+          *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
+          *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+        }
+      }
+    }
+  }
 
   float qf[GT][EPL];
   float m[GT], l[GT], acc[GT][EPL];
@@ -110,44 +233,77 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
     l[g] = 0.f;
 #pragma unroll
     for (int i = 0; i < EPL; ++i) { acc[g][i] = 0.f; qf[g][i] = 0.f; }
-    if (g < gcount && active) {
-      const bf16* qp = q + (size_t)row * a.ldq + (size_t)(kvh * G + g0 + g) * hd + e0;
-      unpack8(*(const uint4*)qp, qf[g]);
+    if (g < gcount) {
+      if (active) unpack8(*(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0), qf[g]);
+      if (RAW) {
+        norm_rope8<LPK>(qf[g], e0, hd, a.q_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) qf[g][i] = (float)(bf16)qf[g][i];   // q is bfloat16 where it is stored
+      }
 #pragma unroll
       for (int i = 0; i < EPL; ++i) qf[g][i] *= a.scale;
     }
   }
+  __syncthreads();  // s_knew, s_vnew
 
-  for (int key = k0 + wave * KPW + grp; key < k1; key += 4 * KPW) {
-    int page = table[key / a.page_size];
-    page = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
-    const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + key % a.page_size) * hd + e0;
-    float kf[EPL], vf[EPL];
-    if (active) {
-      unpack8(*(const uint4*)(kpages + off), kf);
-      unpack8(*(const uint4*)(vpages + off), vf);
-    } else {
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
+  // The slice's page ids go to LDS first (one round trip for all of them, instead of a dependent
+  // table load in front of every key's loads); the loads of the next two keys are issued before the
+  // current key is worked on, so that memory latency overlaps the arithmetic.
+  for (int seg0 = k0; seg0 < k1; seg0 += SEG_PAGES * a.page_size) {
+    const int first_page = a.page_shift >= 0 ? seg0 >> a.page_shift : seg0 / a.page_size;
+    const int seg1 = min(k1, (first_page + SEG_PAGES) * a.page_size);
+    __syncthreads();  // the previous segment's ids are no longer read
+    for (int j = threadIdx.x; j < SEG_PAGES && (first_page + j) * a.page_size < seg1; j += 256) {
+      int page = table[first_page + j];
+      s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
     }
+    __syncthreads();
+    auto fetch = [&](int key, uint4& kr, uint4& vr) {
+      kr = vr = make_uint4(0, 0, 0, 0);
+      if (key < seg1 && !(RAW && key == p) && active) {
+        const int lp = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
+        const size_t off = (((size_t)s_pages[lp - first_page] * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
+        kr = *(const uint4*)(kpages + off);
+        vr = *(const uint4*)(vpages + off);
+      }
+    };
+    uint4 kraw[3], vraw[3];
+    // the wave's first key of this segment keeps the global stride pattern k0 + (4 it + wave) KPW + grp
+    int key = k0 + wave * KPW + grp;
+    if (key < seg0) key += (seg0 - key + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    fetch(key, kraw[0], vraw[0]);
+    fetch(key + 4 * KPW, kraw[1], vraw[1]);
+    for (; key < seg1; key += 4 * KPW) {
+      fetch(key + 8 * KPW, kraw[2], vraw[2]);
+      __builtin_amdgcn_sched_barrier(0);  // the loads above stay ahead of the arithmetic below
+      float kf[EPL], vf[EPL];
+      if (RAW && key == p) {
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      if (g >= gcount) break;
-      float d = 0.f;
+        for (int i = 0; i < EPL; ++i) { kf[i] = active ? s_knew[e0 + i] : 0.f; vf[i] = active ? s_vnew[e0 + i] : 0.f; }
+      } else {
+        unpack8(kraw[0], kf);
+        unpack8(vraw[0], vf);
+      }
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
-      d = group_sum<LPK>(d);
-      const float m_new = fmaxf(m[g], d);
-      const float keep = __expf(m[g] - m_new);  // 0 at the stream's first key
-      const float w = __expf(d - m_new);
-      l[g] = l[g] * keep + w;
+      for (int g = 0; g < GT; ++g) {
+        if (g >= gcount) break;
+        float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
-      m[g] = m_new;
+        for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
+        d = group_sum<LPK>(d);
+        const float m_new = fmaxf(m[g], d);
+        const float keep = __expf(m[g] - m_new);
+        const float w = __expf(d - m_new);
+        l[g] = l[g] * keep + w;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
+        m[g] = m_new;
+      }
+      kraw[0] = kraw[1]; vraw[0] = vraw[1];
+      kraw[1] = kraw[2]; vraw[1] = vraw[2];
     }
   }
 
-  // merge the wave's streams (lanes that differ in the bits above LPK hold different keys)
 #pragma unroll
   for (int g = 0; g < GT; ++g) {
     if (g >= gcount) break;
@@ -166,7 +322,6 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
     }
   }
   __syncthreads();
-  // merge the 4 waves; wave 0's first LPK lanes write the result
   if (wave == 0 && grp == 0) {
 #pragma unroll
     for (int g = 0; g < GT; ++g) {
@@ -245,16 +400,39 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
   }
 }
 
-template <int LPK>
-int launch_decode(int gt, dim3 grid, hipStream_t stream, const bf16* q, const bf16* k, const bf16* v, float* partial,
-                  bf16* out, const DecodeArgs& a) {
+template <int LPK, bool RAW>
+void launch_decode(int gt, dim3 grid, hipStream_t stream, const bf16* q, bf16* k, bf16* v, float* partial, bf16* out,
+                   const DecodeArgs& a) {
   switch (gt) {
-    case 1: attention_decode_kernel<LPK, 1><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 2: attention_decode_kernel<LPK, 2><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 4: attention_decode_kernel<LPK, 4><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    default: attention_decode_kernel<LPK, 8><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 1: attention_decode_kernel<LPK, 1, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 2: attention_decode_kernel<LPK, 2, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 4: attention_decode_kernel<LPK, 4, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
+    default: attention_decode_kernel<LPK, 8, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
   }
-  return 0;
+}
+
+template <bool RAW>
+int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* partial, DecodeArgs a, int n_rows,
+               hipStream_t stream) {
+  const int G = a.nh / a.nkv;
+  const int gt = G >= 8 ? 8 : (G > 2 ? 4 : G);  // 1, 2, 4 or 8 query heads per workgroup
+  a.head_chunks = ceil_div(G, gt);
+  a.page_shift = (a.page_size & (a.page_size - 1)) == 0 ? __builtin_ctz(a.page_size) : -1;
+  GIBBS_REQUIRE((long)a.nkv * a.head_chunks <= 65535, "attention_decode: too many heads");
+  dim3 grid(n_rows, a.nkv * a.head_chunks, a.n_splits);
+  const int lanes = a.hd / EPL;  // lanes that hold data; LPK is the next power of two
+  if (lanes <= 2) launch_decode<2, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 4) launch_decode<4, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 8) launch_decode<8, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 16) launch_decode<16, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else launch_decode<32, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
+  if (a.n_splits > 1) {
+    dim3 mgrid(n_rows, ceil_div(a.nh, 4));
+    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, out, a.nh, a.hd, a.n_splits, a.ldo);
+  }
+  GIBBS_LAUNCH_STATUS("attention_decode");
 }
 }  // namespace
 
@@ -277,321 +455,13 @@ GIBBS_EXPORT int gibbs_attention_decode(const void* q, const void* kpages, const
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_decode: bad cache geometry");
   GIBBS_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || partial), "attention_decode: %d key slices need a workspace", n_splits);
   if (n_rows == 0) return 0;
-  const int G = nh / nkv;
-  const int gt = G >= 8 ? 8 : (G > 2 ? 4 : G);  // 1, 2, 4 or 8 query heads per workgroup
-  const int head_chunks = ceil_div(G, gt);
-  GIBBS_REQUIRE((long)nkv * head_chunks <= 65535, "attention_decode: too many heads");
-  DecodeArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, n_splits, head_chunks};
-  dim3 grid(n_rows, nkv * head_chunks, n_splits);
-  const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
-  const int lanes = hd / EPL;  // lanes that hold data; LPK is the next power of two
-  if (lanes <= 2) launch_decode<2>(gt, grid, stream, qq, kk, vv, partial, (bf16*)out, a);
-  else if (lanes <= 4) launch_decode<4>(gt, grid, stream, qq, kk, vv, partial, (bf16*)out, a);
-  else if (lanes <= 8) launch_decode<8>(gt, grid, stream, qq, kk, vv, partial, (bf16*)out, a);
-  else if (lanes <= 16) launch_decode<16>(gt, grid, stream, qq, kk, vv, partial, (bf16*)out, a);
-  else launch_decode<32>(gt, grid, stream, qq, kk, vv, partial, (bf16*)out, a);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
-  if (n_splits > 1) {
-    dim3 mgrid(n_rows, ceil_div(nh, 4));
-    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, (bf16*)out, nh, hd, n_splits, ldo);
-  }
-  GIBBS_LAUNCH_STATUS("attention_decode");
+  DecodeArgs a{};
+  a.pos = pos; a.row_req = row_req; a.table = table; a.max_pages = max_pages; a.page_size = page_size;
+  a.num_pages = num_pages; a.nh = nh; a.nkv = nkv; a.hd = hd; a.ldq = ldq; a.ldo = ldo; a.scale = scale;
+  a.window = window; a.n_splits = n_splits;
+  // the kernel only reads the pages here
+  return run_decode<false>((const bf16*)q, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, stream);
 }
-
-// ---------------------------------------------------------------------------------------------
-// The same attention for a step of decoded tokens only, with what surrounds it fused in: the rows
-// arrive as the raw fused projection qkv[N, (nh + 2 nkv) hd]; the kernel norms and rotates q on the
-// fly (every slice's workgroup does, it is a few hundred operations), norms and rotates the row's
-// own new key, writes it and the new value to their page (the workgroup of head chunk 0 whose key
-// slice holds the row's position does) and uses them from LDS instead of reading them back.
-// The slices are merged by the separate merge kernel: letting the last workgroup to arrive merge
-// them in place needs device-scope fences, and on this chip (one L2 per XCD) each such fence
-// writes back and invalidates an L2, which cost 130 us a call when it was tried.
-namespace {
-struct FusedDecodeArgs {
-  DecodeArgs d;
-  const float* q_gain;    // [hd] or null
-  const float* k_gain;    // [hd] or null
-  float eps;
-  const float* inv_freq;  // [rot/2] or null
-  int rot, variant;       // 0 half split, 1 interleaved
-  long ld;                // row stride of qkv
-};
-
-// Rotation factors of this lane's 8 elements at position `pos` (the same for every head).
-struct Rot8 {
-  float c[EPL], s[EPL];
-};
-
-__device__ __forceinline__ Rot8 rotation8(int e0, const float* inv_freq, int rot, int variant, int pos) {
-  Rot8 r;
-  const int half = rot / 2;
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int e = e0 + i;
-    r.c[i] = 1.f;
-    r.s[i] = 0.f;
-    if (inv_freq && e < rot) {
-      const int j = variant == 1 ? e / 2 : (e < half ? e : e - half);
-      sincosf((float)pos * inv_freq[j], &r.s[i], &r.c[i]);
-    }
-  }
-  return r;
-}
-
-// Norm (optional) and rotation of one head held 8 elements per lane by LPK neighbouring lanes.
-// `v` are this lane's elements e0 .. e0+7 of the head; returns them normed and rotated.
-template <int LPK>
-__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
-                                           const Rot8& rt, int rot, int variant, int lane) {
-  const bool active = e0 < hd;
-  if (gain) {
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
-    ss = group_sum<LPK>(ss);
-    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
-  }
-  if (!rotate) return;
-  const int half = rot / 2;
-  if (variant == 1) {  // pairs (2j, 2j+1) lie in one lane
-#pragma unroll
-    for (int i = 0; i < EPL; i += 2) {
-      if (e0 + i + 1 < rot) {
-        const float x0 = v[i], x1 = v[i + 1];
-        v[i] = x0 * rt.c[i] - x1 * rt.s[i];
-        v[i + 1] = x0 * rt.s[i] + x1 * rt.c[i];
-      }
-    }
-    return;
-  }
-  // half split: element e pairs with e + half (e < half) or e - half; the partner lies half/8 lanes away
-  const int shift = half / EPL;  // half is a multiple of 8 (rotary sizes in steps of 16)
-  const int base = lane - lane % LPK;
-  const int sub = lane % LPK;
-  const bool low = e0 < half;
-  const int partner = base + (low ? sub + shift : sub - shift);
-  const int src = (partner >= base && partner < base + LPK) ? partner : lane;
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const float other = __shfl(v[i], src, WAVE);
-    if (e0 + i < rot) v[i] = low ? v[i] * rt.c[i] - other * rt.s[i] : other * rt.s[i] + v[i] * rt.c[i];
-  }
-}
-
-template <int LPK, int GT>
-__global__ __launch_bounds__(256) void attention_decode_fused_kernel(const bf16* __restrict__ qkv,
-                                                                     bf16* __restrict__ kpages, bf16* __restrict__ vpages,
-                                                                     float* __restrict__ partial, bf16* __restrict__ out,
-                                                                     FusedDecodeArgs fa) {
-  constexpr int KPW = WAVE / LPK;
-  constexpr int MAX_HD = LPK * EPL;
-  __shared__ float s_ml[4][GT][2];
-  __shared__ float s_acc[4][GT][MAX_HD];
-  __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
-  __shared__ int s_pages[SEG_PAGES];
-  const DecodeArgs& a = fa.d;
-
-  const int row = blockIdx.x;
-  const int kvh = blockIdx.y / a.head_chunks, hc = blockIdx.y % a.head_chunks;
-  const int split = blockIdx.z;
-  const int G = a.nh / a.nkv;
-  const int g0 = hc * GT;
-  const int gcount = min(GT, G - g0);
-  const int hd = a.hd;
-  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
-  const int grp = lane / LPK, sub = lane % LPK;
-  const int e0 = sub * EPL;
-  const bool active = e0 < hd;
-
-  const int p = a.pos[row];
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-  const int len = p + 1 - lo;
-  int per = (len + a.n_splits - 1) / a.n_splits;
-  per = (per + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
-  const int k0 = lo + split * per;
-  const int k1 = min(k0 + per, p + 1);
-  const int* table = a.table + (size_t)a.row_req[row] * a.max_pages;
-  const bf16* qrow = qkv + (size_t)row * fa.ld;
-
-  const Rot8 rt = rotation8(e0, fa.inv_freq, fa.rot, fa.variant, p);
-  const bool rotate = fa.inv_freq != nullptr;
-  // the row's own key and value: wave 0's first LPK lanes prepare them for everyone
-  const bool has_new = p >= k0 && p < k1;
-  if (has_new && wave == 0 && grp == 0) {
-    float kf[EPL], vf[EPL];
-    if (active) {
-      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0), kf);
-      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0), vf);
-    } else {
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
-    }
-    norm_rope8<LPK>(kf, e0, hd, fa.k_gain, fa.eps, rotate, rt, fa.rot, fa.variant, lane);
-    if (active) {
-      // what later steps read from the page is the bfloat16 value: use the same value now
-      uint32_t kw[4], vw[4];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) {
-        const bf16 kb = (bf16)kf[i];
-        kf[i] = (float)kb;
-        s_knew[e0 + i] = kf[i];
-        s_vnew[e0 + i] = vf[i];
-        const uint32_t kbits = __float_as_uint(kf[i]) >> 16, vbits = __float_as_uint(vf[i]) >> 16;
-        if (i % 2 == 0) { kw[i / 2] = kbits; vw[i / 2] = vbits; }
-        else { kw[i / 2] |= kbits << 16; vw[i / 2] |= vbits << 16; }
-      }
-      if (hc == 0) {
-        const int page = table[p / a.page_size];
-        if (page >= 0 && page < a.num_pages) {
-          const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + p % a.page_size) * hd + e0;
-          *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
-          *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-        }
-      }
-    }
-  }
-
-  float qf[GT][EPL];
-  float m[GT], l[GT], acc[GT][EPL];
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    m[g] = -INFINITY;
-    l[g] = 0.f;
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) { acc[g][i] = 0.f; qf[g][i] = 0.f; }
-    if (g < gcount) {
-      if (active) unpack8(*(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0), qf[g]);
-      norm_rope8<LPK>(qf[g], e0, hd, fa.q_gain, fa.eps, rotate, rt, fa.rot, fa.variant, lane);
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) qf[g][i] = (float)(bf16)qf[g][i] * a.scale;   // q is bfloat16 where it is stored
-    }
-  }
-  __syncthreads();  // s_knew, s_vnew
-
-  // The slice's page ids go to LDS first (one round trip for all of them, instead of a dependent
-  // table load in front of every key's loads); the loads of the next two keys are issued before the
-  // current key is worked on, so that memory latency overlaps the arithmetic.
-  for (int seg0 = k0; seg0 < k1; seg0 += SEG_PAGES * a.page_size) {
-    const int first_page = seg0 / a.page_size;
-    const int seg1 = min(k1, (first_page + SEG_PAGES) * a.page_size);
-    __syncthreads();  // the previous segment's ids are no longer read
-    for (int j = threadIdx.x; j < SEG_PAGES && (first_page + j) * a.page_size < seg1; j += 256) {
-      int page = table[first_page + j];
-      s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
-    }
-    __syncthreads();
-    auto fetch = [&](int key, uint4& kr, uint4& vr) {
-      kr = vr = make_uint4(0, 0, 0, 0);
-      if (key < seg1 && key != p && active) {
-        const int lp = key / a.page_size;
-        const size_t off = (((size_t)s_pages[lp - first_page] * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
-        kr = *(const uint4*)(kpages + off);
-        vr = *(const uint4*)(vpages + off);
-      }
-    };
-    uint4 kraw[3], vraw[3];
-    // the wave's first key of this segment keeps the global stride pattern k0 + (4 it + wave) KPW + grp
-    int key = k0 + wave * KPW + grp;
-    if (key < seg0) key += (seg0 - key + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
-    fetch(key, kraw[0], vraw[0]);
-    fetch(key + 4 * KPW, kraw[1], vraw[1]);
-    for (; key < seg1; key += 4 * KPW) {
-      fetch(key + 8 * KPW, kraw[2], vraw[2]);
-      __builtin_amdgcn_sched_barrier(0);  // the loads above stay ahead of the arithmetic below
-      float kf[EPL], vf[EPL];
-      if (key == p) {
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) { kf[i] = active ? s_knew[e0 + i] : 0.f; vf[i] = active ? s_vnew[e0 + i] : 0.f; }
-      } else {
-        unpack8(kraw[0], kf);
-        unpack8(vraw[0], vf);
-      }
-#pragma unroll
-      for (int g = 0; g < GT; ++g) {
-        if (g >= gcount) break;
-        float d = 0.f;
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) d = fmaf(qf[g][i], kf[i], d);
-        d = group_sum<LPK>(d);
-        const float m_new = fmaxf(m[g], d);
-        const float keep = __expf(m[g] - m_new);
-        const float w = __expf(d - m_new);
-        l[g] = l[g] * keep + w;
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) acc[g][i] = fmaf(w, vf[i], acc[g][i] * keep);
-        m[g] = m_new;
-      }
-      kraw[0] = kraw[1]; vraw[0] = vraw[1];
-      kraw[1] = kraw[2]; vraw[1] = vraw[2];
-    }
-  }
-
-#pragma unroll
-  for (int g = 0; g < GT; ++g) {
-    if (g >= gcount) break;
-#pragma unroll
-    for (int o = LPK; o < WAVE; o <<= 1) {
-      const float mb = __shfl_xor(m[g], o, WAVE), lb = __shfl_xor(l[g], o, WAVE);
-      float ab[EPL];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) ab[i] = __shfl_xor(acc[g][i], o, WAVE);
-      fold<EPL>(m[g], l[g], acc[g], mb, lb, ab);
-    }
-    if (grp == 0) {
-      if (sub == 0) { s_ml[wave][g][0] = m[g]; s_ml[wave][g][1] = l[g]; }
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) s_acc[wave][g][e0 + i] = acc[g][i];
-    }
-  }
-  __syncthreads();
-  if (wave == 0 && grp == 0) {
-#pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      if (g >= gcount) break;
-      float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
-      for (int w = 1; w < 4; ++w) {
-        float ab[EPL];
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
-        fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
-      }
-      const int head = kvh * G + g0 + g;
-      if (a.n_splits == 1) {
-        if (active) {
-          const float inv = 1.0f / ll;
-          bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
-#pragma unroll
-          for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
-        }
-      } else {
-        float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
-        if (sub == 0) { ps[0] = mm; ps[1] = ll; }
-        if (active) {
-#pragma unroll
-          for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
-        }
-      }
-    }
-  }
-}
-
-template <int LPK>
-void launch_decode_fused(int gt, dim3 grid, hipStream_t stream, const bf16* qkv, bf16* k, bf16* v, float* partial,
-                         bf16* out, const FusedDecodeArgs& a) {
-  switch (gt) {
-    case 1: attention_decode_fused_kernel<LPK, 1><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
-    case 2: attention_decode_fused_kernel<LPK, 2><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
-    case 4: attention_decode_fused_kernel<LPK, 4><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
-    default: attention_decode_fused_kernel<LPK, 8><<<grid, 256, 0, stream>>>(qkv, k, v, partial, out, a); break;
-  }
-}
-}  // namespace
 
 // qkv: [N, ld] bfloat16, raw projection (q heads, k heads, v heads) of N decoded tokens, one per request.
 GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, void* vpages, void* out, float* partial,
@@ -610,28 +480,10 @@ GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, voi
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_decode_fused: bad cache geometry");
   GIBBS_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || partial), "attention_decode_fused: %d key slices need a workspace", n_splits);
   if (n_rows == 0) return 0;
-  const int G = nh / nkv;
-  const int gt = G >= 8 ? 8 : (G > 2 ? 4 : G);
-  const int head_chunks = ceil_div(G, gt);
-  GIBBS_REQUIRE((long)nkv * head_chunks <= 65535, "attention_decode_fused: too many heads");
-  FusedDecodeArgs fa{};
-  fa.d = DecodeArgs{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ld, ldo, scale, window, n_splits, head_chunks};
-  fa.q_gain = q_gain; fa.k_gain = k_gain; fa.eps = eps; fa.inv_freq = inv_freq; fa.rot = rot; fa.variant = variant;
-  fa.ld = ld;
-  dim3 grid(n_rows, nkv * head_chunks, n_splits);
-  const bf16* qq = (const bf16*)qkv;
-  bf16 *kk = (bf16*)kpages, *vv = (bf16*)vpages, *oo = (bf16*)out;
-  const int lanes = hd / EPL;
-  if (lanes <= 2) launch_decode_fused<2>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
-  else if (lanes <= 4) launch_decode_fused<4>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
-  else if (lanes <= 8) launch_decode_fused<8>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
-  else if (lanes <= 16) launch_decode_fused<16>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
-  else launch_decode_fused<32>(gt, grid, stream, qq, kk, vv, partial, oo, fa);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return gibbs_fail("attention_decode_fused: %s", hipGetErrorString(e));
-  if (n_splits > 1) {
-    dim3 mgrid(n_rows, ceil_div(nh, 4));
-    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, oo, nh, hd, n_splits, ldo);
-  }
-  GIBBS_LAUNCH_STATUS("attention_decode_fused");
+  DecodeArgs a{};
+  a.pos = pos; a.row_req = row_req; a.table = table; a.max_pages = max_pages; a.page_size = page_size;
+  a.num_pages = num_pages; a.nh = nh; a.nkv = nkv; a.hd = hd; a.ldq = ld; a.ldo = ldo; a.scale = scale;
+  a.window = window; a.n_splits = n_splits;
+  a.q_gain = q_gain; a.k_gain = k_gain; a.eps = eps; a.inv_freq = inv_freq; a.rot = rot; a.variant = variant;
+  return run_decode<true>((const bf16*)qkv, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, stream);
 }
