@@ -26,9 +26,9 @@
 // Visibility is by position only: row n sees keys lo .. pos[n] of its request
 // (lo = max(0, pos - window + 1), window 0 = all).
 #include "common.h"
+#include "lane8.h"
 
 namespace {
-constexpr int EPL = 8;  // head-dim elements per lane (16 bytes of bfloat16)
 constexpr int SEG_PAGES = 512;  // page ids of a key slice kept in LDS at a time
 
 struct DecodeArgs {
@@ -49,34 +49,9 @@ struct DecodeArgs {
   float eps;
   const float* inv_freq;  // [rot/2] or null
   int rot, variant;       // 0 half split, 1 interleaved
+  const float2* cs_table; // [table_len, rot/2] (cos, sin) of the first positions, or null
+  int table_len;
 };
-
-__device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
-  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f[2 * i] = __uint_as_float(w[i] << 16);
-    f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
-  }
-}
-
-// Sum over the LPK neighbouring lanes that share a key, every one of them getting the total.
-// Data-parallel-primitive moves (a few cycles each) instead of LDS permutes (tens of cycles each,
-// and this sum sits on the critical path of every key): swap within pairs, within quads, then
-// mirror the half row (lane i <-> 7 - i: the other quad) and the row (i <-> 15 - i: the other half).
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
-}
-template <int LPK>
-__device__ __forceinline__ float group_sum(float v) {
-  if (LPK >= 2) v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
-  if (LPK >= 4) v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
-  if (LPK >= 8) v += dpp_move<0x141>(v);  // row_half_mirror
-  if (LPK >= 16) v += dpp_move<0x140>(v); // row_mirror
-  if (LPK >= 32) v += __shfl_xor(v, 16, WAVE);
-  return v;
-}
 
 // Folds stream b (mb, lb, ab) into stream a.
 template <int N>
@@ -88,69 +63,6 @@ __device__ __forceinline__ void fold(float& ma, float& la, float* aa, float mb, 
 #pragma unroll
   for (int i = 0; i < N; ++i) aa[i] = aa[i] * sa + ab[i] * sb;
   ma = m;
-}
-
-// Rotation factors of this lane's 8 elements at position `pos` (the same for every head).
-struct Rot8 {
-  float c[EPL], s[EPL];
-};
-
-__device__ __forceinline__ Rot8 rotation8(int e0, const float* inv_freq, int rot, int variant, int pos) {
-  Rot8 r;
-  const int half = rot / 2;
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const int e = e0 + i;
-    r.c[i] = 1.f;
-    r.s[i] = 0.f;
-    if (inv_freq && e < rot) {
-      const int j = variant == 1 ? e / 2 : (e < half ? e : e - half);
-      sincosf((float)pos * inv_freq[j], &r.s[i], &r.c[i]);
-    }
-  }
-  return r;
-}
-
-// Norm (optional) and rotation of one head held 8 elements per lane by LPK neighbouring lanes.
-// `v` are this lane's elements e0 .. e0+7 of the head; returns them normed and rotated.
-template <int LPK>
-__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
-                                           const Rot8& rt, int rot, int variant, int lane) {
-  const bool active = e0 < hd;
-  if (gain) {
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
-    ss = group_sum<LPK>(ss);
-    const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
-  }
-  if (!rotate) return;
-  const int half = rot / 2;
-  if (variant == 1) {  // pairs (2j, 2j+1) lie in one lane
-#pragma unroll
-    for (int i = 0; i < EPL; i += 2) {
-      if (e0 + i + 1 < rot) {
-        const float x0 = v[i], x1 = v[i + 1];
-        v[i] = x0 * rt.c[i] - x1 * rt.s[i];
-        v[i + 1] = x0 * rt.s[i] + x1 * rt.c[i];
-      }
-    }
-    return;
-  }
-  // half split: element e pairs with e + half (e < half) or e - half; the partner lies half/8 lanes away
-  const int shift = half / EPL;  // half is a multiple of 8 (rotary sizes in steps of 16)
-  const int base = lane - lane % LPK;
-  const int sub = lane % LPK;
-  const bool low = e0 < half;
-  const int partner = base + (low ? sub + shift : sub - shift);
-  const int src = (partner >= base && partner < base + LPK) ? partner : lane;
-#pragma unroll
-  for (int i = 0; i < EPL; ++i) {
-    const float other = __shfl(v[i], src, WAVE);
-    if (e0 + i < rot) v[i] = low ? v[i] * rt.c[i] - other * rt.s[i] : other * rt.s[i] + v[i] * rt.c[i];
-  }
 }
 
 template <int LPK, int GT, bool RAW>
@@ -187,7 +99,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
   const bf16* qrow = qkv + (size_t)row * a.ldq;
 
   Rot8 rt;
-  if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p);
+  if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p, a.cs_table, a.table_len);
   const bool rotate = a.inv_freq != nullptr;
   // raw rows: the row's own key and value; wave 0's first LPK lanes prepare them for everyone
   const bool has_new = RAW && p >= k0 && p < k1;
@@ -466,8 +378,8 @@ GIBBS_EXPORT int gibbs_attention_decode(const void* q, const void* kpages, const
 // qkv: [N, ld] bfloat16, raw projection (q heads, k heads, v heads) of N decoded tokens, one per request.
 GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, void* vpages, void* out, float* partial,
                                               const float* q_gain, const float* k_gain, float eps,
-                                              const float* inv_freq, int rot, int variant, const int* pos,
-                                              const int* row_req, const int* table, int max_pages, int page_size,
+                                              const float* inv_freq, int rot, int variant, const float* cs_table,
+                                              int table_len, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
                                               int num_pages, int n_rows, int nh, int nkv, int hd, long ld, long ldo,
                                               float scale, int window, int n_splits, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_decode_fused: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
@@ -485,5 +397,6 @@ GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, voi
   a.num_pages = num_pages; a.nh = nh; a.nkv = nkv; a.hd = hd; a.ldq = ld; a.ldo = ldo; a.scale = scale;
   a.window = window; a.n_splits = n_splits;
   a.q_gain = q_gain; a.k_gain = k_gain; a.eps = eps; a.inv_freq = inv_freq; a.rot = rot; a.variant = variant;
+  a.cs_table = (const float2*)cs_table; a.table_len = cs_table ? table_len : 0;
   return run_decode<true>((const bf16*)qkv, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, stream);
 }

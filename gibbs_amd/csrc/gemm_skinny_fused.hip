@@ -52,9 +52,11 @@ struct FusedArgs {
   int K;
 };
 
-template <int NT, int RG, int ROWS, int WAVES, bool RMS, int EPI>
+// KC: the convolution's kernel length when it is 2..4 (its operands are then asked for before the
+// product), 0 for any other length or epilogue.
+template <int NT, int RG, int ROWS, int WAVES, bool RMS, int EPI, int KC>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
-  __shared__ floatx4 red[WAVES / 2][RG][NT][WAVE];
+  __shared__ floatx4 red[WAVES - 1][RG][NT][WAVE];
   __shared__ float red_ss[WAVES][NT][16];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
@@ -76,6 +78,45 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     x_ok[t] = t * 16 + r < a.N;
     xrow[t] = a.X + (size_t)(x_ok[t] ? t * 16 + r : 0) * a.ldx + g * 8;
   }
+  // What the epilogue reads besides the product is asked for now: the product hides the latency
+  // (the state row hangs on a slot index, two dependent loads).  Wave 0 writes the outputs; its lane
+  // holds features o_epi .. +3 of row t*16 + r.
+  constexpr int KH = KC > 1 ? KC - 1 : 1;
+  const int o_epi = o0 + g * 4;
+  const bool epi_lane = wave == 0 && g * 4 < ROWS && o_epi < a.O;
+  float pre_x[NT][4];          // RESIDUAL: the stream; CONV: unused
+  float pre_hist[NT][KH][4];   // CONV: the state rows
+  float pre_taps[KC > 1 ? KC : 1][4], pre_bias[4];
+  if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pre_x[t][i] = (epi_lane && n < a.N && o_epi + i < a.O) ? a.x[(size_t)n * a.O + o_epi + i] : 0.f;
+    }
+  }
+  if (EPI == EPI_CONV && KC > 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = epi_lane && o_epi + i < a.O;
+#pragma unroll
+      for (int j = 0; j < KC; ++j) pre_taps[j][i] = ok ? a.taps[(size_t)(o_epi + i) * KC + j] : 0.f;
+      pre_bias[i] = (ok && a.bias) ? a.bias[o_epi + i] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + r;
+      const bool row = epi_lane && n < a.N;
+      const float* st = a.state + (size_t)(row ? a.slot[n] : 0) * a.slot_stride;
+      const int before = row ? a.ctx[n] : 0;
+#pragma unroll
+      for (int j = 0; j < KH; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          pre_hist[t][j][i] = (row && o_epi + i < a.O && before - (KC - 1) + j >= 0) ? st[(size_t)j * a.O + o_epi + i] : 0.f;
+    }
+  }
+
   floatx4 acc[RG][NT];
   float ss[NT];
 #pragma unroll
@@ -124,25 +165,21 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       if (g == 0) red_ss[wave][t][r] = ss[t];
     }
   }
-  // the waves' partial products meet in a tree (fixed order of additions)
+  // the waves' partial products meet in wave 0, added in the order of the waves
+  if (wave != 0) {
 #pragma unroll
-  for (int stride = WAVES / 2; stride >= 1; stride /= 2) {
-    if (wave >= stride && wave < 2 * stride) {
+    for (int q = 0; q < RG; ++q)
 #pragma unroll
-      for (int q = 0; q < RG; ++q)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) red[wave - stride][q][t][lane] = acc[q][t];
-    }
-    __syncthreads();
-    if (wave < stride) {
-#pragma unroll
-      for (int q = 0; q < RG; ++q)
-#pragma unroll
-        for (int t = 0; t < NT; ++t) acc[q][t] += red[wave][q][t][lane];
-    }
-    __syncthreads();
+      for (int t = 0; t < NT; ++t) red[wave - 1][q][t][lane] = acc[q][t];
   }
+  __syncthreads();
   if (wave != 0) return;
+#pragma unroll(RG * NT <= 2 ? WAVES : 1)
+  for (int w = 1; w < WAVES; ++w)
+#pragma unroll
+    for (int q = 0; q < RG; ++q)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) acc[q][t] += red[w - 1][q][t][lane];
 
   // D[feature g*4 + i][row r] of tile t: lane holds 4 consecutive features of one row
 #pragma unroll
@@ -169,8 +206,10 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     } else if (EPI == EPI_RESIDUAL) {
       float* xp = a.x + (size_t)n * a.O + o;
       bf16* bp = a.xb + (size_t)n * a.O + o;
-      for (int i = 0; i < 4 && o + i < a.O; ++i) {
-        const float v = xp[i] + acc[0][t][i] * scale;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (o + i >= a.O) break;
+        const float v = pre_x[t][i] + acc[0][t][i] * scale;
         xp[i] = v;
         bp[i] = (bf16)v;
       }
@@ -180,7 +219,26 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
         const float gt = acc[0][t][i] * scale, up = acc[RG > 1 ? 1 : 0][t][i] * scale;
         y[i] = (bf16)(gt * (1.0f / (1.0f + expf(-gt))) * up);
       }
-    } else {  // EPI_CONV
+    } else if (KC > 1) {  // EPI_CONV, operands at hand
+      float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
+      bf16* y = a.Y + (size_t)n * a.ldy + o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (o + i >= a.O) break;
+        const int c = o + i;
+        const float bx = (acc[0][t][i] * scale) * (acc[RG > 2 ? 2 : 0][t][i] * scale);
+        const float cg = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        float cv = 0.f;
+#pragma unroll
+        for (int j = 0; j < KC - 1; ++j) cv = fmaf(pre_taps[j][i], pre_hist[t][j][i], cv);
+        cv = fmaf(pre_taps[KC - 1][i], bx, cv);
+        if (a.bias) cv += pre_bias[i];
+        y[i] = (bf16)(cg * cv);
+#pragma unroll
+        for (int j = 0; j + 1 < KC - 1; ++j) st[(size_t)j * a.O + c] = pre_hist[t][j + 1][i];
+        st[(size_t)(KC - 2) * a.O + c] = bx;
+      }
+    } else {  // EPI_CONV, any kernel length
       const int K = a.K;
       float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
       const int before = a.ctx[n];
@@ -212,24 +270,34 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 }
 
-template <int NT, int RG, bool RMS, int EPI>
+template <int NT, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
   // few features: halve the rows per workgroup so that every compute unit gets one
   static const int rows8_below = getenv("GIBBS_SKINNY_ROWS8_BELOW") ? atoi(getenv("GIBBS_SKINNY_ROWS8_BELOW")) : 256;
   if (a.O / 16 < rows8_below) {
-    gemm_skinny_fused_kernel<NT, RG, 8, 8, RMS, EPI><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 8, 8, RMS, EPI, KC><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
   } else {
-    gemm_skinny_fused_kernel<NT, RG, 16, 8, RMS, EPI><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 16, 8, RMS, EPI, KC><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
   }
 }
 
-template <int RG, bool RMS, int EPI>
+template <int RG, bool RMS, int EPI, int KC = 0>
 void launch_nt(const FusedArgs& a, hipStream_t s) {
   const int nt = ceil_div(a.N, 16);
-  if (nt == 1) launch_rows<1, RG, RMS, EPI>(a, s);
-  else if (nt == 2) launch_rows<2, RG, RMS, EPI>(a, s);
-  else if (nt == 3) launch_rows<3, RG, RMS, EPI>(a, s);
-  else launch_rows<4, RG, RMS, EPI>(a, s);
+  if (nt == 1) launch_rows<1, RG, RMS, EPI, KC>(a, s);
+  else if (nt == 2) launch_rows<2, RG, RMS, EPI, KC>(a, s);
+  else if (nt == 3) launch_rows<3, RG, RMS, EPI, KC>(a, s);
+  else launch_rows<4, RG, RMS, EPI, KC>(a, s);
+}
+
+template <bool RMS>
+void launch_conv(const FusedArgs& a, hipStream_t s) {
+  switch (a.K) {
+    case 2: launch_nt<3, RMS, EPI_CONV, 2>(a, s); break;
+    case 3: launch_nt<3, RMS, EPI_CONV, 3>(a, s); break;
+    case 4: launch_nt<3, RMS, EPI_CONV, 4>(a, s); break;
+    default: launch_nt<3, RMS, EPI_CONV, 0>(a, s); break;
+  }
 }
 
 int check_common(const char* what, const void* X, const void* W, int N, int O, int I, long ldx, long ldw) {
@@ -290,7 +358,7 @@ GIBBS_EXPORT int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N,
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = C; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
   a.group_stride = C; a.Y = (bf16*)Y; a.ldy = C;
   a.taps = taps; a.bias = bias; a.state = state; a.slot_stride = slot_stride; a.slot = slot; a.ctx = ctx; a.K = K;
-  if (rms) launch_nt<3, true, EPI_CONV>(a, stream);
-  else launch_nt<3, false, EPI_CONV>(a, stream);
+  if (rms) launch_conv<true>(a, stream);
+  else launch_conv<false>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_conv");
 }

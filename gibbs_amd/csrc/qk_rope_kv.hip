@@ -7,8 +7,17 @@
 // The norm comes before the rotation.  Rotation of pair (i0, i1) by angle = float(pos) * inv_freq[j]
 // (a float32 product): half-split pairs (j, j + rot/2), interleaved pairs (2j, 2j+1); elements
 // beyond rotary_dim pass through.  Sums, the root, angles, sine and cosine are float32.
-// One wave per (row, head).  Pages are laid out [page, kv head, slot in page, hd].
+// Pages are laid out [page, kv head, slot in page, hd].
+//
+// Cosines and sines come from a table [positions, rot/2] of (cos, sin) that `rope_table` fills once
+// (accurate sinf/cosf cost more than everything else here together); positions beyond the table
+// are computed in place with the same functions.
+//
+// Two kernels: the general one (any element type, any even rotary size; one wave per (row, head),
+// element by element), and the bfloat16 one for head and rotary sizes in steps of 16 (a lane
+// holds 8 elements, 16-byte loads and stores, several heads per wave).
 #include "common.h"
+#include "lane8.h"
 
 namespace {
 enum { ROPE_HALF_SPLIT = 0, ROPE_INTERLEAVED = 1 };
@@ -19,6 +28,8 @@ struct QkRopeArgs {
   float eps;
   const float* inv_freq;  // [rot / 2] or null: no rotation
   int rot, variant;
+  const float2* cs_table;  // [table_len, rot / 2] or null
+  int table_len;
   const int* pos;      // [N] absolute position of each row
   const int* row_req;  // [N] batch index of each row's request
   const int* table;    // [n_req, max_pages] page ids of the layer's cache group
@@ -74,18 +85,84 @@ __global__ __launch_bounds__(256) void qk_rope_kv_kernel(T* __restrict__ qkv, T*
     const int i0 = a.variant == ROPE_HALF_SPLIT ? j : 2 * j;
     const int i1 = a.variant == ROPE_HALF_SPLIT ? j + half : 2 * j + 1;
     const float x0 = normed(i0), x1 = normed(i1);
-    const float angle = (float)p * a.inv_freq[j];
-    const float c = cosf(angle), s = sinf(angle);
+    float c, s;
+    if (a.cs_table && p < a.table_len) {
+      const float2 cs = a.cs_table[(size_t)p * half + j];
+      c = cs.x;
+      s = cs.y;
+    } else {
+      rope_cos_sin((float)p * a.inv_freq[j], &c, &s);
+    }
     dst[i0] = from_float<T>(x0 * c - x1 * s);
     dst[i1] = from_float<T>(x0 * s + x1 * c);
   }
   for (int e = 2 * half + lane; e < hd; e += WAVE) dst[e] = from_float<T>(normed(e));
 }
+
+// bfloat16, hd and rot multiples of 16: LPK lanes per (row, head), 64 / LPK heads per wave.
+template <int LPK>
+__global__ __launch_bounds__(256) void qk_rope_kv_bf16x8_kernel(bf16* __restrict__ qkv, bf16* __restrict__ kpages,
+                                                                bf16* __restrict__ vpages, QkRopeArgs a, int n_rows) {
+  constexpr int HPW = WAVE / LPK;  // heads per wave
+  const int slots = a.nh + 2 * a.nkv;
+  const int lane = threadIdx.x % WAVE;
+  const int sub = lane % LPK, e0 = sub * EPL;
+  const long item = ((long)blockIdx.x * (blockDim.x / WAVE) + threadIdx.x / WAVE) * HPW + lane / LPK;
+  const bool item_ok = item < (long)n_rows * slots;
+  const int n = item_ok ? (int)(item / slots) : 0;
+  const int hs = item_ok ? (int)(item % slots) : 0;
+  const int hd = a.hd;
+  const bool active = item_ok && e0 < hd;
+  const bool is_q = hs < a.nh, is_k = !is_q && hs < a.nh + a.nkv;
+  const int p = a.pos[n];
+  bf16* src = qkv + (size_t)n * a.ld + (size_t)hs * hd + e0;
+  bf16* dst = src;
+  bool write = active;
+  if (!is_q) {
+    write = false;
+    if (kpages && active) {
+      const int page = a.table[(size_t)a.row_req[n] * a.max_pages + p / a.page_size];
+      if (page >= 0 && page < a.num_pages) {  // the host never asks for another; never write outside
+        const int g = is_k ? hs - a.nh : hs - a.nh - a.nkv;
+        dst = (is_k ? kpages : vpages) + (((size_t)page * a.nkv + g) * a.page_size + p % a.page_size) * hd + e0;
+        write = true;
+      }
+    }
+  }
+  const uint4 raw = active ? *(const uint4*)src : make_uint4(0, 0, 0, 0);
+  if (!is_q && !is_k) {
+    if (write) *(uint4*)dst = raw;
+    return;  // whole lane groups leave: the sums below stay within a group
+  }
+  float v[EPL];
+  unpack8(raw, v);
+  const Rot8 rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p, a.cs_table, a.table_len);
+  norm_rope8<LPK>(v, e0, hd, is_q ? a.q_gain : a.k_gain, a.eps, a.inv_freq != nullptr, rt, a.rot, a.variant, lane);
+  if (write) *(uint4*)dst = pack8(v);
+}
+
+// (cos, sin) of float(pos) * inv_freq[j] for pos < n_pos, j < half.
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* __restrict__ table, const float* __restrict__ inv_freq,
+                                                         int half, long total) {
+  const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int pos = (int)(i / half), j = (int)(i % half);
+  float c, s;
+  rope_cos_sin((float)pos * inv_freq[j], &c, &s);
+  table[i] = make_float2(c, s);
+}
 }  // namespace
+
+GIBBS_EXPORT int gibbs_rope_table(float* table, const float* inv_freq, int half, int n_pos, hipStream_t stream) {
+  GIBBS_REQUIRE(half > 0 && n_pos > 0, "rope_table: bad sizes half=%d positions=%d", half, n_pos);
+  const long total = (long)half * n_pos;
+  rope_table_kernel<<<ceil_div(total, 256), 256, 0, stream>>>((float2*)table, inv_freq, half, total);
+  GIBBS_LAUNCH_STATUS("rope_table");
+}
 
 GIBBS_EXPORT int gibbs_qk_rope_kv(void* qkv, void* kpages, void* vpages, int dtype, const float* q_gain,
                                   const float* k_gain, float eps, const float* inv_freq, int rot, int variant,
-                                  const int* pos, const int* row_req, const int* table, int max_pages,
+                                  const float* cs_table, int table_len, const int* pos, const int* row_req, const int* table, int max_pages,
                                   int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ld,
                                   hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv >= 0 && hd > 0, "qk_rope_kv: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
@@ -94,11 +171,25 @@ GIBBS_EXPORT int gibbs_qk_rope_kv(void* qkv, void* kpages, void* vpages, int dty
   GIBBS_REQUIRE(variant == ROPE_HALF_SPLIT || variant == ROPE_INTERLEAVED, "qk_rope_kv: unknown rotation variant %d", variant);
   GIBBS_REQUIRE(!kpages || (vpages && table && page_size > 0 && max_pages > 0 && num_pages > 0), "qk_rope_kv: cache pages without a block table");
   if (n_rows == 0) return 0;
-  QkRopeArgs a{q_gain, k_gain, eps, inv_freq, rot, variant, pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ld};
+  QkRopeArgs a{q_gain, k_gain, eps, inv_freq, rot, variant, (const float2*)cs_table, cs_table ? table_len : 0, pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ld};
   const int slots = nh + 2 * nkv;
   dim3 grid(n_rows, ceil_div(slots, 4));
   GIBBS_REQUIRE(grid.y <= 65535, "qk_rope_kv: too many heads (%d)", slots);
-  if (dtype == GIBBS_F32)
+  const bool lanes8 = dtype == GIBBS_BF16 && hd % 16 == 0 && hd <= 256 && (!inv_freq || rot % 16 == 0) && ld % 8 == 0 &&
+                      ((uintptr_t)qkv % 16) == 0;
+  if (lanes8) {
+    const int lanes = hd / EPL;
+    const long items = (long)n_rows * slots;
+#define GIBBS_ROPE8(LPK)                                                                                   \
+  qk_rope_kv_bf16x8_kernel<LPK><<<ceil_div(items, 4 * (WAVE / LPK)), 256, 0, stream>>>((bf16*)qkv, (bf16*)kpages, \
+                                                                                        (bf16*)vpages, a, n_rows)
+    if (lanes <= 2) GIBBS_ROPE8(2);
+    else if (lanes <= 4) GIBBS_ROPE8(4);
+    else if (lanes <= 8) GIBBS_ROPE8(8);
+    else if (lanes <= 16) GIBBS_ROPE8(16);
+    else GIBBS_ROPE8(32);
+#undef GIBBS_ROPE8
+  } else if (dtype == GIBBS_F32)
     qk_rope_kv_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, (float*)kpages, (float*)vpages, a);
   else if (dtype == GIBBS_BF16)
     qk_rope_kv_kernel<bf16><<<grid, 256, 0, stream>>>((bf16*)qkv, (bf16*)kpages, (bf16*)vpages, a);

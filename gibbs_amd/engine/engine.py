@@ -60,14 +60,14 @@ class Engine:
         self.model = DecoderModel(self.spec)
         if weights is None:
             weights = load_weights(model_dir, self.model.tensor_decls(), self.dtype, self.device)
-        self.rt = Runtime(self.device, self.dtype)
+        self.page_size = page_size
+        self.ctx_limit = int(ctx) if ctx else self.spec.max_position
+        num_pages = max(1, -(-max_tokens // page_size))
+        self.rt = Runtime(self.device, self.dtype, max_positions=min(self.ctx_limit, num_pages * page_size))
         self.model.bind(weights, self.rt)
         self.weight_bytes = weights.nbytes()
         del weights
 
-        self.page_size = page_size
-        self.ctx_limit = int(ctx) if ctx else self.spec.max_position
-        num_pages = max(1, -(-max_tokens // page_size))
         self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), page_size, num_pages,
                                   max_requests)
         self.device_cache = DeviceCache(self.cache, self.dtype, self.device)

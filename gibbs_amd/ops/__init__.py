@@ -247,11 +247,12 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
                            k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
                            rotary_dim: int, variant: str, window: Optional[int] = None,
                            max_seq: int = 0, n_splits: Optional[int] = None,
-                           out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Decode attention straight from the raw fused projection qkv[N, (nh + 2 nkv) hd] of N decoded
     tokens: q/k norm and rotation, the write of the new key and value to their pages, attention over
-    split keys in one kernel (followed by the merge of the slices)."""
-    require_cuda(qkv, kpages, vpages, table, pos, row_req, q_gain, k_gain, inv_freq)
+    split keys in one kernel (followed by the merge of the slices).  `cos_sin` as in `qk_rope_kv`."""
+    require_cuda(qkv, kpages, vpages, table, pos, row_req, q_gain, k_gain, inv_freq, cos_sin)
+    table_len = _check_cos_sin(cos_sin, inv_freq, rotary_dim)
     if qkv.dtype != torch.bfloat16:
         raise KernelError("attention_decode_fused is a bfloat16 kernel")
     if hd % 16 or hd > 256:
@@ -276,8 +277,8 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
         out = torch.empty((n_rows, nh * hd), dtype=qkv.dtype, device=qkv.device)
     assert out.shape == (n_rows, nh * hd) and out.dtype == qkv.dtype and out.is_contiguous()
     call("gibbs_attention_decode_fused", ptr(qkv), ptr(kpages), ptr(vpages), ptr(out), ptr(partial),
-         ptr(q_gain), ptr(k_gain), float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(pos),
-         ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
+         ptr(q_gain), ptr(k_gain), float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(cos_sin),
+         table_len, ptr(pos), ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
          qkv.stride(0) if n_rows > 1 else qkv.shape[1], nh * hd, float(scale), int(window or 0), n_splits, stream())
     return out
 
@@ -327,11 +328,14 @@ def _check_pages(pages: torch.Tensor, nkv: int, hd: int, dtype: torch.dtype) -> 
 def qk_rope_kv(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, *, q_gain: Optional[torch.Tensor],
                k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor], rotary_dim: int,
                variant: str, pos: torch.Tensor, row_req: torch.Tensor, kpages: Optional[torch.Tensor],
-               vpages: Optional[torch.Tensor], table: Optional[torch.Tensor], n_req: int) -> None:
+               vpages: Optional[torch.Tensor], table: Optional[torch.Tensor], n_req: int,
+               cos_sin: Optional[torch.Tensor] = None) -> None:
     """In place on the q heads of qkv[N, (nh + 2 nkv) hd]: per-head RMSNorm then rotation; k heads the
     same and into their cache page; v heads copied to theirs.  With kpages None only q is treated
-    (nkv then counts the k, v heads that the rows hold, usually 0)."""
-    require_cuda(qkv, q_gain, k_gain, inv_freq, pos, row_req, kpages, vpages, table)
+    (nkv then counts the k, v heads that the rows hold, usually 0).  `cos_sin`: what `rope_table`
+    made for these frequencies; positions beyond it are computed in the kernel."""
+    require_cuda(qkv, q_gain, k_gain, inv_freq, pos, row_req, kpages, vpages, table, cos_sin)
+    table_len = _check_cos_sin(cos_sin, inv_freq, rotary_dim)
     assert qkv.dim() == 2 and qkv.shape[0] == n_rows and qkv.stride(1) == 1
     assert qkv.shape[1] >= (nh + 2 * nkv) * hd
     for g in (q_gain, k_gain):
@@ -349,9 +353,27 @@ def qk_rope_kv(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, *, q_
         _i32(table, n_req, "block table")
         max_pages = table.shape[1]
     call("gibbs_qk_rope_kv", ptr(qkv), ptr(kpages), ptr(vpages), dtype_code(qkv.dtype), ptr(q_gain), ptr(k_gain),
-         float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(pos), ptr(row_req), ptr(table),
-         max_pages, page_size, num_pages, n_rows, nh, nkv, hd, qkv.stride(0) if n_rows > 1 else qkv.shape[1],
-         stream())
+         float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(cos_sin), table_len, ptr(pos),
+         ptr(row_req), ptr(table), max_pages, page_size, num_pages, n_rows, nh, nkv, hd,
+         qkv.stride(0) if n_rows > 1 else qkv.shape[1], stream())
+
+
+def _check_cos_sin(cos_sin: Optional[torch.Tensor], inv_freq: Optional[torch.Tensor], rotary_dim: int) -> int:
+    if cos_sin is None or inv_freq is None:
+        return 0
+    assert cos_sin.dtype == torch.float32 and cos_sin.dim() == 3 and cos_sin.is_contiguous()
+    assert cos_sin.shape[1:] == (rotary_dim // 2, 2), "the cos/sin table belongs to another rotary size"
+    return cos_sin.shape[0]
+
+
+def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
+    """[n_pos, len(inv_freq), 2] float32: cos and sin of float32(pos) * inv_freq[j], computed by the
+    functions that the kernels use for positions beyond a table."""
+    require_cuda(inv_freq)
+    assert inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and inv_freq.is_contiguous() and n_pos > 0
+    out = torch.empty((n_pos, inv_freq.shape[0], 2), dtype=torch.float32, device=inv_freq.device)
+    call("gibbs_rope_table", ptr(out), ptr(inv_freq), inv_freq.shape[0], n_pos, stream())
+    return out
 
 
 def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,

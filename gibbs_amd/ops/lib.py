@@ -41,13 +41,14 @@ _SIGNATURES = {
     "gibbs_skinny_conv": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_int, c_float, c_void_p,
                           c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p],
     "gibbs_attention_decode_fused": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                     c_float, c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     c_float, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_void_p],
     "gibbs_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_shortconv": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                         c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_rope_table": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gibbs_qk_rope_kv": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int,
-                         c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long,
+                         c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long,
                          c_void_p],
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p],

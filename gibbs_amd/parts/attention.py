@@ -80,7 +80,7 @@ class AttentionMixer(Mixer):
 
     def small_tensors(self):
         return [t for t in (self.q_gain, self.k_gain, None if self.position is None else self.position.inv_freq)
-                if t is not None]
+                if t is not None]   # of the cos/sin table a step reads one row per token: not counted
 
     def fold_input_gain(self, gain: torch.Tensor) -> None:
         """The preceding norm's gain, multiplied into the columns of the q, k, v projections."""
@@ -107,7 +107,7 @@ class AttentionMixer(Mixer):
             batch.tables[cache.group], batch.n_req, batch.pos, batch.row_req, self.scale, q_gain=self.q_gain,
             k_gain=self.k_gain, eps=self.qk_norm_eps, inv_freq=None if pos is None else pos.inv_freq,
             rotary_dim=0 if pos is None else pos.rotary_dim, variant="half_split" if pos is None else pos.variant,
-            window=self.window, max_seq=batch.max_seq)
+            window=self.window, max_seq=batch.max_seq, cos_sin=None if pos is None else pos.cos_sin)
 
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
@@ -127,7 +127,7 @@ class AttentionMixer(Mixer):
                        variant="half_split" if pos is None else pos.variant,
                        pos=batch.pos, row_req=batch.row_req,
                        kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None,
-                       table=table, n_req=batch.n_req)
+                       table=table, n_req=batch.n_req, cos_sin=None if pos is None else pos.cos_sin)
         a = self.attend(qkv, batch, cache, table)
         return linear(a, self.w_out, partial_ok=True)
 

@@ -36,6 +36,7 @@ class Runtime:
     """What a part needs to know about the run it is bound into."""
     device: torch.device
     act_dtype: torch.dtype          # activations and cache pages: bfloat16, or float32 for the 32-bit path
+    max_positions: int = 0          # positions a request can reach (tables over positions are sized by it); 0: unknown
 
 
 @dataclass

@@ -6,14 +6,22 @@ float32 operation, as LFM2's spec asks (/root/reference/src/arch/gen.rs:154-164,
 /root/reference/arch/families/lfm2.json5:64).  The angle of position p is float32(p) * inv_freq[j]
 (/root/reference/src/graph/cpu.rs:673); variant `half_split` turns the pair (j, j + rot/2),
 `interleaved` the pair (2j, 2j + 1) (:676-695).
+
+Cosine and sine of every angle up to the run's longest position are computed once, when the part is
+bound, into a table that the kernels read (the same float32 angle, the same functions: positions
+beyond the table are computed in the kernels and agree to the bit).
 """
 from __future__ import annotations
 
 import numpy as np
 import torch
 
+from .. import ops
 from ..weights.loader import WeightStore
 from .base import PositionEncoding, Runtime, register_position
+
+
+MAX_TABLE_POSITIONS = 1 << 20   # 8 bytes * rotary_dim / 2 each
 
 
 def rope_inv_freq(rotary_dim: int, theta: float, precision: str = "f64") -> np.ndarray:
@@ -44,3 +52,5 @@ class RotaryPosition(PositionEncoding):
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
         self.inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)
+        n_pos = min(int(rt.max_positions), MAX_TABLE_POSITIONS)
+        self.cos_sin = ops.rope_table(self.inv_freq, n_pos) if n_pos > 0 else None

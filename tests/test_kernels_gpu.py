@@ -332,8 +332,9 @@ def test_attention_far_key_stands_out(dtype):
 
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("variant", ["half_split", "interleaved"])
-@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 2, 128, 128)])
-def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot):
+@pytest.mark.parametrize("table_len", [0, 6, 64])       # no table; positions 9 and 17 beyond it; all from it
+@pytest.mark.parametrize("nh,nkv,hd,rot", [(4, 2, 16, 16), (3, 1, 48, 32), (2, 2, 128, 128), (2, 1, 24, 12)])
+def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot, table_len):
     from gibbs_amd import ops
     from gibbs_amd.parts.rope import rope_inv_freq
     n, page, num_pages = 6, 8, 10
@@ -346,8 +347,15 @@ def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot):
     table = i32([[4, 7, -1], [2, 9, 0], [5, 1, -1]])
     kp = torch.zeros(num_pages, nkv, page, hd, dtype=dtype, device=DEV)
     vp = torch.zeros_like(kp)
+    cos_sin = ops.rope_table(inv, table_len) if table_len else None
     ops.qk_rope_kv(qkv, n, nh, nkv, hd, q_gain=qg, k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
-                   pos=i32(positions), row_req=i32(row_req), kpages=kp, vpages=vp, table=table, n_req=3)
+                   pos=i32(positions), row_req=i32(row_req), kpages=kp, vpages=vp, table=table, n_req=3, cos_sin=cos_sin)
+    if table_len:   # a table changes nothing, to the bit: it holds what the kernel computes
+        qkv1, kp1, vp1 = qkv0.clone(), torch.zeros_like(kp), torch.zeros_like(vp)
+        ops.qk_rope_kv(qkv1, n, nh, nkv, hd, q_gain=qg, k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot,
+                       variant=variant, pos=i32(positions), row_req=i32(row_req), kpages=kp1, vpages=vp1, table=table,
+                       n_req=3)
+        assert torch.equal(qkv1, qkv) and torch.equal(kp1, kp) and torch.equal(vp1, vp)
 
     def ref(x, gain):                                     # x: [n, heads, hd] float64
         x = F.rms_norm(x, (hd,), gain.double(), eps=1e-6)
@@ -370,6 +378,17 @@ def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot):
         close(kp[pg, :, p % page], kr[i], dtype, "k page", bf16=8e-3)
         assert torch.equal(vp[pg, :, p % page], v0[i])
     assert kp.float().abs().sum(dim=(1, 3)).count_nonzero().item() == n, "exactly one page slot per row was written"
+
+
+def test_rope_table():
+    from gibbs_amd import ops
+    from gibbs_amd.parts.rope import rope_inv_freq
+    inv = torch.from_numpy(rope_inv_freq(48, 1e6, "f32")).to(DEV)
+    t = ops.rope_table(inv, 5000)
+    ang = (torch.arange(5000, dtype=torch.float32, device=DEV)[:, None] * inv[None, :]).double()   # float32 products
+    assert t.shape == (5000, 24, 2)
+    assert (t[..., 0].double() - ang.cos()).abs().max().item() < 2e-7
+    assert (t[..., 1].double() - ang.sin()).abs().max().item() < 2e-7
 
 
 def test_argmax_rules():
@@ -480,11 +499,11 @@ def test_embed_and_residual_mirror():
     close(out, F.rms_norm(x.double(), (72,), None, 1e-5), torch.bfloat16, "gain-free norm")
 
 
-@pytest.mark.parametrize("n_splits", [1, 4, None])
+@pytest.mark.parametrize("n_splits,table_len", [(1, 0), (4, 20), (None, 1024)])   # rows at 699 and 32 beyond a table of 20
 @pytest.mark.parametrize("variant", ["half_split", "interleaved"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,page,window", [(4, 2, 16, 16, 16, None), (32, 8, 64, 64, 16, None), (6, 1, 48, 32, 8, None),
                                                        (5, 5, 80, 80, 32, 37), (16, 2, 128, 128, 16, None), (24, 2, 32, 32, 16, None)])
-def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_splits):
+def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_splits, table_len):
     """The fused decode attention against the separate kernels: same pages afterwards, same output,
     for rows at a page's first slot, its last slot, position 0 and far into the cache."""
     from gibbs_amd import ops
@@ -505,7 +524,8 @@ def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_split
     kp1, vp1 = kp.clone(), vp.clone()
     got = ops.attention_decode_fused(qkv, n, nh, nkv, hd, kp1, vp1, table, n, pos, row_req, scale, q_gain=qg,
                                      k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
-                                     window=window, max_seq=700, n_splits=n_splits)
+                                     window=window, max_seq=700, n_splits=n_splits,
+                                     cos_sin=ops.rope_table(inv, table_len) if table_len else None)
     close(kp1, kp2, dtype, "new keys in the pages", bf16=8e-3)
     assert torch.equal(vp1, vp2)
     close(got, want, dtype, "fused decode attention", bf16=8e-3)
