@@ -1,13 +1,13 @@
 // Paged attention for rows that each attend over a long cache with few queries: decoded tokens
 // (and short prompt portions).  bfloat16 cache, float32 scores, maxima, sums and outputs.
 //
-// The work is bound by reading keys and values once, so it is split to fill the chip: one
-// workgroup per (row, kv head [, chunk of the group's query heads], slice of the keys).  All query
+// The work is reading keys and values once, so it is split to fill the chip: one workgroup of 4 or
+// 8 waves per (row, kv head [, chunk of the group's query heads], slice of the keys).  All query
 // heads that share the kv head are served from the same loads.  Inside a workgroup every LPK
 // neighbouring lanes own one key at a time (8 head-dim elements = 16 bytes per lane, so a wave
 // reads 1 KB of contiguous cache per instruction) and keep an online-softmax stream of their own
 // (max, sum, weighted values); the streams are merged at the end, first across the wave by
-// shuffles, then across the 4 waves through LDS.  With more than one slice the workgroup writes a
+// shuffles, then across the waves through LDS (wave g folds head g).  With more than one slice the workgroup writes a
 // partial (max, sum, values) and a second kernel merges the slices.  The slice's page ids are
 // staged in LDS, and the loads of the next two keys are in flight while a key is worked on.
 //
@@ -65,14 +65,14 @@ __device__ __forceinline__ void fold(float& ma, float& la, float* aa, float mb, 
   ma = m;
 }
 
-template <int LPK, int GT, bool RAW>
-__global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
+template <int LPK, int GT, bool RAW, int NW>
+__global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
                                                                bf16* __restrict__ vpages, float* __restrict__ partial,
                                                                bf16* __restrict__ out, DecodeArgs a) {
   constexpr int KPW = WAVE / LPK;
   constexpr int MAX_HD = LPK * EPL;
-  __shared__ float s_ml[4][GT][2];
-  __shared__ float s_acc[4][GT][MAX_HD];
+  __shared__ float s_ml[NW][GT][2];
+  __shared__ float s_acc[NW][GT][MAX_HD];
   __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
   __shared__ int s_pages[SEG_PAGES];
 
@@ -92,26 +92,44 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
   const int len = p + 1 - lo;
   int per = (len + a.n_splits - 1) / a.n_splits;
-  per = (per + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+  per = (per + NW * KPW - 1) / (NW * KPW) * (NW * KPW);
   const int k0 = lo + split * per;
   const int k1 = min(k0 + per, p + 1);
   const int* table = a.table + (size_t)a.row_req[row] * a.max_pages;
   const bf16* qrow = qkv + (size_t)row * a.ldq;
 
+  // Everything that does not hang on earlier arithmetic is asked for first: the query heads, the
+  // row's own key and value, the page ids of the slice's first segment (kept in registers until
+  // the prologue below is through, then put into LDS).
+  uint4 qraw[GT];
+#pragma unroll
+  for (int g = 0; g < GT; ++g)
+    qraw[g] = (g < gcount && active) ? *(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0) : make_uint4(0, 0, 0, 0);
+  const bool has_new = RAW && p >= k0 && p < k1;  // raw rows: this slice holds the row's own position
+  const bool new_lane = has_new && wave == 0 && grp == 0;
+  uint4 knew_raw = make_uint4(0, 0, 0, 0), vnew_raw = make_uint4(0, 0, 0, 0);
+  if (new_lane && active) {
+    knew_raw = *(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0);
+    vnew_raw = *(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0);
+  }
+  constexpr int PRE = (SEG_PAGES + NW * WAVE - 1) / (NW * WAVE);
+  const int first_page0 = a.page_shift >= 0 ? k0 >> a.page_shift : k0 / a.page_size;
+  const int seg1_0 = min(k1, (first_page0 + SEG_PAGES) * a.page_size);
+  int pre_page[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    const int j = threadIdx.x + i * NW * WAVE;
+    pre_page[i] = (j < SEG_PAGES && (first_page0 + j) * a.page_size < seg1_0) ? table[first_page0 + j] : 0;
+  }
+
   Rot8 rt;
   if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p, a.cs_table, a.table_len);
   const bool rotate = a.inv_freq != nullptr;
   // raw rows: the row's own key and value; wave 0's first LPK lanes prepare them for everyone
-  const bool has_new = RAW && p >= k0 && p < k1;
-  if (has_new && wave == 0 && grp == 0) {
+  if (new_lane) {
     float kf[EPL], vf[EPL];
-    if (active) {
-      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0), kf);
-      unpack8(*(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0), vf);
-    } else {
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) kf[i] = vf[i] = 0.f;
-    }
+    unpack8(knew_raw, kf);
+    unpack8(vnew_raw, vf);
     norm_rope8<LPK>(kf, e0, hd, a.k_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
     if (active) {
       // what later steps read from the page is the bfloat16 value: use the same value now
@@ -146,7 +164,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
 #pragma unroll
     for (int i = 0; i < EPL; ++i) { acc[g][i] = 0.f; qf[g][i] = 0.f; }
     if (g < gcount) {
-      if (active) unpack8(*(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0), qf[g]);
+      unpack8(qraw[g], qf[g]);
       if (RAW) {
         norm_rope8<LPK>(qf[g], e0, hd, a.q_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
 #pragma unroll
@@ -156,7 +174,6 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
       for (int i = 0; i < EPL; ++i) qf[g][i] *= a.scale;
     }
   }
-  __syncthreads();  // s_knew, s_vnew
 
   // The slice's page ids go to LDS first (one round trip for all of them, instead of a dependent
   // table load in front of every key's loads); the loads of the next two keys are issued before the
@@ -164,12 +181,16 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
   for (int seg0 = k0; seg0 < k1; seg0 += SEG_PAGES * a.page_size) {
     const int first_page = a.page_shift >= 0 ? seg0 >> a.page_shift : seg0 / a.page_size;
     const int seg1 = min(k1, (first_page + SEG_PAGES) * a.page_size);
-    __syncthreads();  // the previous segment's ids are no longer read
-    for (int j = threadIdx.x; j < SEG_PAGES && (first_page + j) * a.page_size < seg1; j += 256) {
-      int page = table[first_page + j];
-      s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
+    if (seg0 != k0) __syncthreads();  // the previous segment's ids are no longer read
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      const int j = threadIdx.x + i * NW * WAVE;
+      if (j < SEG_PAGES && (first_page + j) * a.page_size < seg1) {
+        const int page = seg0 == k0 ? pre_page[i] : table[first_page + j];
+        s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
+      }
     }
-    __syncthreads();
+    __syncthreads();  // the ids, and at the first segment the row's own key and value, are in LDS
     auto fetch = [&](int key, uint4& kr, uint4& vr) {
       kr = vr = make_uint4(0, 0, 0, 0);
       if (key < seg1 && !(RAW && key == p) && active) {
@@ -180,13 +201,13 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
       }
     };
     uint4 kraw[3], vraw[3];
-    // the wave's first key of this segment keeps the global stride pattern k0 + (4 it + wave) KPW + grp
+    // the wave's first key of this segment keeps the global stride pattern k0 + (NW it + wave) KPW + grp
     int key = k0 + wave * KPW + grp;
-    if (key < seg0) key += (seg0 - key + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    if (key < seg0) key += (seg0 - key + NW * KPW - 1) / (NW * KPW) * (NW * KPW);
     fetch(key, kraw[0], vraw[0]);
-    fetch(key + 4 * KPW, kraw[1], vraw[1]);
-    for (; key < seg1; key += 4 * KPW) {
-      fetch(key + 8 * KPW, kraw[2], vraw[2]);
+    fetch(key + NW * KPW, kraw[1], vraw[1]);
+    for (; key < seg1; key += NW * KPW) {
+      fetch(key + 2 * NW * KPW, kraw[2], vraw[2]);
       __builtin_amdgcn_sched_barrier(0);  // the loads above stay ahead of the arithmetic below
       float kf[EPL], vf[EPL];
       if (RAW && key == p) {
@@ -234,34 +255,33 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(const bf16* __res
     }
   }
   __syncthreads();
-  if (wave == 0 && grp == 0) {
+  // the waves' streams of head g meet in wave g % NW
+  if (grp != 0) return;
+  for (int g = wave; g < gcount; g += NW) {
+    float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
-      if (g >= gcount) break;
-      float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
+    for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
-      for (int w = 1; w < 4; ++w) {
-        float ab[EPL];
+    for (int w = 1; w < NW; ++w) {
+      float ab[EPL];
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
-        fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
+      for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
+      fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
+    }
+    const int head = kvh * G + g0 + g;
+    if (a.n_splits == 1) {
+      if (active) {
+        const float inv = 1.0f / ll;
+        bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
       }
-      const int head = kvh * G + g0 + g;
-      if (a.n_splits == 1) {
-        if (active) {
-          const float inv = 1.0f / ll;
-          bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
+    } else {
+      float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
+      if (sub == 0) { ps[0] = mm; ps[1] = ll; }
+      if (active) {
 #pragma unroll
-          for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
-        }
-      } else {
-        float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
-        if (sub == 0) { ps[0] = mm; ps[1] = ll; }
-        if (active) {
-#pragma unroll
-          for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
-        }
+        for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
       }
     }
   }
@@ -312,19 +332,27 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
   }
 }
 
-template <int LPK, bool RAW>
+template <int LPK, bool RAW, int NW>
 void launch_decode(int gt, dim3 grid, hipStream_t stream, const bf16* q, bf16* k, bf16* v, float* partial, bf16* out,
                    const DecodeArgs& a) {
   switch (gt) {
-    case 1: attention_decode_kernel<LPK, 1, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 2: attention_decode_kernel<LPK, 2, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 4: attention_decode_kernel<LPK, 4, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
-    default: attention_decode_kernel<LPK, 8, RAW><<<grid, 256, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 1: attention_decode_kernel<LPK, 1, RAW, NW><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 2: attention_decode_kernel<LPK, 2, RAW, NW><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 4: attention_decode_kernel<LPK, 4, RAW, NW><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
+    default: attention_decode_kernel<LPK, 8, RAW, NW><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
   }
 }
 
+template <int LPK, bool RAW>
+void launch_waves(int waves, int gt, dim3 grid, hipStream_t stream, const bf16* q, bf16* k, bf16* v, float* partial,
+                  bf16* out, const DecodeArgs& a) {
+  // 8 waves keep their streams of up to 8 heads of up to LPK * 8 elements in LDS: only where that fits
+  if (waves >= 8 && LPK * gt <= 128) launch_decode<LPK, RAW, 8>(gt, grid, stream, q, k, v, partial, out, a);
+  else launch_decode<LPK, RAW, 4>(gt, grid, stream, q, k, v, partial, out, a);
+}
+
 template <bool RAW>
-int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* partial, DecodeArgs a, int n_rows,
+int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* partial, DecodeArgs a, int n_rows, int waves,
                hipStream_t stream) {
   const int G = a.nh / a.nkv;
   const int gt = G >= 8 ? 8 : (G > 2 ? 4 : G);  // 1, 2, 4 or 8 query heads per workgroup
@@ -333,11 +361,11 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   GIBBS_REQUIRE((long)a.nkv * a.head_chunks <= 65535, "attention_decode: too many heads");
   dim3 grid(n_rows, a.nkv * a.head_chunks, a.n_splits);
   const int lanes = a.hd / EPL;  // lanes that hold data; LPK is the next power of two
-  if (lanes <= 2) launch_decode<2, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
-  else if (lanes <= 4) launch_decode<4, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
-  else if (lanes <= 8) launch_decode<8, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
-  else if (lanes <= 16) launch_decode<16, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
-  else launch_decode<32, RAW>(gt, grid, stream, q, kpages, vpages, partial, out, a);
+  if (lanes <= 2) launch_waves<2, RAW>(waves, gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 4) launch_waves<4, RAW>(waves, gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 8) launch_waves<8, RAW>(waves, gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else if (lanes <= 16) launch_waves<16, RAW>(waves, gt, grid, stream, q, kpages, vpages, partial, out, a);
+  else launch_waves<32, RAW>(waves, gt, grid, stream, q, kpages, vpages, partial, out, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
   if (a.n_splits > 1) {
@@ -358,7 +386,7 @@ GIBBS_EXPORT long gibbs_attention_decode_workspace(int n_rows, int nh, int hd, i
 GIBBS_EXPORT int gibbs_attention_decode(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
                                         const int* pos, const int* row_req, const int* table, int max_pages,
                                         int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                        long ldo, float scale, int window, int n_splits, hipStream_t stream) {
+                                        long ldo, float scale, int window, int n_splits, int waves, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_decode: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_decode: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd % 8 == 0 && hd <= 256, "attention_decode: head size %d must be a multiple of 8 up to 256", hd);
@@ -372,7 +400,7 @@ GIBBS_EXPORT int gibbs_attention_decode(const void* q, const void* kpages, const
   a.num_pages = num_pages; a.nh = nh; a.nkv = nkv; a.hd = hd; a.ldq = ldq; a.ldo = ldo; a.scale = scale;
   a.window = window; a.n_splits = n_splits;
   // the kernel only reads the pages here
-  return run_decode<false>((const bf16*)q, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, stream);
+  return run_decode<false>((const bf16*)q, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, waves, stream);
 }
 
 // qkv: [N, ld] bfloat16, raw projection (q heads, k heads, v heads) of N decoded tokens, one per request.
@@ -381,7 +409,7 @@ GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, voi
                                               const float* inv_freq, int rot, int variant, const float* cs_table,
                                               int table_len, const int* pos, const int* row_req, const int* table, int max_pages, int page_size,
                                               int num_pages, int n_rows, int nh, int nkv, int hd, long ld, long ldo,
-                                              float scale, int window, int n_splits, hipStream_t stream) {
+                                              float scale, int window, int n_splits, int waves, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention_decode_fused: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_decode_fused: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd % 16 == 0 && hd <= 256, "attention_decode_fused: head size %d must be a multiple of 16 up to 256", hd);
@@ -398,5 +426,5 @@ GIBBS_EXPORT int gibbs_attention_decode_fused(const void* qkv, void* kpages, voi
   a.window = window; a.n_splits = n_splits;
   a.q_gain = q_gain; a.k_gain = k_gain; a.eps = eps; a.inv_freq = inv_freq; a.rot = rot; a.variant = variant;
   a.cs_table = (const float2*)cs_table; a.table_len = cs_table ? table_len : 0;
-  return run_decode<true>((const bf16*)qkv, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, stream);
+  return run_decode<true>((const bf16*)qkv, (bf16*)kpages, (bf16*)vpages, (bf16*)out, partial, a, n_rows, waves, stream);
 }

@@ -247,7 +247,8 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
                            k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
                            rotary_dim: int, variant: str, window: Optional[int] = None,
                            max_seq: int = 0, n_splits: Optional[int] = None,
-                           out: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           out: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None,
+                           waves: Optional[int] = None) -> torch.Tensor:
     """Decode attention straight from the raw fused projection qkv[N, (nh + 2 nkv) hd] of N decoded
     tokens: q/k norm and rotation, the write of the new key and value to their pages, attention over
     split keys in one kernel (followed by the merge of the slices).  `cos_sin` as in `qk_rope_kv`."""
@@ -268,8 +269,10 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
         assert inv_freq.dtype == torch.float32 and inv_freq.shape == (rotary_dim // 2,) and inv_freq.is_contiguous()
         if rotary_dim % 16:
             raise KernelError(f"attention_decode_fused: rotary_dim {rotary_dim} must be a multiple of 16")
-    if n_splits is None:
-        n_splits = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+    if n_splits is None or waves is None:
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+        n_splits = auto_splits if n_splits is None else n_splits
+        waves = auto_waves if waves is None else waves
     partial = None
     if n_splits > 1:
         partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=qkv.device)
@@ -279,7 +282,8 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
     call("gibbs_attention_decode_fused", ptr(qkv), ptr(kpages), ptr(vpages), ptr(out), ptr(partial),
          ptr(q_gain), ptr(k_gain), float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(cos_sin),
          table_len, ptr(pos), ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
-         qkv.stride(0) if n_rows > 1 else qkv.shape[1], nh * hd, float(scale), int(window or 0), n_splits, stream())
+         qkv.stride(0) if n_rows > 1 else qkv.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves),
+         stream())
     return out
 
 
@@ -396,19 +400,23 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
     return out
 
 
-def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int) -> int:
-    """Key slices per (row, kv head) for the decode attention: enough workgroups to give each of
-    the 256 compute units two (measured best at batch 1, 8 and 64), but at least 64 keys to a slice."""
+def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int) -> tuple:
+    """(key slices per (row, kv head), waves per workgroup) for the decode attention.  Few rows:
+    enough slices of at least 64 keys to give each of the 256 compute units two workgroups of 4
+    waves.  Rows and heads that fill the chip by themselves: no slices, 8 waves (measured at batch
+    1 to 64 and 2,048 to 8,192 keys; a slice costs every wave its own prologue and final fold)."""
     gt = 8 if group >= 8 else (4 if group > 2 else group)
     per_split = n_rows * nkv * -(-group // gt)
+    if per_split >= 256:
+        return 1, 8
     want = -(-512 // per_split)
-    return max(1, min(want, max_seq // 64, 256))
+    return max(1, min(want, max_seq // 64, 256)), 4
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                      vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
                      scale: float, window: Optional[int] = None, max_seq: int = 0, n_splits: Optional[int] = None,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, waves: Optional[int] = None) -> torch.Tensor:
     """bfloat16 paged attention for rows with few queries and long caches (decoded tokens): the
     keys of each (row, kv head) are cut into `n_splits` slices that run as workgroups of their own
     and are merged afterwards.  Same operands and result as `attention_plain`."""
@@ -422,8 +430,10 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
     assert table.dim() == 2 and table.shape[0] >= n_req
     _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
-    if n_splits is None:
-        n_splits = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+    if n_splits is None or waves is None:
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+        n_splits = auto_splits if n_splits is None else n_splits
+        waves = auto_waves if waves is None else waves
     partial = None
     if n_splits > 1:
         partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=q.device)
@@ -432,7 +442,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
     call("gibbs_attention_decode", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(pos), ptr(row_req),
          ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
-         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, stream())
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves), stream())
     return out
 
 
