@@ -1,0 +1,164 @@
+"""`gibbs --bench SUITE.json`: the reference's suite protocol on this engine.
+
+A suite is `{"defaults": {...}, "models": [{...}, ...]}` (/root/reference/bench/loop.json).  Every
+model entry inherits the defaults; the keys that mean something here:
+
+    id              a model folder (config.json + model.safetensors), or "random:CONFIG.json" for
+                    random weights of that configuration (seed 0); relative to the suite file
+    name            label of the row (default: the folder's or file's name)
+    prefill_tokens  length of the timed prompt (default 512)
+    decode_tokens   decoded tokens per timed run (default 128)
+    runs            timed runs, of which the median counts (default 3)
+    batch           requests decoded side by side (default 1)
+    dtype           "bfloat16" (default) or "float32"
+    min_tok_s       the run fails (exit status 3) if decode is slower
+
+Protocol (/root/reference/src/bench.rs:241-322): prompts are seeded synthetic ids (the reference
+cycles an encoded sentence to length, :255-259; without tokenizers on this path the ids are drawn
+instead); one warm-up prefill, then the median of `runs`; 16 warm-up decode steps, then `runs`
+runs of `decode_tokens` steps with sampling on the device, median tokens a second.
+`roofline_tok_s = batch * ceiling / bytes a step must read` (:298).  One JSON row per model, then
+`METRIC <slug>_tok_s=...` lines and `METRIC geomean_roofline_pct=...` (:522, :739-746).  Exit
+status 2 on an error, 3 on a missed `min_tok_s` (:751-757).
+"""
+from __future__ import annotations
+
+import json
+import math
+import os
+import re
+import sys
+import time
+from typing import Dict, List
+
+DEFAULTS = {"prefill_tokens": 512, "decode_tokens": 128, "runs": 3, "batch": 1, "dtype": "bfloat16"}
+WARMUP_STEPS = 16
+
+
+def _median(xs: List[float]) -> float:
+    xs = sorted(xs)
+    return xs[len(xs) // 2]
+
+
+def _slug(name: str) -> str:
+    return re.sub(r"[^a-z0-9]+", "_", name.lower()).strip("_")
+
+
+def _load(entry: Dict, base: str):
+    import torch
+
+    from .config import config_from_dict
+    from .engine import Engine
+    from .parts import DecoderModel
+    from .weights import random_weights_on_device
+    ident = entry["id"]
+    batch, ctx = int(entry["batch"]), int(entry["prefill_tokens"]) + int(entry["decode_tokens"]) * (int(entry["runs"]) + 1) + WARMUP_STEPS + 64
+    if ident.startswith("random:"):
+        path = os.path.join(base, ident[len("random:"):])
+        with open(path) as f:
+            cfg = config_from_dict(json.load(f))
+        decls = DecoderModel(cfg.model_spec()).tensor_decls()
+        compute = torch.bfloat16 if entry["dtype"] == "bfloat16" else torch.float32
+        weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0")
+        return Engine(config=cfg, weights=weights, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
+    path = ident if os.path.isabs(ident) else os.path.join(base, ident)
+    return Engine(path, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
+
+
+def measure(entry: Dict, base: str) -> Dict:
+    import numpy as np
+    import torch
+
+    from . import roofline
+    from .engine.decode import DecodeLoop
+    engine = _load(entry, base)
+    vocab = engine.spec.vocab
+    n_prompt, n_decode, runs, batch = (int(entry[k]) for k in ("prefill_tokens", "decode_tokens", "runs", "batch"))
+    rng = np.random.default_rng(0)
+
+    def prompt():
+        return rng.integers(0, vocab, size=n_prompt).tolist()
+
+    times = []
+    for _ in range(runs + 1):                                   # the first is the warm-up
+        ids = prompt()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([("prefill", ids, [n_prompt - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        engine.release("prefill")
+    prefill_s = _median(times[1:])
+
+    rids = [f"r{i}" for i in range(batch)]
+    first = [int(engine.step([(rid, prompt(), [n_prompt - 1])]).argmax(-1).item()) for rid in rids]
+    loop = DecodeLoop(engine, rids, first)
+    loop.run(WARMUP_STEPS)
+    torch.cuda.synchronize()
+    wall, seq_lens = [], []
+    for _ in range(runs):
+        seq_lens.append([engine.cached_tokens(r) + n_decode // 2 for r in rids])
+        t0 = time.perf_counter()
+        loop.run(n_decode)
+        torch.cuda.synchronize()
+        wall.append(time.perf_counter() - t0)
+    mid = wall.index(_median(wall))
+    decode_s = wall[mid]
+    step_bytes = roofline.decode_bytes(engine, seq_lens[mid])
+    for rid in rids:
+        engine.release(rid)
+    tok_s = batch * n_decode / decode_s
+    roof = batch * roofline.HBM_BYTES_PER_S / step_bytes
+    return {"model": entry["name"], "batch": batch, "dtype": entry["dtype"],
+            "bytes_per_token": int(step_bytes // batch), "ceiling_gbps": roofline.HBM_BYTES_PER_S / 1e9,
+            "decode_tok_s": round(tok_s, 1), "roofline_tok_s": round(roof, 1),
+            "roofline_pct": round(100.0 * tok_s / roof, 2), "wall_ms": round(1e3 * decode_s, 3),
+            "ms_per_step": round(1e3 * decode_s / n_decode, 4), "prefill_tokens": n_prompt,
+            "prefill_tok_s": round(n_prompt / prefill_s, 1),
+            "prefill_peak_frac": round(roofline.prefill_flops(engine, n_prompt) / prefill_s
+                                       / roofline.PEAK_FLOPS[entry["dtype"]], 4)}
+
+
+def run_suite(path: str) -> int:
+    """Runs every model of the suite; returns the process's exit status."""
+    try:
+        with open(path) as f:
+            suite = json.load(f)
+        models = suite["models"]
+        if not models:
+            raise ValueError("the suite names no models")
+    except (OSError, ValueError, KeyError) as e:
+        print(f"gibbs --bench: cannot read suite {path!r}: {e}", file=sys.stderr)
+        return 2
+    base = os.path.dirname(os.path.abspath(path))
+    rows, missed, failed = [], [], False
+    for m in models:
+        entry = dict(DEFAULTS)
+        entry.update(suite.get("defaults", {}))
+        entry.update(m)
+        if "id" not in entry:
+            print("gibbs --bench: a model entry has no id", file=sys.stderr)
+            failed = True
+            continue
+        ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
+        entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
+        try:
+            row = measure(entry, base)
+        except Exception as e:     # one model's failure is reported; the others still run (bench.rs:751)
+            print(f"gibbs --bench: {entry['name']}: {type(e).__name__}: {e}", file=sys.stderr)
+            failed = True
+            continue
+        rows.append(row)
+        print(json.dumps(row), flush=True)
+        floor = entry.get("min_tok_s")
+        if floor is not None and row["decode_tok_s"] < float(floor):
+            missed.append(f"{row['model']}: {row['decode_tok_s']} tok/s is below min_tok_s {floor}")
+    for row in rows:
+        print(f"METRIC {_slug(row['model'])}_tok_s={row['decode_tok_s']}")
+        print(f"METRIC {_slug(row['model'])}_prefill_tok_s={row['prefill_tok_s']}")
+    if rows:
+        geo = math.exp(sum(math.log(max(r["roofline_pct"], 1e-9)) for r in rows) / len(rows))
+        print(f"METRIC geomean_roofline_pct={geo:.2f}")
+    for line in missed:
+        print(f"gibbs --bench: {line}", file=sys.stderr)
+    return 2 if failed else (3 if missed else 0)

@@ -279,3 +279,32 @@ def test_command_line(dirs, tmp_path):
     p = run("--model", str(tmp_path / "fresh"), "--random-weights", str(cfgfile), "--seed", "5", "--prompt-ids", "3,4",
             "--max-tokens", "3")
     assert p.returncode == 0 and os.path.isfile(tmp_path / "fresh" / "model.safetensors"), p.stderr[-2000:]
+
+
+def test_bench_suite_through_the_command_line(dirs, tmp_path):
+    """`gibbs --bench SUITE.json`: one JSON row per model, METRIC lines, and the reference's exit
+    statuses (3 for a missed min_tok_s, 2 for a suite that cannot be run)."""
+    run = lambda *a: subprocess.run([sys.executable, os.path.join(ROOT, "bin", "gibbs"), *a], capture_output=True,
+                                    text=True, timeout=300, env=dict(os.environ))
+    (tmp_path / "cfg.json").write_text(json.dumps(H.TINY["C"]))
+    suite = {"defaults": {"prefill_tokens": 40, "decode_tokens": 8, "runs": 2},
+             "models": [{"id": dirs["A"], "name": "Tiny A", "dtype": "float32"},
+                        {"id": "random:cfg.json", "batch": 3}]}
+    (tmp_path / "suite.json").write_text(json.dumps(suite))
+    p = run("--bench", str(tmp_path / "suite.json"))
+    assert p.returncode == 0, p.stderr[-2000:]
+    rows = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
+    assert [r["model"] for r in rows] == ["Tiny A", "cfg"] and rows[1]["batch"] == 3
+    for r in rows:
+        assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0 and 0 < r["roofline_pct"] < 100
+        assert abs(r["roofline_tok_s"] * r["bytes_per_token"] - r["ceiling_gbps"] * 1e9) < 1e-3 * r["ceiling_gbps"] * 1e9
+    assert "METRIC tiny_a_tok_s=" in p.stdout and "METRIC cfg_prefill_tok_s=" in p.stdout
+    assert "METRIC geomean_roofline_pct=" in p.stdout
+    suite["models"][0]["min_tok_s"] = 1e12
+    (tmp_path / "suite.json").write_text(json.dumps(suite))
+    p = run("--bench", str(tmp_path / "suite.json"))
+    assert p.returncode == 3 and "below min_tok_s" in p.stderr
+    assert run("--bench", str(tmp_path / "absent.json")).returncode == 2
+    suite["models"].append({"id": str(tmp_path / "no_such_model")})
+    (tmp_path / "suite.json").write_text(json.dumps(suite))
+    assert run("--bench", str(tmp_path / "suite.json")).returncode == 2
