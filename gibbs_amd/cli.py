@@ -1,7 +1,7 @@
 """Command line in the manner of the reference's `gibbs` binary (/root/reference/src/main.rs:27-189):
 the same option names and meanings where it has them (`--model`, `--prompt`, `--max-tokens`, `--ctx`,
-`--backend`, `--seed`, `--arch`, `--arch-dump`, `--bench`, `--probe-top5`), and this engine's own
-beside them.  One-shot generation prints the reference's lines (main.rs:741-772,
+`--backend`, `--seed`, `--arch`, `--arch-dump`, `--bench`, `--bench-parity`, `--probe-top5`), and this
+engine's own beside them (`--replay`, `--random-weights`, sampling and cache options).  One-shot generation prints the reference's lines (main.rs:741-772,
 scheduler/mod.rs:1113-1120)."""
 from __future__ import annotations
 
@@ -26,6 +26,11 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--arch-dump", action="store_true",
                     help="print the resolved configuration and the tensor table (JSON), then exit")
     ap.add_argument("--bench", help="benchmark suite (JSON): prints one JSON row per model and METRIC lines")
+    ap.add_argument("--bench-parity", action="store_true",
+                    help="8 greedy steps in bfloat16 and in float32: same tokens, cosine of the logits >= 0.999")
+    ap.add_argument("--replay", metavar="TRACE",
+                    help="replay a trace (JSON lines as for bin/trace_run; '-' is standard input) and write logits to --out")
+    ap.add_argument("--out", help="folder for the logits of --replay")
     ap.add_argument("--probe-top5", help="print the top-5 next-token logits (JSON) for these comma-separated ids")
     ap.add_argument("--temperature", type=float, default=None, help="sampling temperature (one-shot default 0.7; <= 1e-4 is greedy)")
     ap.add_argument("--top-p", type=float, default=None, help="nucleus cut (default 0.9)")
@@ -37,6 +42,7 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--chunk", type=int, default=None, help="most prompt tokens of one request per step")
     ap.add_argument("--page-size", type=int, default=None, help="tokens per cache page")
     ap.add_argument("--cache-tokens", type=int, default=None, help="tokens the cache pool holds")
+    ap.add_argument("--num-pages", type=int, default=None, help="pages the cache pool holds (instead of --cache-tokens)")
     ap.add_argument("--max-requests", type=int, default=8, help="requests that may be live at once")
     ap.add_argument("--ignore-eos", action="store_true", help="do not stop at an end-of-sequence token")
     return ap
@@ -48,6 +54,33 @@ def _tokenizer(model_dir: str):
         return None
     from tokenizers import Tokenizer
     return Tokenizer.from_file(path)
+
+
+def _parity(make_engine, prompt: List[int], steps: int = 8) -> int:
+    """The reference's device-parity gate (/root/reference/src/bench.rs:761-883: 8 greedy steps on
+    Metal and on the CPU, same argmax, cosine >= 0.999), here between the bfloat16 path and the
+    true 32-bit path.  The float32 run's tokens are forced on the bfloat16 run so that every step
+    compares logits of the same sequence."""
+    import torch
+    rows = {}
+    forced: List[int] = []
+    for dt in ("float32", "bfloat16"):
+        engine = make_engine(dt)
+        logits = [engine.step([("p", prompt, [len(prompt) - 1])])[0].float()]
+        for i in range(steps - 1):
+            tok = forced[i] if dt == "bfloat16" else int(logits[-1].argmax())
+            if dt == "float32":
+                forced.append(tok)
+            logits.append(engine.step([("p", [tok], [0])])[0].float())
+        rows[dt] = torch.stack(logits).cpu()
+        del engine
+    a, b = rows["float32"], rows["bfloat16"]
+    cos = torch.nn.functional.cosine_similarity(a, b, dim=-1)
+    same = (a.argmax(-1) == b.argmax(-1))
+    ok = bool(same.all()) and float(cos.min()) >= 0.999
+    print(json.dumps({"steps": steps, "same_argmax": same.tolist(), "cosine": [round(float(c), 6) for c in cos],
+                      "pass": ok}))
+    return 0 if ok else 1
 
 
 def _ids(text: str) -> List[int]:
@@ -86,10 +119,27 @@ def main(argv: Optional[List[str]] = None) -> int:
 
     from .engine import Engine, Generator
     from .sampling import SamplingParams
+    from .engine.engine import DEFAULT_PAGE_SIZE
     max_tokens = 64 if args.max_tokens is None else args.max_tokens
-    engine = Engine(args.model, dtype=args.dtype, arch=args.arch, ctx=args.ctx, max_requests=args.max_requests,
-                    max_tokens=args.cache_tokens or 16384,
-                    **({"page_size": args.page_size} if args.page_size else {}))
+    page = args.page_size or DEFAULT_PAGE_SIZE
+    pool = args.num_pages * page if args.num_pages else (args.cache_tokens or 16384)
+    dtype = {"bf16": "bfloat16", "fp32": "float32"}.get(args.dtype, args.dtype)
+
+    def make_engine(dt):
+        return Engine(args.model, dtype=dt, arch=args.arch, ctx=args.ctx, max_requests=args.max_requests,
+                      max_tokens=pool, page_size=page)
+
+    if args.bench_parity:
+        return _parity(make_engine, _ids(args.prompt_ids) if args.prompt_ids else [1, 2, 3, 4, 5, 6])
+    engine = make_engine(dtype)
+    if args.replay:
+        if not args.out:
+            print("gibbs: --replay needs --out", file=sys.stderr)
+            return 2
+        from .replay import replay
+        lines = sys.stdin if args.replay == "-" else open(args.replay)
+        replay(engine, lines, args.out)
+        return 0
     if args.probe_top5:
         ids = _ids(args.probe_top5)
         logits = engine.step([("probe", ids, [len(ids) - 1])])[0]

@@ -16,7 +16,35 @@ import json
 import os
 import sys
 
-import numpy as np
+
+def replay(engine, lines, out_dir: str, report=print) -> None:
+    """Runs the steps of `lines` (JSON objects, one a line) through `engine.step`."""
+    from .engine import Entry
+    os.makedirs(out_dir, exist_ok=True)
+    for line in lines:
+        line = line.strip()
+        if not line:
+            continue
+        rec = json.loads(line)
+        step = rec["step"]
+        entries = [Entry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
+        if entries:
+            logits = engine.step(entries)
+            if logits is not None:
+                arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
+                tmp = os.path.join(out_dir, f".{step}.f32.tmp")
+                arr.tofile(tmp)
+                os.replace(tmp, os.path.join(out_dir, f"{step}.f32"))
+        for rid in rec.get("end", []):
+            if rid in engine.cache:
+                engine.release(rid)
+        report(f"done {step}", flush=True)
+
+
+def pool_tokens_for(max_tokens: int, page: int) -> int:
+    """Every request's count is rounded up to a multiple of max(64, page size)."""
+    unit = max(64, page)
+    return -(-max_tokens // unit) * unit
 
 
 def main(argv=None) -> int:
@@ -32,36 +60,14 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
 
     print("trace_run: loading kernels and model", file=sys.stderr, flush=True)
-    from .engine import Engine, Entry
+    from .engine import Engine
     from .engine.engine import DEFAULT_PAGE_SIZE
 
     page = args.page_size or DEFAULT_PAGE_SIZE
-    # every request's count is rounded up to a multiple of max(64, page size)
-    unit = max(64, page)
-    pool_tokens = -(-args.max_tokens // unit) * unit
-    engine = Engine(args.model, dtype=args.dtype, max_tokens=pool_tokens, max_requests=args.max_requests,
-                    page_size=page)
-    os.makedirs(args.out, exist_ok=True)
+    engine = Engine(args.model, dtype=args.dtype, max_tokens=pool_tokens_for(args.max_tokens, page),
+                    max_requests=args.max_requests, page_size=page)
     print("trace_run: ready", file=sys.stderr, flush=True)
-
-    for line in sys.stdin:
-        line = line.strip()
-        if not line:
-            continue
-        rec = json.loads(line)
-        step = rec["step"]
-        entries = [Entry(e["id"], e["tokens"], e.get("want", [])) for e in rec.get("entries", [])]
-        if entries:
-            logits = engine.step(entries)
-            if logits is not None:
-                arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
-                tmp = os.path.join(args.out, f".{step}.f32.tmp")
-                arr.tofile(tmp)
-                os.replace(tmp, os.path.join(args.out, f"{step}.f32"))
-        for rid in rec.get("end", []):
-            if rid in engine.cache:
-                engine.release(rid)
-        print(f"done {step}", flush=True)
+    replay(engine, sys.stdin, args.out)
     return 0
 
 

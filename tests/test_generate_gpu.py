@@ -281,6 +281,26 @@ def test_command_line(dirs, tmp_path):
     assert p.returncode == 0 and os.path.isfile(tmp_path / "fresh" / "model.safetensors"), p.stderr[-2000:]
 
 
+def test_command_line_replay_and_parity(dirs, tmp_path):
+    run = lambda *a, **k: subprocess.run([sys.executable, os.path.join(ROOT, "bin", "gibbs"), *a], capture_output=True,
+                                         text=True, timeout=300, env=dict(os.environ), **k)
+    toks = H.tokens(11, 20, 256)
+    trace = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:12], "want": [11]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": toks[12:], "want": [0, 7]}], "end": ["a"]}]
+    (tmp_path / "trace.jsonl").write_text("".join(json.dumps(t) + "\n" for t in trace))
+    p = run("--model", dirs["A"], "--dtype", "fp32", "--replay", str(tmp_path / "trace.jsonl"), "--out",
+            str(tmp_path / "logits"), "--num-pages", "8")
+    assert p.returncode == 0 and p.stdout.split() == ["done", "0", "done", "1"], p.stderr[-2000:]
+    want = H.plain_logits(dirs["A"], toks)
+    got = np.fromfile(tmp_path / "logits" / "1.f32", dtype="<f4").reshape(2, -1)
+    H.assert_close(got, want[[12, 19]], "float32", "replay through the command line")
+    assert run("--model", dirs["A"], "--replay", "-", input="").returncode == 2          # no --out
+    p = run("--model", dirs["A"], "--bench-parity", "--prompt-ids", ",".join(map(str, toks[:9])))
+    row = json.loads(p.stdout.strip().splitlines()[-1])
+    assert row["steps"] == 8 and len(row["cosine"]) == 8 and min(row["cosine"]) >= 0.999
+    assert p.returncode == (0 if row["pass"] else 1) and row["pass"] == all(row["same_argmax"])
+
+
 def test_bench_suite_through_the_command_line(dirs, tmp_path):
     """`gibbs --bench SUITE.json`: one JSON row per model, METRIC lines, and the reference's exit
     statuses (3 for a missed min_tok_s, 2 for a suite that cannot be run)."""
