@@ -1,7 +1,7 @@
 // Matrix product for few rows (decode: one row per live request, up to 64):
 //   Y[n, o] = sum_k X[n, k] * W[o, k],  bfloat16 operands, float32 accumulation.
 // The work is reading W once, so the layout serves that: a workgroup owns 16 output features and a
-// range of k; its 8 waves split the range, each streaming its part of the 16 rows of W straight
+// range of k (or 4 such tiles at once, for many rows of X); its 8 waves split the range, each streaming its part of the 16 rows of W straight
 // from memory into the A operand of v_mfma_f32_16x16x32_bf16 (a lane holds 8 consecutive k of one
 // row, so no LDS staging is needed), with X (small, cache resident) as the B operand: 16 rows of
 // X per MFMA, NT such tiles for up to 64 rows.  The waves' sums meet in LDS.  When 16-feature
@@ -16,14 +16,17 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 enum { OUT_BF16 = 0, OUT_F32 = 1 };
 constexpr int WAVES = 8;
 
-template <int NT, int OUT>
+// FT: tiles of 16 features per workgroup, computed from the same B operands (for more than 32 rows
+// of X: every workgroup re-reads X from L2, so it should use each B operand for more of W).
+template <int NT, int FT, int OUT>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ W, const bf16* __restrict__ X,
                                                           void* __restrict__ Yv, int N, int O, int I, long ldw,
                                                           long ldx, long ldy, int k_per_block, long split_stride) {
-  __shared__ floatx4 red[WAVES - 1][NT][WAVE];
+  static_assert(FT <= WAVES, "wave f finishes tile f");
+  __shared__ floatx4 red[WAVES][FT][NT][WAVE];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int o0 = blockIdx.x * 16;
+  const int o0 = blockIdx.x * 16 * FT;
   const int kb0 = blockIdx.y * k_per_block;
   const int kb1 = min(I, kb0 + k_per_block);
   // the wave's share of the block's range, in whole MFMA steps of 32
@@ -32,8 +35,13 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
   const int k_begin = kb0 + wave * per_wave * 32;
   const int k_end = min(kb1, k_begin + per_wave * 32);
 
-  const bool row_ok = o0 + r < O;
-  const bf16* wrow = W + (size_t)(row_ok ? o0 + r : 0) * ldw + g * 8;
+  bool row_ok[FT];
+  const bf16* wrow[FT];
+#pragma unroll
+  for (int f = 0; f < FT; ++f) {
+    row_ok[f] = o0 + f * 16 + r < O;
+    wrow[f] = W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
+  }
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -41,72 +49,92 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
     x_ok[t] = t * 16 + r < N;
     xrow[t] = X + (size_t)(x_ok[t] ? t * 16 + r : 0) * ldx + g * 8;
   }
-  floatx4 acc[NT];
+  floatx4 acc[FT][NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) acc[t] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int f = 0; f < FT; ++f)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[f][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  constexpr int U = 4;  // MFMA steps per iteration: 4 loads of W in flight per lane
+  constexpr int U = FT * NT >= 8 ? 2 : 4;  // MFMA steps per iteration: U * FT loads of W in flight per lane
   for (int k = k_begin; k < k_end; k += 32 * U) {
-    bf16x8 a[U], b[U][NT];
+    bf16x8 a[U][FT], b[U][NT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int kk = k + u * 32;
       const bool k_ok = kk + g * 8 < k_end;
-      a[u] = (row_ok && k_ok) ? *(const bf16x8*)(wrow + kk) : zero;
+#pragma unroll
+      for (int f = 0; f < FT; ++f) a[u][f] = (row_ok[f] && k_ok) ? *(const bf16x8*)(wrow[f] + kk) : zero;
 #pragma unroll
       for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u], b[u][t], acc[t], 0, 0, 0);
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][f], b[u][t], acc[f][t], 0, 0, 0);
   }
 
-  if (wave > 0) {
+  // the waves' sums meet in LDS; wave f adds those of tile f in the order of the waves
 #pragma unroll
-    for (int t = 0; t < NT; ++t) red[wave - 1][t][lane] = acc[t];
-  }
+  for (int f = 0; f < FT; ++f)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave][f][t][lane] = acc[f][t];
   __syncthreads();
-  if (wave != 0) return;
+  if (wave >= FT) return;
+  const int tile = wave;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
+    floatx4 sum = red[0][tile][t][lane];
 #pragma unroll
-    for (int w = 0; w < WAVES - 1; ++w) acc[t] += red[w][t][lane];
+    for (int w = 1; w < WAVES; ++w) sum += red[w][tile][t][lane];
     // D[feature (lane/16)*4 + i][row lane%16]: 4 consecutive features of one row of Y
-    const int n = t * 16 + r, o = o0 + g * 4;
+    const int n = t * 16 + r, o = o0 + tile * 16 + g * 4;
     if (n >= N) continue;
     if (OUT == OUT_BF16) {
       bf16* y = (bf16*)Yv + (size_t)n * ldy + o;
       if (o + 3 < O && (ldy % 4 == 0)) {
         typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
-        bf16x4 v = {(bf16)acc[t][0], (bf16)acc[t][1], (bf16)acc[t][2], (bf16)acc[t][3]};
+        bf16x4 v = {(bf16)sum[0], (bf16)sum[1], (bf16)sum[2], (bf16)sum[3]};
         *(bf16x4*)y = v;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (o + i < O) y[i] = (bf16)acc[t][i];
+          if (o + i < O) y[i] = (bf16)sum[i];
       }
     } else {
       float* y = (float*)Yv + (size_t)blockIdx.y * split_stride + (size_t)n * ldy + o;
       if (o + 3 < O && (ldy % 4 == 0)) {
-        *(floatx4*)y = acc[t];
+        *(floatx4*)y = sum;
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (o + i < O) y[i] = acc[t][i];
+          if (o + i < O) y[i] = sum[i];
       }
     }
   }
 }
 
 template <int NT>
-void launch(int out, dim3 grid, hipStream_t s, const bf16* W, const bf16* X, void* Y, int N, int O, int I, long ldw,
-            long ldx, long ldy, int kpb, long ss) {
+void launch(int out, int ft, int n_out, int k_splits, hipStream_t s, const bf16* W, const bf16* X, void* Y, int N, int O, int I,
+            long ldw, long ldx, long ldy, int kpb, long ss) {
+  if constexpr (NT >= 3) {
+    if (ft == 4) {
+      dim3 grid(ceil_div(n_out, 64), k_splits);
+      if (out == OUT_BF16)
+        gemm_skinny_kernel<NT, 4, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+      else
+        gemm_skinny_kernel<NT, 4, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+      return;
+    }
+  }
+  dim3 grid(ceil_div(n_out, 16), k_splits);
   if (out == OUT_BF16)
-    gemm_skinny_kernel<NT, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+    gemm_skinny_kernel<NT, 1, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
   else
-    gemm_skinny_kernel<NT, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+    gemm_skinny_kernel<NT, 1, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
 }
 }  // namespace
 
@@ -125,14 +153,15 @@ GIBBS_EXPORT int gibbs_gemm_skinny(const void* X, const void* W, void* Y, int ou
   int kpb = ceil_div(ceil_div(I, k_splits), 128) * 128;
   const int used = ceil_div(I, kpb);
   GIBBS_REQUIRE(used == k_splits, "gemm_skinny: %d k splits leave some empty for inner size %d (use %d)", k_splits, I, used);
-  dim3 grid(ceil_div(O, 16), k_splits);
   const int out = out_dtype == GIBBS_BF16 ? OUT_BF16 : OUT_F32;
+  // more than 32 rows of X: 4 tiles of 16 features per workgroup where that leaves enough workgroups
+  const int ft = (N > 32 && (long)ceil_div(O, 64) * k_splits >= 128) ? 4 : 1;
   const long ss = (long)N * ldy;
   const bf16 *w = (const bf16*)W, *x = (const bf16*)X;
   const int nt = ceil_div(N, 16);
-  if (nt == 1) launch<1>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
-  else if (nt == 2) launch<2>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
-  else if (nt == 3) launch<3>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
-  else launch<4>(out, grid, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  if (nt == 1) launch<1>(out, ft, O, k_splits, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else if (nt == 2) launch<2>(out, ft, O, k_splits, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else if (nt == 3) launch<3>(out, ft, O, k_splits, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+  else launch<4>(out, ft, O, k_splits, stream, w, x, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
   GIBBS_LAUNCH_STATUS("gemm_skinny");
 }

@@ -26,6 +26,11 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
+// (Non-temporal loads of W, meant to keep the rows of X in the L2, made the products slower: measured.)
+__device__ __forceinline__ bf16x8 load_w(const bf16* p) {
+  return *(const bf16x8*)p;
+}
+
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_GLU = 2, EPI_CONV = 3 };
 constexpr int MAX_TAPS = 8;
 
@@ -54,23 +59,32 @@ struct FusedArgs {
 
 // KC: the convolution's kernel length when it is 2..4 (its operands are then asked for before the
 // product), 0 for any other length or epilogue.
-template <int NT, int RG, int ROWS, int WAVES, bool RMS, int EPI, int KC>
+// FT: tiles of ROWS features that a workgroup computes from the same B operands (more rows of X
+// than one or two MFMA tiles: X is re-read from L2 by every workgroup, so a workgroup should use
+// each B operand for more of W).  Wave f sums tile f over the waves and runs its epilogue.
+template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
-  __shared__ floatx4 red[WAVES - 1][RG][NT][WAVE];
+  static_assert(FT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only");
+  __shared__ floatx4 red[WAVES][FT][RG][NT][WAVE];
   __shared__ float red_ss[WAVES][NT][16];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
-  const int o0 = blockIdx.x * ROWS;
+  const int o0 = blockIdx.x * ROWS * FT;
   // the wave's share of k, in whole MFMA steps of 32
   const int steps = (a.I + 31) / 32;
   const int per_wave = (steps + WAVES - 1) / WAVES;
   const int k_begin = wave * per_wave * 32;
   const int k_end = min(a.I, k_begin + per_wave * 32);
 
-  const bool row_ok = r < ROWS && o0 + r < a.O;
-  const bf16* wrow[RG];
+  bool row_ok[FT];
+  const bf16* wrow[FT][RG];
 #pragma unroll
-  for (int q = 0; q < RG; ++q) wrow[q] = a.W + ((size_t)q * a.group_stride + (row_ok ? o0 + r : 0)) * a.ldw + g * 8;
+  for (int f = 0; f < FT; ++f) {
+    row_ok[f] = r < ROWS && o0 + f * ROWS + r < a.O;
+#pragma unroll
+    for (int q = 0; q < RG; ++q)
+      wrow[f][q] = a.W + ((size_t)q * a.group_stride + (row_ok[f] ? o0 + f * ROWS + r : 0)) * a.ldw + g * 8;
+  }
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -117,25 +131,29 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     }
   }
 
-  floatx4 acc[RG][NT];
+  floatx4 acc[FT][RG][NT];
   float ss[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     ss[t] = 0.f;
 #pragma unroll
-    for (int q = 0; q < RG; ++q) acc[q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int f = 0; f < FT; ++f)
+#pragma unroll
+      for (int q = 0; q < RG; ++q) acc[f][q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  constexpr int U = (RG * NT >= 6) ? 2 : 4;  // MFMA steps per iteration
+  constexpr int U = (FT * RG * NT >= 6) ? 2 : 4;  // MFMA steps per iteration
   for (int k = k_begin; k < k_end; k += 32 * U) {
-    bf16x8 av[U][RG], bv[U][NT];
+    bf16x8 av[U][FT][RG], bv[U][NT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int kk = k + u * 32;
       const bool k_ok = kk + g * 8 < k_end;
 #pragma unroll
-      for (int q = 0; q < RG; ++q) av[u][q] = (row_ok && k_ok) ? *(const bf16x8*)(wrow[q] + kk) : zero;
+      for (int f = 0; f < FT; ++f)
+#pragma unroll
+        for (int q = 0; q < RG; ++q) av[u][f][q] = (row_ok[f] && k_ok) ? load_w(wrow[f][q] + kk) : zero;
 #pragma unroll
       for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
     }
@@ -151,8 +169,10 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
           }
         }
 #pragma unroll
-        for (int q = 0; q < RG; ++q)
-          acc[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][q], bv[u][t], acc[q][t], 0, 0, 0);
+        for (int f = 0; f < FT; ++f)
+#pragma unroll
+          for (int q = 0; q < RG; ++q)
+            acc[f][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][f][q], bv[u][t], acc[f][q][t], 0, 0, 0);
       }
   }
 
@@ -165,27 +185,33 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       if (g == 0) red_ss[wave][t][r] = ss[t];
     }
   }
-  // the waves' partial products meet in wave 0, added in the order of the waves
-  if (wave != 0) {
+  // the waves' partial products meet in LDS; wave f adds those of tile f in the order of the waves
+#pragma unroll
+  for (int f = 0; f < FT; ++f)
 #pragma unroll
     for (int q = 0; q < RG; ++q)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) red[wave - 1][q][t][lane] = acc[q][t];
-  }
+      for (int t = 0; t < NT; ++t) red[wave][f][q][t][lane] = acc[f][q][t];
   __syncthreads();
-  if (wave != 0) return;
+  if (wave >= FT) return;
+  const int tile = wave;
+  floatx4 sum[RG][NT];
+#pragma unroll
+  for (int q = 0; q < RG; ++q)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) sum[q][t] = red[0][tile][q][t][lane];
 #pragma unroll(RG * NT <= 2 ? WAVES : 1)
   for (int w = 1; w < WAVES; ++w)
 #pragma unroll
     for (int q = 0; q < RG; ++q)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) acc[q][t] += red[w - 1][q][t][lane];
+      for (int t = 0; t < NT; ++t) sum[q][t] += red[w][tile][q][t][lane];
 
   // D[feature g*4 + i][row r] of tile t: lane holds 4 consecutive features of one row
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int n = t * 16 + r;
-    const int o = o0 + g * 4;
+    const int o = o0 + tile * ROWS + g * 4;
     if (n >= a.N || g * 4 >= ROWS || o >= a.O) continue;
     float scale = 1.f;
     if (RMS) {
@@ -198,10 +224,10 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     if (EPI == EPI_STORE) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       if (full && a.ldy % 4 == 0) {
-        *(bf16x4*)y = bf16x4{(bf16)(acc[0][t][0] * scale), (bf16)(acc[0][t][1] * scale), (bf16)(acc[0][t][2] * scale),
-                             (bf16)(acc[0][t][3] * scale)};
+        *(bf16x4*)y = bf16x4{(bf16)(sum[0][t][0] * scale), (bf16)(sum[0][t][1] * scale), (bf16)(sum[0][t][2] * scale),
+                             (bf16)(sum[0][t][3] * scale)};
       } else {
-        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = (bf16)(acc[0][t][i] * scale);
+        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = (bf16)(sum[0][t][i] * scale);
       }
     } else if (EPI == EPI_RESIDUAL) {
       float* xp = a.x + (size_t)n * a.O + o;
@@ -209,14 +235,14 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (o + i >= a.O) break;
-        const float v = pre_x[t][i] + acc[0][t][i] * scale;
+        const float v = pre_x[t][i] + sum[0][t][i] * scale;
         xp[i] = v;
         bp[i] = (bf16)v;
       }
     } else if (EPI == EPI_GLU) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
-        const float gt = acc[0][t][i] * scale, up = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        const float gt = sum[0][t][i] * scale, up = sum[RG > 1 ? 1 : 0][t][i] * scale;
         y[i] = (bf16)(gt * (1.0f / (1.0f + expf(-gt))) * up);
       }
     } else if (KC > 1) {  // EPI_CONV, operands at hand
@@ -226,8 +252,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       for (int i = 0; i < 4; ++i) {
         if (o + i >= a.O) break;
         const int c = o + i;
-        const float bx = (acc[0][t][i] * scale) * (acc[RG > 2 ? 2 : 0][t][i] * scale);
-        const float cg = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        const float bx = (sum[0][t][i] * scale) * (sum[RG > 2 ? 2 : 0][t][i] * scale);
+        const float cg = sum[RG > 1 ? 1 : 0][t][i] * scale;
         float cv = 0.f;
 #pragma unroll
         for (int j = 0; j < KC - 1; ++j) cv = fmaf(pre_taps[j][i], pre_hist[t][j][i], cv);
@@ -245,8 +271,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
         const int c = o + i;
-        const float bx = (acc[0][t][i] * scale) * (acc[RG > 2 ? 2 : 0][t][i] * scale);
-        const float cg = acc[RG > 1 ? 1 : 0][t][i] * scale;
+        const float bx = (sum[0][t][i] * scale) * (sum[RG > 2 ? 2 : 0][t][i] * scale);
+        const float cg = sum[RG > 1 ? 1 : 0][t][i] * scale;
         float hist[MAX_TAPS - 1];
         float cv = 0.f;
 #pragma unroll
@@ -272,12 +298,20 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 
 template <int NT, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
-  // few features: halve the rows per workgroup so that every compute unit gets one
   static const int rows8_below = getenv("GIBBS_SKINNY_ROWS8_BELOW") ? atoi(getenv("GIBBS_SKINNY_ROWS8_BELOW")) : 256;
-  if (a.O / 16 < rows8_below) {
-    gemm_skinny_fused_kernel<NT, RG, 8, 8, RMS, EPI, KC><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+  static const int tiles2_from = getenv("GIBBS_SKINNY_TILES2_FROM") ? atoi(getenv("GIBBS_SKINNY_TILES2_FROM")) : 192;
+  if constexpr (NT >= 3 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
+    // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
+    if (a.O / 32 >= tiles2_from) {
+      gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(a);
+      return;
+    }
+  }
+  // few features: halve the rows per workgroup so that every compute unit gets one
+  if (NT <= 2 && a.O / 16 < rows8_below) {
+    gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
   } else {
-    gemm_skinny_fused_kernel<NT, RG, 16, 8, RMS, EPI, KC><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
   }
 }
 

@@ -101,28 +101,32 @@ GIBBS_EXPORT int gibbs_add_partials_rmsnorm(float* x, const float* partials, int
 }
 
 // x[r] += delta[r] alone (the last residual add of a model whose tail norms only some rows
-// still has to leave x whole for callers that read it).
+// still has to leave x whole for callers that read it).  float32 delta may be `n_partials` partial
+// sums, `partial_stride` elements apart, added in ascending order.
 template <typename T>
-__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, bf16* __restrict__ mirror,
-                                    size_t count) {
+__global__ void residual_add_kernel(float* __restrict__ x, const T* __restrict__ delta, int n_partials,
+                                    size_t partial_stride, bf16* __restrict__ mirror, size_t count) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < count) {
-    const float v = delta ? x[i] + to_float(delta[i]) : x[i];
+    float v = x[i];
+    if (delta)
+      for (int s = 0; s < n_partials; ++s) v += to_float(delta[s * partial_stride + i]);
     x[i] = v;
     if (mirror) mirror[i] = (bf16)v;
   }
 }
 
 // x += delta (delta may be null); mirror (optional) = bfloat16(x).
-GIBBS_EXPORT int gibbs_residual_add(float* x, const void* delta, int dtype, void* mirror, long count,
-                                    hipStream_t stream) {
-  GIBBS_REQUIRE(count >= 0, "residual_add: bad count");
+GIBBS_EXPORT int gibbs_residual_add(float* x, const void* delta, int dtype, int n_partials, long partial_stride,
+                                    void* mirror, long count, hipStream_t stream) {
+  GIBBS_REQUIRE(count >= 0 && n_partials >= 1 && (n_partials == 1 || (dtype == GIBBS_F32 && partial_stride >= count)),
+                "residual_add: bad count %ld or partial sums (%d, stride %ld)", count, n_partials, partial_stride);
   if (count == 0) return 0;
   const int blocks = ceil_div(count, 256);
   if (dtype == GIBBS_F32)
-    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (bf16*)mirror, (size_t)count);
+    residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, n_partials, (size_t)partial_stride, (bf16*)mirror, (size_t)count);
   else if (dtype == GIBBS_BF16)
-    residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (bf16*)mirror, (size_t)count);
+    residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, 1, 0, (bf16*)mirror, (size_t)count);
   else
     return gibbs_fail("residual_add: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("residual_add");

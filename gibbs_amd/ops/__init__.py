@@ -66,18 +66,22 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], gain: Optional[t
 
 
 def residual_add(x: torch.Tensor, delta: Optional[torch.Tensor], mirror: Optional[torch.Tensor] = None) -> None:
-    """x += delta (if given; float32 parts [S, N, H] are summed first); `mirror` (optional, bfloat16,
-    same shape as x) = bfloat16(x)."""
+    """x += delta (if given; float32 parts [S, N, H] are added in ascending s); `mirror` (optional,
+    bfloat16, same shape as x) = bfloat16(x)."""
     require_cuda(x, delta, mirror)
     assert x.dtype == torch.float32 and x.is_contiguous()
+    parts = 1
     if delta is not None:
+        assert delta.is_contiguous()
         if delta.dim() == 3:
-            delta = delta.sum(0)
-        assert delta.is_contiguous() and delta.shape == x.shape
+            assert delta.dtype == torch.float32 and delta.shape[1:] == x.shape
+            parts = delta.shape[0]
+        else:
+            assert delta.shape == x.shape
     if mirror is not None:
         assert mirror.dtype == torch.bfloat16 and mirror.shape == x.shape and mirror.is_contiguous()
-    call("gibbs_residual_add", ptr(x), ptr(delta), dtype_code(delta.dtype) if delta is not None else 0, ptr(mirror),
-         x.numel(), stream())
+    call("gibbs_residual_add", ptr(x), ptr(delta), dtype_code(delta.dtype) if delta is not None else 0, parts,
+         x.numel(), ptr(mirror), x.numel(), stream())
 
 
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -131,11 +135,11 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     return out
 
 
-def skinny_splits(n_out: int, inner: int, want_blocks: int = 512) -> int:
+def skinny_splits(n_out: int, inner: int, want_blocks: int = 512, features: int = 16, min_k: int = 1024) -> int:
     """How many ranges of k `gemm_skinny` should cut a product into so that at least `want_blocks`
-    workgroups run (a workgroup owns 16 output features), each with at least 1024 of k."""
-    blocks = -(-n_out // 16)
-    s = max(1, min(-(-want_blocks // blocks), inner // 1024))
+    workgroups run (a workgroup owns `features` output features), each with at least `min_k` of k."""
+    blocks = -(-n_out // features)
+    s = max(1, min(-(-want_blocks // blocks), inner // min_k))
     per = -(-(-(-inner // s)) // 128) * 128
     return -(-inner // per)
 
@@ -201,6 +205,12 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
     o = w.shape[0]
     assert stream_x.dtype == torch.float32 and stream_x.shape == (n, o) and stream_x.is_contiguous()
     assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, o) and mirror.is_contiguous()
+    if n > 32:
+        # many rows: every workgroup re-reads x_in, so workgroups take 64 features each and the chip is
+        # filled by cutting k instead; the partial sums are added to the stream by a second kernel
+        parts = gemm_skinny(x_in, w, torch.float32, skinny_splits(o, i, want_blocks=256, features=64, min_k=256))
+        residual_add(stream_x, parts if parts.dim() == 3 else parts[None], mirror)
+        return
     call("gibbs_skinny_residual", ptr(x_in), ptr(w), ptr(stream_x), ptr(mirror), n, o, i, ldx, w.stride(0), stream())
 
 
@@ -208,7 +218,7 @@ def skinny_glu(x: torch.Tensor, w_gate_up: torch.Tensor, rms_eps: Optional[float
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = silu(s x @ gate^T) * (s x @ up^T) with w_gate_up = [gate rows; up rows]."""
     n, i, ldx = _skinny_check(x, w_gate_up, "skinny_glu")
-    assert w_gate_up.shape[0] % 2 == 0 and w_gate_up.is_contiguous()
+    assert w_gate_up.shape[0] % 2 == 0
     f = w_gate_up.shape[0] // 2
     if out is None:
         out = torch.empty((n, f), dtype=torch.bfloat16, device=x.device)

@@ -25,7 +25,7 @@ class KernelError(RuntimeError):
 _SIGNATURES = {
     "gibbs_embed": [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p],
     "gibbs_add_rmsnorm": [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p],
-    "gibbs_residual_add": [c_void_p, c_void_p, c_int, c_void_p, c_long, c_void_p],
+    "gibbs_residual_add": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_long, c_void_p],
     "gibbs_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_gemm_bf16_plain": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_gemm_bf16": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],

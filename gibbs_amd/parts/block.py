@@ -13,13 +13,15 @@ into the stream, so a half of a layer is two or three kernels.
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .. import ops
-from ..ops.linear import SKINNY_ROWS
 from .base import Block, Runtime, Stream, register_arrangement
 
-FUSED_DECODE_ROWS = SKINNY_ROWS
+# rows (decoded tokens) up to which a step takes the fused decode kernels; they take at most 64
+FUSED_DECODE_ROWS = min(64, int(os.environ.get("GIBBS_FUSED_DECODE_ROWS", "64")))
 
 
 @register_arrangement("pre_norm")

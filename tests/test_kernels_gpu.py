@@ -92,7 +92,8 @@ def test_gemm_bf16(shape, out_dtype):
 
 @pytest.mark.parametrize("out_dtype", DT)
 @pytest.mark.parametrize("n,o,i,splits", [(1, 64, 128, 1), (8, 331, 1000, 1), (16, 2048, 2048, 2), (17, 200, 8192, 8),
-                                          (33, 48, 72, 1), (64, 515, 1024, 1), (5, 2048, 8192, 4), (64, 96, 4096, 3)])
+                                          (33, 48, 72, 1), (64, 515, 1024, 1), (5, 2048, 8192, 4), (64, 96, 4096, 3),
+                                          (64, 2048, 2048, 8), (40, 8200, 512, 1), (50, 1000, 4096, 16)])   # 4 tiles a workgroup
 def test_gemm_skinny(n, o, i, splits, out_dtype):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -427,7 +428,8 @@ def rms_scale(x, eps):
     return 1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
 
 
-@pytest.mark.parametrize("n,o,i", [(1, 64, 128), (8, 3072, 2048), (16, 331 * 8, 1000), (17, 200, 512), (64, 96, 4096), (5, 40, 72)])
+@pytest.mark.parametrize("n,o,i", [(1, 64, 128), (8, 3072, 2048), (16, 331 * 8, 1000), (17, 200, 512), (64, 96, 4096), (5, 40, 72),
+                                   (48, 8200, 512), (64, 3072, 2048)])      # two tiles a workgroup; many rows, one tile
 def test_skinny_store_with_rms_prologue(n, o, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=3.0), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -436,7 +438,8 @@ def test_skinny_store_with_rms_prologue(n, o, i):
     close(ops.skinny_store(x, w, rms_eps=1e-5), plain * rms_scale(x, 1e-5), torch.bfloat16, "skinny_store rms", bf16=4e-3)
 
 
-@pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96)])
+@pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96), (64, 2048, 2048),
+                                   (40, 1000, 4096)])                       # many rows: partial sums over k, then the add
 def test_skinny_residual(n, o, i):
     from gibbs_amd import ops
     y, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -448,7 +451,8 @@ def test_skinny_residual(n, o, i):
     assert torch.equal(mirror, x.to(torch.bfloat16))
 
 
-@pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024)])
+@pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024), (64, 6200, 256),
+                                   (36, 8192, 2048)])                       # two tiles a workgroup
 def test_skinny_glu(n, f, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=2.0), rnd(2 * f, i, dtype=torch.bfloat16, scale=0.05, seed=1)
@@ -495,6 +499,10 @@ def test_embed_and_residual_mirror():
     x0 = x.clone()
     ops.residual_add(x, d, mirror)
     assert torch.equal(x, x0 + d.float()) and torch.equal(mirror, x.to(torch.bfloat16))
+    parts = rnd(3, 4, 72, seed=4)                                      # float32 partial sums, added in order
+    x1 = x.clone()
+    ops.residual_add(x, parts, mirror)
+    assert torch.equal(x, ((x1 + parts[0]) + parts[1]) + parts[2]) and torch.equal(mirror, x.to(torch.bfloat16))
     out = ops.add_rmsnorm(x, None, None, 1e-5, torch.bfloat16)       # no gain
     close(out, F.rms_norm(x.double(), (72,), None, 1e-5), torch.bfloat16, "gain-free norm")
 
