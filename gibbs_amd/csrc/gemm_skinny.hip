@@ -35,13 +35,20 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
   const int k_begin = kb0 + wave * per_wave * 32;
   const int k_end = min(kb1, k_begin + per_wave * 32);
 
+  // ldw == 0: W is in tile order (pack_weight): [ceil(O/16)][ceil(I/32)][64 lanes][8], a wave's A
+  // operand 1 KB of consecutive memory
+  const bool packed = ldw == 0;
+  const int ktiles = (I + 31) / 32;
   bool row_ok[FT];
   const bf16* wrow[FT];
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     row_ok[f] = o0 + f * 16 + r < O;
-    wrow[f] = W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
+    wrow[f] = packed ? W + ((size_t)(o0 / 16 + f) * ktiles) * 512 + lane * 8
+                     : W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
   }
+  const int kstride = packed ? 512 : 32;
+  const int koff = packed ? 0 : g * 8;
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -64,7 +71,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
       const int kk = k + u * 32;
       const bool k_ok = kk + g * 8 < k_end;
 #pragma unroll
-      for (int f = 0; f < FT; ++f) a[u][f] = (row_ok[f] && k_ok) ? *(const bf16x8*)(wrow[f] + kk) : zero;
+      for (int f = 0; f < FT; ++f)
+        a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
 #pragma unroll
       for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
     }
@@ -138,14 +146,14 @@ void launch(int out, int ft, int n_out, int k_splits, hipStream_t s, const bf16*
 }
 }  // namespace
 
-// X: [N <= 64, I], W: [O, I] bfloat16.  k_splits == 1: Y [N, O] bfloat16 (out_dtype 1) or float32 (0).
+// X: [N <= 64, I], W: [O, I] bfloat16 (ldw == 0: in tile order, see the kernel).  k_splits == 1: Y [N, O] bfloat16 (out_dtype 1) or float32 (0).
 // k_splits > 1: Y is float32 [k_splits, N, O] (split stride N * ldy): partial sums over k ranges.
 GIBBS_EXPORT int gibbs_gemm_skinny(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx,
                                    long ldw, long ldy, int k_splits, hipStream_t stream) {
   GIBBS_REQUIRE(N > 0 && N <= 64 && O > 0 && I > 0, "gemm_skinny: bad sizes N=%d O=%d I=%d (N up to 64)", N, O, I);
   GIBBS_REQUIRE(I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: inner size %d and row strides (%ld, %ld) must be multiples of 8", I, ldx, ldw);
   GIBBS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_skinny: operands must be 16-byte aligned");
-  GIBBS_REQUIRE(ldx >= I && ldw >= I && ldy >= O, "gemm_skinny: row strides shorter than rows");
+  GIBBS_REQUIRE(ldx >= I && (ldw == 0 || ldw >= I) && ldy >= O, "gemm_skinny: row strides shorter than rows");
   GIBBS_REQUIRE(k_splits >= 1 && k_splits <= 1024, "gemm_skinny: %d k splits", k_splits);
   GIBBS_REQUIRE(k_splits == 1 || out_dtype == GIBBS_F32, "gemm_skinny: partial sums are float32");
   GIBBS_REQUIRE(out_dtype == GIBBS_F32 || out_dtype == GIBBS_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);

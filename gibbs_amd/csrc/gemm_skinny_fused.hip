@@ -6,6 +6,10 @@
 //   v_mfma_f32_16x16x32_bf16, the workgroup's waves splitting k and meeting in LDS, as in
 //   gemm_skinny.  On top of that:
 //
+//   packed W      W may come in MFMA-tile order (`pack_weight`: [row group][16-row tile][32-k tile][lane][8],
+//                  zero-padded): a wave's load of an A operand is then 1 KB of consecutive memory, 8 requests
+//                  of 128 bytes instead of 16 of 64, which is worth a fifth of the time of these products
+//                  (the compute unit's memory pipe is bound by requests in flight, not by bytes).
 //   prologue RMS   the rows of X are the bfloat16 mirror of the residual stream; the workgroup sums
 //                  their squares from the B operands it loads anyway and scales its outputs by
 //                  1/sqrt(mean(x^2) + eps).  The norm's gain is folded into W when weights are bound.
@@ -26,16 +30,14 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
-// (Non-temporal loads of W, meant to keep the rows of X in the L2, made the products slower: measured.)
-__device__ __forceinline__ bf16x8 load_w(const bf16* p) {
-  return *(const bf16x8*)p;
-}
-
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_GLU = 2, EPI_CONV = 3 };
 constexpr int MAX_TAPS = 8;
 
 struct FusedArgs {
   const bf16* W;
+  int packed;        // W is in tile order
+  int ktiles;        // packed: 32-k tiles per 16-row tile
+  long group_tiles;  // packed: 16-row tiles per row group
   const bf16* X;   // [N, I] bfloat16 (the mirror of the residual stream when rms)
   int N, O, I;     // O: features per row group
   long ldw, ldx;
@@ -83,8 +85,17 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     row_ok[f] = r < ROWS && o0 + f * ROWS + r < a.O;
 #pragma unroll
     for (int q = 0; q < RG; ++q)
-      wrow[f][q] = a.W + ((size_t)q * a.group_stride + (row_ok[f] ? o0 + f * ROWS + r : 0)) * a.ldw + g * 8;
+      if (a.packed) {
+        // 16-row tile of the feature tile, and this lane's place in it (8-row workgroups take half a tile)
+        const int o_tile = (o0 + f * ROWS) / 16;
+        const int in_tile = ROWS == 16 ? lane : g * 16 + ((o0 / 8) % 2) * 8 + (r % 8);
+        wrow[f][q] = a.W + (((size_t)q * a.group_tiles + o_tile) * a.ktiles) * 512 + in_tile * 8;
+      } else {
+        wrow[f][q] = a.W + ((size_t)q * a.group_stride + (row_ok[f] ? o0 + f * ROWS + r : 0)) * a.ldw + g * 8;
+      }
   }
+  const int kstride = a.packed ? 512 : 32;  // elements between a lane's A operands of consecutive MFMA steps
+  const int koff = a.packed ? 0 : g * 8;    // packed tiles are whole (zero-padded)
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -153,7 +164,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
       for (int f = 0; f < FT; ++f)
 #pragma unroll
-        for (int q = 0; q < RG; ++q) av[u][f][q] = (row_ok[f] && k_ok) ? load_w(wrow[f][q] + kk) : zero;
+        for (int q = 0; q < RG; ++q)
+          av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
 #pragma unroll
       for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
     }
@@ -338,18 +350,29 @@ int check_common(const char* what, const void* X, const void* W, int N, int O, i
   GIBBS_REQUIRE(N > 0 && N <= 64 && O > 0 && I > 0, "%s: bad sizes N=%d O=%d I=%d (N up to 64)", what, N, O, I);
   GIBBS_REQUIRE(I % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "%s: inner size %d and row strides (%ld, %ld) must be multiples of 8", what, I, ldx, ldw);
   GIBBS_REQUIRE(((uintptr_t)X % 16) == 0 && ((uintptr_t)W % 16) == 0, "%s: operands must be 16-byte aligned", what);
-  GIBBS_REQUIRE(ldx >= I && ldw >= I, "%s: row strides shorter than rows", what);
+  GIBBS_REQUIRE(ldx >= I && (ldw == 0 || ldw >= I), "%s: row strides shorter than rows", what);
   return 0;
+}
+
+// A row stride of 0 says that W is in tile order (pack_weight).
+void note_layout(FusedArgs& a) {
+  if (a.ldw != 0) return;
+  a.packed = 1;
+  a.ktiles = ceil_div(a.I, 32);
+  a.group_tiles = ceil_div(a.O, 16);
 }
 }  // namespace
 
+// In all of these, ldw == 0 means that W is in tile order: [row group][ceil(O/16)][ceil(I/32)][64 lanes][8],
+// lane (r, g) of a tile holding W[tile row * 16 + r][k tile * 32 + g * 8 .. + 8], zeros beyond O and I.
+//
 // Y[n, o] = scale_n * sum_k X[n, k] W[o, k], bfloat16 out; scale_n = 1/sqrt(mean_k X[n,k]^2 + eps) if rms.
 GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N, int O, int I, long ldx, long ldw,
                                     long ldy, int rms, float eps, hipStream_t stream) {
   if (check_common("skinny_store", X, W, N, O, I, ldx, ldw)) return 1;
   GIBBS_REQUIRE(ldy >= O, "skinny_store: output rows shorter than %d", O);
   FusedArgs a{};
-  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.Y = (bf16*)Y; a.ldy = ldy;
   if (rms) launch_nt<1, true, EPI_STORE>(a, stream);
   else launch_nt<1, false, EPI_STORE>(a, stream);
@@ -361,7 +384,7 @@ GIBBS_EXPORT int gibbs_skinny_residual(const void* X, const void* W, float* x, v
                                        long ldw, hipStream_t stream) {
   if (check_common("skinny_residual", X, W, N, O, I, ldx, ldw)) return 1;
   FusedArgs a{};
-  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx;
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; note_layout(a);
   a.x = x; a.xb = (bf16*)xb;
   launch_nt<1, false, EPI_RESIDUAL>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_residual");
@@ -373,7 +396,7 @@ GIBBS_EXPORT int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, 
   if (check_common("skinny_glu", X, W, N, F, I, ldx, ldw)) return 1;
   GIBBS_REQUIRE(ldy >= F, "skinny_glu: output rows shorter than %d", F);
   FusedArgs a{};
-  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy;
   if (rms) launch_nt<2, true, EPI_GLU>(a, stream);
   else launch_nt<2, false, EPI_GLU>(a, stream);
@@ -389,7 +412,7 @@ GIBBS_EXPORT int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N,
   GIBBS_REQUIRE(K >= 2 && K <= MAX_TAPS, "skinny_conv: kernel length %d outside 2..%d", K, MAX_TAPS);
   GIBBS_REQUIRE(slot_stride >= (long)(K - 1) * C, "skinny_conv: state slot stride %ld shorter than (K-1)*C", slot_stride);
   FusedArgs a{};
-  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = C; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps;
+  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = C; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.group_stride = C; a.Y = (bf16*)Y; a.ldy = C;
   a.taps = taps; a.bias = bias; a.state = state; a.slot_stride = slot_stride; a.slot = slot; a.ctx = ctx; a.K = K;
   if (rms) launch_conv<true>(a, stream);

@@ -135,6 +135,44 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     return out
 
 
+class PackedWeight:
+    """A matrix [groups * rows, inner] (bfloat16) in the order the few-row products read it:
+    [group][ceil(rows/16)][ceil(inner/32)][64 lanes][8], lane (r, g) of a tile holding
+    W[tile row * 16 + r][k tile * 32 + g * 8 .. + 8], zeros beyond rows and inner.  A wave's load of
+    an MFMA A operand is then 1 KB of consecutive memory (8 requests of 128 bytes instead of 16 of
+    64), which is worth a fifth of the time of a weight-streaming product.  `shape`, `dtype` and
+    `stride(0) == 0` let it stand where the row-major matrix does."""
+
+    def __init__(self, w: torch.Tensor, groups: int = 1):
+        assert w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[0] % groups == 0
+        total, inner = w.shape
+        rows = total // groups
+        rows_p, inner_p = -(-rows // 16) * 16, -(-inner // 32) * 32
+        padded = torch.zeros((groups, rows_p, inner_p), dtype=w.dtype, device=w.device)
+        padded[:, :rows, :inner] = w.reshape(groups, rows, inner)
+        tiles = padded.view(groups, rows_p // 16, 16, inner_p // 32, 4, 8).permute(0, 1, 3, 4, 2, 5)
+        self.data = tiles.contiguous()                     # [group][row tile][k tile][g][r][8]
+        self.shape, self.dtype, self.groups, self.device = (total, inner), w.dtype, groups, w.device
+
+    def dim(self) -> int:
+        return 2
+
+    def stride(self, d: int) -> int:
+        return 0 if d == 0 else 1
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    @property
+    def is_cuda(self) -> bool:
+        return self.data.is_cuda
+
+
+def _w(w) -> torch.Tensor:
+    """The tensor behind a weight operand (a row-major matrix, or a PackedWeight's tiles)."""
+    return w.data if isinstance(w, PackedWeight) else w
+
+
 def skinny_splits(n_out: int, inner: int, want_blocks: int = 512, features: int = 16, min_k: int = 1024) -> int:
     """How many ranges of k `gemm_skinny` should cut a product into so that at least `want_blocks`
     workgroups run (a workgroup owns `features` output features), each with at least `min_k` of k."""
@@ -147,8 +185,10 @@ def skinny_splits(n_out: int, inner: int, want_blocks: int = 512, features: int 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, k_splits: int = 1,
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ w^T for at most 64 rows of x, streaming w once.  k_splits > 1 returns float32
-    partial sums [k_splits, N, O] (ranges of k) for the consumer to add."""
-    require_cuda(x, w)
+    partial sums [k_splits, N, O] (ranges of k) for the consumer to add.  `w` may be a PackedWeight."""
+    require_cuda(x, _w(w))
+    if isinstance(w, PackedWeight) and w.groups != 1:
+        raise KernelError("gemm_skinny: the weights are packed in row groups")
     assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
     assert x.dim() == 2 and w.dim() == 2 and x.shape[1] == w.shape[1], (x.shape, w.shape)
     assert x.stride(1) == 1 and w.stride(1) == 1
@@ -167,13 +207,15 @@ def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch
     if out is None:
         out = torch.empty(shape, dtype=out_dtype, device=x.device)
     assert out.shape == shape and out.dtype == out_dtype and out.is_contiguous()
-    call("gibbs_gemm_skinny", ptr(x), ptr(w), ptr(out), dtype_code(out_dtype), n, o, i, ldx, w.stride(0), o, k_splits,
+    call("gibbs_gemm_skinny", ptr(x), ptr(_w(w)), ptr(out), dtype_code(out_dtype), n, o, i, ldx, w.stride(0), o, k_splits,
          stream())
     return out
 
 
-def _skinny_check(x: torch.Tensor, w: torch.Tensor, what: str) -> tuple[int, int, int]:
-    require_cuda(x, w)
+def _skinny_check(x: torch.Tensor, w, what: str, groups: int = 1) -> tuple[int, int, int]:
+    require_cuda(x, _w(w))
+    if isinstance(w, PackedWeight) and w.groups != groups:
+        raise KernelError(f"{what}: the weights are packed in {w.groups} row groups, the product reads {groups}")
     assert x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.dim() == 2 and w.dim() == 2
     assert x.shape[1] == w.shape[1] and x.stride(1) == 1 and w.stride(1) == 1, (x.shape, w.shape)
     n, i = x.shape
@@ -194,7 +236,7 @@ def skinny_store(x: torch.Tensor, w: torch.Tensor, rms_eps: Optional[float] = No
     if out is None:
         out = torch.empty((n, o), dtype=torch.bfloat16, device=x.device)
     assert out.shape == (n, o) and out.dtype == torch.bfloat16 and out.is_contiguous()
-    call("gibbs_skinny_store", ptr(x), ptr(w), ptr(out), n, o, i, ldx, w.stride(0), o, int(rms_eps is not None),
+    call("gibbs_skinny_store", ptr(x), ptr(_w(w)), ptr(out), n, o, i, ldx, w.stride(0), o, int(rms_eps is not None),
          float(rms_eps or 0.0), stream())
     return out
 
@@ -211,19 +253,19 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
         parts = gemm_skinny(x_in, w, torch.float32, skinny_splits(o, i, want_blocks=256, features=64, min_k=256))
         residual_add(stream_x, parts if parts.dim() == 3 else parts[None], mirror)
         return
-    call("gibbs_skinny_residual", ptr(x_in), ptr(w), ptr(stream_x), ptr(mirror), n, o, i, ldx, w.stride(0), stream())
+    call("gibbs_skinny_residual", ptr(x_in), ptr(_w(w)), ptr(stream_x), ptr(mirror), n, o, i, ldx, w.stride(0), stream())
 
 
 def skinny_glu(x: torch.Tensor, w_gate_up: torch.Tensor, rms_eps: Optional[float] = None,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out = silu(s x @ gate^T) * (s x @ up^T) with w_gate_up = [gate rows; up rows]."""
-    n, i, ldx = _skinny_check(x, w_gate_up, "skinny_glu")
+    n, i, ldx = _skinny_check(x, w_gate_up, "skinny_glu", groups=2)
     assert w_gate_up.shape[0] % 2 == 0
     f = w_gate_up.shape[0] // 2
     if out is None:
         out = torch.empty((n, f), dtype=torch.bfloat16, device=x.device)
     assert out.shape == (n, f) and out.dtype == torch.bfloat16 and out.is_contiguous()
-    call("gibbs_skinny_glu", ptr(x), ptr(w_gate_up), ptr(out), n, f, i, ldx, w_gate_up.stride(0), f,
+    call("gibbs_skinny_glu", ptr(x), ptr(_w(w_gate_up)), ptr(out), n, f, i, ldx, w_gate_up.stride(0), f,
          int(rms_eps is not None), float(rms_eps or 0.0), stream())
     return out
 
@@ -233,10 +275,10 @@ def skinny_conv(x: torch.Tensor, w_in: torch.Tensor, taps: torch.Tensor, bias: O
                 out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """In-projection and gated short convolution for a step of decoded tokens (row n is one token of
     the request in slot[n] with ctx[n] cached positions): w_in = [B rows; C rows; x rows]."""
-    n, i, ldx = _skinny_check(x, w_in, "skinny_conv")
+    n, i, ldx = _skinny_check(x, w_in, "skinny_conv", groups=3)
     require_cuda(taps, bias, state, slot, ctx)
     c, k = taps.shape
-    assert w_in.shape[0] == 3 * c and w_in.is_contiguous()
+    assert w_in.shape[0] == 3 * c
     assert taps.dtype == torch.float32 and taps.is_contiguous()
     assert bias is None or (bias.dtype == torch.float32 and bias.shape == (c,) and bias.is_contiguous())
     assert state.dtype == torch.float32 and state.shape[1:] == (k - 1, c) and state.stride(2) == 1 and state.stride(1) == c
@@ -246,7 +288,7 @@ def skinny_conv(x: torch.Tensor, w_in: torch.Tensor, taps: torch.Tensor, bias: O
     if out is None:
         out = torch.empty((n, c), dtype=torch.bfloat16, device=x.device)
     assert out.shape == (n, c) and out.dtype == torch.bfloat16 and out.is_contiguous()
-    call("gibbs_skinny_conv", ptr(x), ptr(w_in), ptr(out), n, c, i, ldx, w_in.stride(0), int(rms_eps is not None),
+    call("gibbs_skinny_conv", ptr(x), ptr(_w(w_in)), ptr(out), n, c, i, ldx, w_in.stride(0), int(rms_eps is not None),
          float(rms_eps or 0.0), ptr(taps), ptr(bias), ptr(state), state.stride(0), ptr(slot), ptr(ctx), k, stream())
     return out
 

@@ -14,7 +14,7 @@ from typing import Optional
 
 import torch
 
-from . import gemm_bf16, gemm_bf16_plain, gemm_f32, gemm_skinny, skinny_splits
+from . import PackedWeight, gemm_bf16, gemm_bf16_plain, gemm_f32, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
 # rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
@@ -24,10 +24,11 @@ USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
-           partial_ok: bool = False) -> torch.Tensor:
+           partial_ok: bool = False, packed: Optional[PackedWeight] = None) -> torch.Tensor:
     """`partial_ok`: the caller can take float32 partial sums [S, N, O] (to be added in order)
     instead of the finished product; the few-row kernel then also splits k over workgroups when
-    the output alone is too narrow to fill the chip."""
+    the output alone is too narrow to fill the chip.  `packed`: the same matrix in the order the
+    few-row kernel reads fastest, used when that kernel is the one that runs."""
     require_cuda(x, w)
     if x.dtype != w.dtype:
         raise KernelError(f"linear: activations are {x.dtype}, weights {w.dtype}")
@@ -42,7 +43,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
             return gemm_bf16_plain(x, w, out_dtype)             # what the matrix-core kernels refuse
         if 1 <= x.shape[0] <= SKINNY_ROWS:
             splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
-            return gemm_skinny(x, w, out_dtype, splits)
+            return gemm_skinny(x, w if packed is None else packed, out_dtype, splits)
         if USE_LIBRARY_GEMM and out_dtype == torch.bfloat16:
             return torch.matmul(x, w.t())
         return gemm_bf16(x, w, out_dtype)

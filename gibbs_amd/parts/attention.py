@@ -70,6 +70,7 @@ class AttentionMixer(Mixer):
         else:
             self.w_qkv = weights[t["q_proj"]]
         self.w_out = weights[t["out_proj"]]
+        self.p_qkv = self.p_out = None
         self.q_gain = weights[t["q_norm"]] if self.qk_norm else None
         self.k_gain = weights[t["k_norm"]] if self.qk_norm and self.source is None else None
         if self.position is not None:
@@ -86,6 +87,10 @@ class AttentionMixer(Mixer):
         """The preceding norm's gain, multiplied into the columns of the q, k, v projections."""
         self.w_qkv = (self.w_qkv.float() * gain[None, :]).to(self.w_qkv.dtype)
 
+    def pack_matrices(self) -> None:
+        self.p_qkv = ops.PackedWeight(self.w_qkv)
+        self.p_out = ops.PackedWeight(self.w_out)
+
     def can_decode_fused(self, batch) -> bool:
         rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
         return (self.source is None and self.hidden % 8 == 0 and self.head_dim % 16 == 0 and self.head_dim <= 256
@@ -95,8 +100,8 @@ class AttentionMixer(Mixer):
         """norm -> q, k, v in one kernel; q/k norm, rotation, the write of the new key and value and
         attention over split keys in a second (and the merge of the slices); out_proj + residual
         add in a third."""
-        qkv = ops.skinny_store(stream.mirror, self.w_qkv, rms_eps=norm_eps)
-        ops.skinny_residual(self._attend_decoded(qkv, batch, cache), self.w_out, stream.x, stream.mirror)
+        qkv = ops.skinny_store(stream.mirror, self.p_qkv or self.w_qkv, rms_eps=norm_eps)
+        ops.skinny_residual(self._attend_decoded(qkv, batch, cache), self.p_out or self.w_out, stream.x, stream.mirror)
 
     def _attend_decoded(self, qkv, batch, cache) -> torch.Tensor:
         """A step of single decoded tokens, from the raw projection: one kernel norms and rotates q and
@@ -118,7 +123,7 @@ class AttentionMixer(Mixer):
         rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
         if (owns and self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and self.head_dim % 16 == 0
                 and self.head_dim <= 256 and rot_ok):
-            return linear(self._attend_decoded(qkv, batch, cache), self.w_out, partial_ok=True)
+            return linear(self._attend_decoded(qkv, batch, cache), self.w_out, partial_ok=True, packed=self.p_out)
         pos = self.position
         ops.qk_rope_kv(qkv, n, self.heads, self.kv_heads if owns else 0, self.head_dim,
                        q_gain=self.q_gain, k_gain=self.k_gain, eps=self.qk_norm_eps,
@@ -129,7 +134,7 @@ class AttentionMixer(Mixer):
                        kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None,
                        table=table, n_req=batch.n_req, cos_sin=None if pos is None else pos.cos_sin)
         a = self.attend(qkv, batch, cache, table)
-        return linear(a, self.w_out, partial_ok=True)
+        return linear(a, self.w_out, partial_ok=True, packed=self.p_out)
 
     def attend(self, qkv, batch, cache, table) -> torch.Tensor:
         """Attention of the step's rows over the cache.  bfloat16: rows that are all single decoded

@@ -66,6 +66,10 @@ class Part:
         """Gains, biases, taps and tables that a step also reads."""
         return []
 
+    def pack_matrices(self) -> None:
+        """Called once the matrices have their final values (gains folded in): a part may keep
+        copies in the order its few-row kernels read fastest (`ops.PackedWeight`)."""
+
 
 class Norm(Part):
     def __init__(self, spec: NormSpec, width: int):

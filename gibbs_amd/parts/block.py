@@ -30,6 +30,9 @@ class PreNormBlock(Block):
         super().bind(weights, rt)
         self.mixer_folded = self._fold(self.mixer_norm, self.mixer)
         self.ffn_folded = self._fold(self.ffn_norm, self.ffn)
+        if self.rt.act_dtype == torch.bfloat16:
+            self.mixer.pack_matrices()
+            self.ffn.pack_matrices()
 
     def _fold(self, norm, part) -> bool:
         if self.rt.act_dtype != torch.bfloat16:

@@ -32,6 +32,7 @@ class GluFeedForward(FeedForward):
         t = self.spec.tensors
         self.w_gate_up = torch.cat([weights[t["gate"]], weights[t["up"]]], dim=0).contiguous()
         self.w_down = weights[t["down"]]
+        self.p_gate_up = self.p_down = None
 
     def matrices(self):
         return [self.w_gate_up, self.w_down]
@@ -40,14 +41,18 @@ class GluFeedForward(FeedForward):
         """The preceding norm's gain, multiplied into the columns of the gate and up matrices."""
         self.w_gate_up = (self.w_gate_up.float() * gain[None, :]).to(self.w_gate_up.dtype)
 
+    def pack_matrices(self) -> None:
+        self.p_gate_up = ops.PackedWeight(self.w_gate_up, groups=2)
+        self.p_down = ops.PackedWeight(self.w_down)
+
     def can_decode_fused(self, batch) -> bool:
         return self.hidden % 8 == 0 and self.inter % 8 == 0
 
     def decode_fused(self, stream, norm_eps: float, batch) -> None:
         """norm -> gate/up -> activation in one kernel, down + residual add in another."""
-        act = ops.skinny_glu(stream.mirror, self.w_gate_up, rms_eps=norm_eps)
-        ops.skinny_residual(act, self.w_down, stream.x, stream.mirror)
+        act = ops.skinny_glu(stream.mirror, self.p_gate_up or self.w_gate_up, rms_eps=norm_eps)
+        ops.skinny_residual(act, self.p_down or self.w_down, stream.x, stream.mirror)
 
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         gu = linear(h, self.w_gate_up)
-        return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True)
+        return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True, packed=self.p_down)

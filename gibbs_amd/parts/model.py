@@ -70,6 +70,7 @@ class DecoderModel(Part):
         self.rt = rt
         self.table = weights[self.spec.embedding]
         self.head = weights[self.spec.head] if self.spec.head is not None else self.table
+        self.head_packed = ops.PackedWeight(self.head) if rt.act_dtype == torch.bfloat16 else None
         self.final_norm.bind(weights, rt)
         for b in self.blocks:
             b.bind(weights, rt)
@@ -89,4 +90,4 @@ class DecoderModel(Part):
         if batch.n_logits == 0:
             return None
         h = self.final_norm.forward(stream.x, stream.pending, batch.logit_rows, batch.n_logits)
-        return linear(h, self.head, out_dtype=torch.float32)
+        return linear(h, self.head, out_dtype=torch.float32, packed=self.head_packed)

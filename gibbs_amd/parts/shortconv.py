@@ -49,6 +49,7 @@ class ShortConvMixer(Mixer):
         self.w_in = weights[t["in_proj"]]
         self.taps = weights[t["conv"]].reshape(self.width, self.kernel).contiguous()
         self.w_out = weights[t["out_proj"]]
+        self.p_in = self.p_out = None
         self.conv_bias = weights[t["conv_bias"]] if self.bias else None
 
     def matrices(self):
@@ -64,15 +65,19 @@ class ShortConvMixer(Mixer):
     def can_decode_fused(self, batch) -> bool:
         return self.hidden % 8 == 0 and self.width % 8 == 0 and self.kernel <= 8
 
+    def pack_matrices(self) -> None:
+        self.p_in = ops.PackedWeight(self.w_in, groups=3)
+        self.p_out = ops.PackedWeight(self.w_out)
+
     def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
         """norm -> in_proj -> gated convolution with its state in one kernel, out_proj + residual
         add in another."""
-        y = ops.skinny_conv(stream.mirror, self.w_in, self.taps, self.conv_bias, cache.states[STATE], batch.slot,
+        y = ops.skinny_conv(stream.mirror, self.p_in or self.w_in, self.taps, self.conv_bias, cache.states[STATE], batch.slot,
                             batch.ctx, rms_eps=norm_eps)
-        ops.skinny_residual(y, self.w_out, stream.x, stream.mirror)
+        ops.skinny_residual(y, self.p_out or self.w_out, stream.x, stream.mirror)
 
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         bcx = linear(h, self.w_in)
         y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,
                           batch.n_rows, batch.n_req)
-        return linear(y, self.w_out, partial_ok=True)
+        return linear(y, self.w_out, partial_ok=True, packed=self.p_out)

@@ -113,6 +113,25 @@ def test_gemm_skinny(n, o, i, splits, out_dtype):
           f32=2e-5, bf16=4e-3)
 
 
+def test_packed_weight_layout():
+    """[group][16-row tile][32-k tile][lane = g * 16 + r][8] with zeros beyond the matrix."""
+    from gibbs_amd import ops
+    w = rnd(2 * 40, 72, dtype=torch.bfloat16)
+    p = ops.PackedWeight(w, groups=2)
+    assert p.shape == (80, 72) and p.stride(0) == 0 and tuple(p.data.shape) == (2, 3, 3, 4, 16, 8)
+    for q, ot, kt, g, r in [(0, 0, 0, 0, 0), (1, 2, 1, 3, 7), (0, 1, 2, 0, 15), (1, 0, 2, 1, 3)]:
+        row, k = ot * 16 + r, kt * 32 + g * 8
+        want = torch.zeros(8, dtype=torch.bfloat16, device=DEV)
+        if row < 40 and k < 72:
+            want[:min(8, 72 - k)] = w[q * 40 + row, k:k + 8]
+        assert torch.equal(p.data[q, ot, kt, g, r], want), (q, ot, kt, g, r)
+    x = rnd(5, 72, dtype=torch.bfloat16, seed=2)
+    for splits in (1, 2):
+        w1 = rnd(50, 256, dtype=torch.bfloat16, seed=3)
+        x1 = rnd(5, 256, dtype=torch.bfloat16, seed=4)
+        assert torch.equal(ops.gemm_skinny(x1, ops.PackedWeight(w1), torch.float32, splits), ops.gemm_skinny(x1, w1, torch.float32, splits))
+
+
 def test_skinny_splits_cover_k():
     from gibbs_amd import ops
     for o, i in [(2048, 2048), (2048, 8192), (6144, 2048), (65536, 2048), (96, 96), (200, 1000), (64, 12800)]:
@@ -435,7 +454,9 @@ def test_skinny_store_with_rms_prologue(n, o, i):
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=3.0), rnd(o, i, dtype=torch.bfloat16, seed=1)
     plain = x.double() @ w.double().t()
     close(ops.skinny_store(x, w), plain, torch.bfloat16, "skinny_store", bf16=4e-3)
-    close(ops.skinny_store(x, w, rms_eps=1e-5), plain * rms_scale(x, 1e-5), torch.bfloat16, "skinny_store rms", bf16=4e-3)
+    got = ops.skinny_store(x, w, rms_eps=1e-5)
+    close(got, plain * rms_scale(x, 1e-5), torch.bfloat16, "skinny_store rms", bf16=4e-3)
+    assert torch.equal(ops.skinny_store(x, ops.PackedWeight(w), rms_eps=1e-5), got), "tile-ordered weights: same sums"
 
 
 @pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96), (64, 2048, 2048),
@@ -446,9 +467,12 @@ def test_skinny_residual(n, o, i):
     x = rnd(n, o, scale=2.0, seed=2)
     want = x.double() + y.double() @ w.double().t()
     mirror = torch.zeros(n, o, dtype=torch.bfloat16, device=DEV)
+    x0 = x.clone()
     ops.skinny_residual(y, w, x, mirror)
     close(x, want, torch.float32, "skinny_residual", f32=2e-5)
     assert torch.equal(mirror, x.to(torch.bfloat16))
+    ops.skinny_residual(y, ops.PackedWeight(w), x0, mirror)
+    assert torch.equal(x0, x), "tile-ordered weights: same sums"
 
 
 @pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024), (64, 6200, 256),
@@ -458,7 +482,11 @@ def test_skinny_glu(n, f, i):
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=2.0), rnd(2 * f, i, dtype=torch.bfloat16, scale=0.05, seed=1)
     gu = (x.double() @ w.double().t()) * rms_scale(x, 1e-6)
     want = F.silu(gu[:, :f]) * gu[:, f:]
-    close(ops.skinny_glu(x, w, rms_eps=1e-6), want, torch.bfloat16, "skinny_glu", bf16=6e-3)
+    got = ops.skinny_glu(x, w, rms_eps=1e-6)
+    close(got, want, torch.bfloat16, "skinny_glu", bf16=6e-3)
+    assert torch.equal(ops.skinny_glu(x, ops.PackedWeight(w, groups=2), rms_eps=1e-6), got), "tile-ordered weights: same sums"
+    with pytest.raises(ops.KernelError, match="row groups"):
+        ops.skinny_glu(x, ops.PackedWeight(w), rms_eps=1e-6)
 
 
 @pytest.mark.parametrize("n,c,i,k,bias", [(1, 2048, 2048, 3, False), (8, 72, 96, 4, True), (20, 40, 64, 2, True), (64, 96, 128, 3, False)])
@@ -471,8 +499,10 @@ def test_skinny_conv(n, c, i, k, bias):
     slots = torch.randperm(n + 3)[:n].to(torch.int32).to(DEV)
     ctx = i32([j % (k + 1) for j in range(n)])             # 0 (fresh), shorter than the history, longer
     state = rnd(n + 3, k - 1, c, seed=6)
-    state2 = state.clone()
+    state2, state3 = state.clone(), state.clone()
     y = ops.skinny_conv(x, w, taps, b, state, slots, ctx, rms_eps=1e-5)
+    y3 = ops.skinny_conv(x, ops.PackedWeight(w, groups=3), taps, b, state3, slots, ctx, rms_eps=1e-5)
+    assert torch.equal(y3, y) and torch.equal(state3, state), "tile-ordered weights: same sums"
     bcx = (x.double() @ w.double().t()) * rms_scale(x, 1e-5)
     B, C, X = bcx[:, :c], bcx[:, c:2 * c], bcx[:, 2 * c:]
     bx = B * X
