@@ -154,7 +154,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  constexpr int U = (FT * RG * NT >= 6) ? 2 : 4;  // MFMA steps per iteration
+  constexpr int U = (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);  // MFMA steps per iteration
   for (int k = k_begin; k < k_end; k += 32 * U) {
     bf16x8 av[U][FT][RG], bv[U][NT];
 #pragma unroll
