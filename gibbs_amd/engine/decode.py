@@ -20,6 +20,11 @@ from .batch import StepBatch
 from .engine import Engine, OutOfPages, StepError
 
 
+# steps per launch of the longer captured graph (a launch costs the host and the queue about as much
+# as four kernels of a step)
+UNROLL = 8
+
+
 class DecodeLoop:
     def __init__(self, engine: Engine, rids: Sequence[Hashable], last_tokens: Sequence[int],
                  params: Optional[Sequence[SamplingParams]] = None, use_graph: bool = True,
@@ -33,7 +38,8 @@ class DecodeLoop:
             raise StepError("a decode loop needs at least one request")
         self.use_graph = use_graph
         self.capacity = max_steps
-        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.graph: Optional[torch.cuda.CUDAGraph] = None          # one step
+        self.graph_many: Optional[torch.cuda.CUDAGraph] = None     # UNROLL steps: fewer launches from the host
         self._allocate(params)
         self.rebind(rids, last_tokens, params, first_index)
 
@@ -168,7 +174,19 @@ class DecodeLoop:
             with torch.cuda.graph(g):
                 self._step()
             self.graph = g                                  # the capture itself ran nothing
-        for _ in range(n_steps):
+        left = n_steps
+        if self.graph is not None and left >= UNROLL:
+            if self.graph_many is None:
+                g = torch.cuda.CUDAGraph()
+                torch.cuda.synchronize()
+                with torch.cuda.graph(g):
+                    for _ in range(UNROLL):
+                        self._step()
+                self.graph_many = g
+            while left >= UNROLL:
+                self.graph_many.replay()
+                left -= UNROLL
+        for _ in range(left):
             if self.graph is not None:
                 self.graph.replay()
             else:
