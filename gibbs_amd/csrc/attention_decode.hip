@@ -74,6 +74,7 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
   __shared__ float s_ml[NW][GT][2];
   __shared__ float s_acc[NW][GT][MAX_HD];
   __shared__ float s_knew[MAX_HD], s_vnew[MAX_HD];
+  __shared__ float s_q[GT][MAX_HD];
   __shared__ int s_pages[SEG_PAGES];
 
   const int row = blockIdx.x;
@@ -101,12 +102,14 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
   // Everything that does not hang on earlier arithmetic is asked for first: the query heads, the
   // row's own key and value, the page ids of the slice's first segment (kept in registers until
   // the prologue below is through, then put into LDS).
+  // (query head g is prepared by wave g % NW alone and handed to the others through LDS)
   uint4 qraw[GT];
 #pragma unroll
   for (int g = 0; g < GT; ++g)
-    qraw[g] = (g < gcount && active) ? *(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0) : make_uint4(0, 0, 0, 0);
+    qraw[g] = (g < gcount && g % NW == wave && active) ? *(const uint4*)(qrow + (size_t)(kvh * G + g0 + g) * hd + e0)
+                                                       : make_uint4(0, 0, 0, 0);
   const bool has_new = RAW && p >= k0 && p < k1;  // raw rows: this slice holds the row's own position
-  const bool new_lane = has_new && wave == 0 && grp == 0;
+  const bool new_lane = has_new && wave == NW - 1 && grp == 0;  // the last wave has the fewest query heads to prepare
   uint4 knew_raw = make_uint4(0, 0, 0, 0), vnew_raw = make_uint4(0, 0, 0, 0);
   if (new_lane && active) {
     knew_raw = *(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0);
@@ -125,7 +128,8 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
   Rot8 rt;
   if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p, a.cs_table, a.table_len);
   const bool rotate = a.inv_freq != nullptr;
-  // raw rows: the row's own key and value; wave 0's first LPK lanes prepare them for everyone
+  // raw rows: the row's own key and value; the last wave's first LPK lanes prepare them for everyone
+  uint32_t kw[4] = {0, 0, 0, 0}, vw[4] = {0, 0, 0, 0};  // the new key and value as they go to their page
   if (new_lane) {
     float kf[EPL], vf[EPL];
     unpack8(knew_raw, kf);
@@ -133,7 +137,6 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
     norm_rope8<LPK>(kf, e0, hd, a.k_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
     if (active) {
       // what later steps read from the page is the bfloat16 value: use the same value now
-      uint32_t kw[4], vw[4];
 #pragma unroll
       for (int i = 0; i < EPL; ++i) {
         const bf16 kb = (bf16)kf[i];
@@ -143,14 +146,6 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
         const uint32_t kbits = __float_as_uint(kf[i]) >> 16, vbits = __float_as_uint(vf[i]) >> 16;
         if (i % 2 == 0) { kw[i / 2] = kbits; vw[i / 2] = vbits; }
         else { kw[i / 2] |= kbits << 16; vw[i / 2] |= vbits << 16; }
-      }
-      if (hc == 0) {
-        const int page = table[p / a.page_size];
-        if (page >= 0 && page < a.num_pages) {
-          const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + p % a.page_size) * hd + e0;
-          *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
-          *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
-        }
       }
     }
   }
@@ -163,15 +158,18 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
     l[g] = 0.f;
 #pragma unroll
     for (int i = 0; i < EPL; ++i) { acc[g][i] = 0.f; qf[g][i] = 0.f; }
-    if (g < gcount) {
-      unpack8(qraw[g], qf[g]);
+    if (g < gcount && g % NW == wave) {
+      float qv[EPL];
+      unpack8(qraw[g], qv);
       if (RAW) {
-        norm_rope8<LPK>(qf[g], e0, hd, a.q_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
+        norm_rope8<LPK>(qv, e0, hd, a.q_gain, a.eps, rotate, rt, a.rot, a.variant, lane);
 #pragma unroll
-        for (int i = 0; i < EPL; ++i) qf[g][i] = (float)(bf16)qf[g][i];   // q is bfloat16 where it is stored
+        for (int i = 0; i < EPL; ++i) qv[i] = (float)(bf16)qv[i];   // q is bfloat16 where it is stored
       }
+      if (grp == 0 && active) {
 #pragma unroll
-      for (int i = 0; i < EPL; ++i) qf[g][i] *= a.scale;
+        for (int i = 0; i < EPL; ++i) s_q[g][e0 + i] = qv[i] * a.scale;
+      }
     }
   }
 
@@ -187,15 +185,32 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
       const int j = threadIdx.x + i * NW * WAVE;
       if (j < SEG_PAGES && (first_page + j) * a.page_size < seg1) {
         const int page = seg0 == k0 ? pre_page[i] : table[first_page + j];
-        s_pages[j] = page < 0 ? 0 : (page >= a.num_pages ? a.num_pages - 1 : page);  // never read outside the pool
+        s_pages[j] = page;
       }
     }
-    __syncthreads();  // the ids, and at the first segment the row's own key and value, are in LDS
+    __syncthreads();  // the ids, and at the first segment the queries and the row's own key and value, are in LDS
+    if (seg0 == k0) {
+#pragma unroll
+      for (int g = 0; g < GT; ++g)
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) qf[g][i] = (g < gcount && active) ? s_q[g][e0 + i] : 0.f;
+    }
+    if (new_lane && hc == 0 && active && p >= seg0 && p < seg1) {
+      // the row's own key and value go to their page (its id has just been staged)
+      const int lp = a.page_shift >= 0 ? p >> a.page_shift : p / a.page_size;
+      const int page = s_pages[lp - first_page];
+      if (page >= 0 && page < a.num_pages) {   // the host never asks for another; never write outside
+        const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + (p - lp * a.page_size)) * hd + e0;
+        *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
+        *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
+      }
+    }
     auto fetch = [&](int key, uint4& kr, uint4& vr) {
       kr = vr = make_uint4(0, 0, 0, 0);
       if (key < seg1 && !(RAW && key == p) && active) {
         const int lp = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
-        const size_t off = (((size_t)s_pages[lp - first_page] * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
+        const int page = min(max(s_pages[lp - first_page], 0), a.num_pages - 1);  // never read outside the pool
+        const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
         kr = *(const uint4*)(kpages + off);
         vr = *(const uint4*)(vpages + off);
       }
