@@ -66,7 +66,7 @@ __device__ __forceinline__ void fold(float& ma, float& la, float* aa, float mb, 
 }
 
 template <int LPK, int GT, bool RAW, int NW>
-__global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
+__global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
                                                                bf16* __restrict__ vpages, float* __restrict__ partial,
                                                                bf16* __restrict__ out, DecodeArgs a) {
   constexpr int KPW = WAVE / LPK;
@@ -129,7 +129,6 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
   if (RAW) rt = rotation8(e0, a.inv_freq, a.rot, a.variant, p, a.cs_table, a.table_len);
   const bool rotate = a.inv_freq != nullptr;
   // raw rows: the row's own key and value; the last wave's first LPK lanes prepare them for everyone
-  uint32_t kw[4] = {0, 0, 0, 0}, vw[4] = {0, 0, 0, 0};  // the new key and value as they go to their page
   if (new_lane) {
     float kf[EPL], vf[EPL];
     unpack8(knew_raw, kf);
@@ -143,9 +142,6 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
         kf[i] = (float)kb;
         s_knew[e0 + i] = kf[i];
         s_vnew[e0 + i] = vf[i];
-        const uint32_t kbits = __float_as_uint(kf[i]) >> 16, vbits = __float_as_uint(vf[i]) >> 16;
-        if (i % 2 == 0) { kw[i / 2] = kbits; vw[i / 2] = vbits; }
-        else { kw[i / 2] |= kbits << 16; vw[i / 2] |= vbits << 16; }
       }
     }
   }
@@ -200,6 +196,13 @@ __global__ __launch_bounds__(NW * WAVE) void attention_decode_kernel(const bf16*
       const int lp = a.page_shift >= 0 ? p >> a.page_shift : p / a.page_size;
       const int page = s_pages[lp - first_page];
       if (page >= 0 && page < a.num_pages) {   // the host never asks for another; never write outside
+        // (both are bfloat16 values held as float: the upper 16 bits are the element)
+        uint32_t kw[4], vw[4];
+#pragma unroll
+        for (int i = 0; i < EPL; i += 2) {
+          kw[i / 2] = (__float_as_uint(s_knew[e0 + i]) >> 16) | (__float_as_uint(s_knew[e0 + i + 1]) & 0xffff0000u);
+          vw[i / 2] = (__float_as_uint(s_vnew[e0 + i]) >> 16) | (__float_as_uint(s_vnew[e0 + i + 1]) & 0xffff0000u);
+        }
         const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + (p - lp * a.page_size)) * hd + e0;
         *(uint4*)(kpages + off) = make_uint4(kw[0], kw[1], kw[2], kw[3]);
         *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);

@@ -23,7 +23,17 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
                                                           void* __restrict__ Yv, int N, int O, int I, long ldw,
                                                           long ldx, long ldy, int k_per_block, long split_stride) {
   static_assert(FT <= WAVES, "wave f finishes tile f");
-  __shared__ floatx4 red[WAVES][FT][NT][WAVE];
+  // More than 16 rows of X: a wave brings its part of X in through LDS (its own region: no barrier),
+  // 128 contiguous bytes or more of a row per request instead of the 64 that a lane group of an MFMA
+  // operand covers; see gemm_skinny_fused.
+  constexpr bool STAGE = NT >= 2;
+  constexpr int U = FT * NT >= 8 ? 2 : 4;     // MFMA steps per iteration: U * FT loads of W in flight per lane
+  constexpr int CH = 4 * U;                   // 16-byte chunks of a row per iteration
+  constexpr int RED_BYTES = WAVES * FT * NT * WAVE * 16;
+  constexpr int STAGE_BYTES = STAGE ? WAVES * NT * 16 * CH * 16 : 0;
+  __shared__ __attribute__((aligned(16))) char smem[RED_BYTES > STAGE_BYTES ? RED_BYTES : STAGE_BYTES];
+  floatx4 (*red)[FT][NT][WAVE] = reinterpret_cast<floatx4 (*)[FT][NT][WAVE]>(smem);
+  bf16x8* stage = reinterpret_cast<bf16x8*>(smem) + (size_t)(threadIdx.x / WAVE) * NT * 16 * CH;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
   const int o0 = blockIdx.x * 16 * FT;
@@ -63,18 +73,61 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
     for (int t = 0; t < NT; ++t) acc[f][t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  constexpr int U = FT * NT >= 8 ? 2 : 4;  // MFMA steps per iteration: U * FT loads of W in flight per lane
+  constexpr int RPI = WAVE / CH;              // rows per staging load
+  constexpr int LPT = 16 / RPI;               // staging loads per tile of 16 rows
+  const bf16* srow[NT][LPT];
+  bool s_ok[NT][LPT];
+  int s_chunk[LPT];
+  int read_slot[U];
+  if (STAGE) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int row = i * RPI + lane / CH;
+      s_chunk[i] = (lane % CH + row * U / 4) % CH;   // rotated so that the operand reads do not collide
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        s_ok[t][i] = t * 16 + row < N;
+        srow[t][i] = X + (size_t)(s_ok[t][i] ? t * 16 + row : 0) * ldx + s_chunk[i] * 8;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) read_slot[u] = r * CH + ((u * 4 + g - r * U / 4) & (CH - 1));
+  }
   for (int k = k_begin; k < k_end; k += 32 * U) {
     bf16x8 a[U][FT], b[U][NT];
+    if (STAGE) {
+      bf16x8 sv[NT][LPT];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = k + u * 32;
-      const bool k_ok = kk + g * 8 < k_end;
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int f = 0; f < FT; ++f)
-        a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
+        for (int i = 0; i < LPT; ++i)
+          sv[t][i] = (s_ok[t][i] && k + s_chunk[i] * 8 < k_end) ? *(const bf16x8*)(srow[t][i] + k) : zero;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+      for (int u = 0; u < U; ++u) {
+        const int kk = k + u * 32;
+#pragma unroll
+        for (int f = 0; f < FT; ++f)
+          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) stage[(t * LPT + i) * WAVE + lane] = sv[t][i];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) b[u][t] = stage[t * 16 * CH + read_slot[u]];
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kk = k + u * 32;
+        const bool k_ok = kk + g * 8 < k_end;
+#pragma unroll
+        for (int f = 0; f < FT; ++f)
+          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -84,6 +137,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
         for (int t = 0; t < NT; ++t)
           acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][f], b[u][t], acc[f][t], 0, 0, 0);
   }
+  if (STAGE) __syncthreads();  // the staging regions become the reduction buffer
 
   // the waves' sums meet in LDS; wave f adds those of tile f in the order of the waves
 #pragma unroll

@@ -67,7 +67,17 @@ struct FusedArgs {
 template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
   static_assert(FT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only");
-  __shared__ floatx4 red[WAVES][FT][RG][NT][WAVE];
+  // More than 16 rows of X: a wave brings its part of X in through LDS, 128 contiguous bytes or more of
+  // a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory pipe
+  // of a compute unit is bound by requests in flight).  The wave's region is its own: no barrier.
+  constexpr bool STAGE = NT >= 2;
+  constexpr int U = (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);  // MFMA steps per iteration
+  constexpr int CH = 4 * U;                    // 16-byte chunks of a row per iteration
+  constexpr int RED_BYTES = WAVES * FT * RG * NT * WAVE * 16;
+  constexpr int STAGE_BYTES = STAGE ? WAVES * NT * 16 * CH * 16 : 0;
+  __shared__ __attribute__((aligned(16))) char smem[RED_BYTES > STAGE_BYTES ? RED_BYTES : STAGE_BYTES];
+  floatx4 (*red)[FT][RG][NT][WAVE] = reinterpret_cast<floatx4 (*)[FT][RG][NT][WAVE]>(smem);
+  bf16x8* stage = reinterpret_cast<bf16x8*>(smem) + (size_t)(threadIdx.x / WAVE) * NT * 16 * CH;
   __shared__ float red_ss[WAVES][NT][16];
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
@@ -154,20 +164,67 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  constexpr int U = (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);  // MFMA steps per iteration
+  // staging: lane l of load instruction i brings chunk (l % CH + rot) % CH of row i * (64 / CH) + l / CH to
+  // slot i * 64 + l; rot(row) = row * U / 4 makes the operand reads below free of bank conflicts
+  constexpr int RPI = WAVE / CH;               // rows per load instruction
+  constexpr int LPT = 16 / RPI;                // load instructions per tile of 16 rows
+  const bf16* srow[NT][LPT];
+  bool s_ok[NT][LPT];
+  int s_chunk[LPT];
+  int read_slot[U];
+  if (STAGE) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int row = i * RPI + lane / CH;
+      s_chunk[i] = (lane % CH + row * U / 4) % CH;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        s_ok[t][i] = t * 16 + row < a.N;
+        srow[t][i] = a.X + (size_t)(s_ok[t][i] ? t * 16 + row : 0) * a.ldx + s_chunk[i] * 8;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) read_slot[u] = r * CH + ((u * 4 + g - r * U / 4) & (CH - 1));
+  }
   for (int k = k_begin; k < k_end; k += 32 * U) {
     bf16x8 av[U][FT][RG], bv[U][NT];
+    if (STAGE) {
+      bf16x8 sv[NT][LPT];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = k + u * 32;
-      const bool k_ok = kk + g * 8 < k_end;
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int f = 0; f < FT; ++f)
+        for (int i = 0; i < LPT; ++i)
+          sv[t][i] = (s_ok[t][i] && k + s_chunk[i] * 8 < k_end) ? *(const bf16x8*)(srow[t][i] + k) : zero;
 #pragma unroll
-        for (int q = 0; q < RG; ++q)
-          av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
+      for (int u = 0; u < U; ++u) {
+        const int kk = k + u * 32;
 #pragma unroll
-      for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+        for (int f = 0; f < FT; ++f)
+#pragma unroll
+          for (int q = 0; q < RG; ++q)
+            av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
+      }
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int i = 0; i < LPT; ++i) stage[(t * LPT + i) * WAVE + lane] = sv[t][i];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int t = 0; t < NT; ++t) bv[u][t] = stage[t * 16 * CH + read_slot[u]];
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kk = k + u * 32;
+        const bool k_ok = kk + g * 8 < k_end;
+#pragma unroll
+        for (int f = 0; f < FT; ++f)
+#pragma unroll
+          for (int q = 0; q < RG; ++q)
+            av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
+      }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
@@ -187,6 +244,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
             acc[f][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][f][q], bv[u][t], acc[f][q][t], 0, 0, 0);
       }
   }
+  if (STAGE) __syncthreads();  // the staging regions become the reduction buffer
 
   // sum of squares of row n = t*16 + r: over the 4 lane groups, then over the waves
   if (RMS) {

@@ -2,6 +2,7 @@
 what the kernel and its grid assume, then queues the kernel on the current stream."""
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -247,7 +248,7 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
     o = w.shape[0]
     assert stream_x.dtype == torch.float32 and stream_x.shape == (n, o) and stream_x.is_contiguous()
     assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, o) and mirror.is_contiguous()
-    if n > 32:
+    if n > 32 and not os.environ.get("GIBBS_RESIDUAL_DIRECT"):
         # many rows: every workgroup re-reads x_in, so workgroups take 64 features each and the chip is
         # filled by cutting k instead; the partial sums are added to the stream by a second kernel
         parts = gemm_skinny(x_in, w, torch.float32, skinny_splits(o, i, want_blocks=256, features=64, min_k=256))
