@@ -64,7 +64,8 @@ __global__ __launch_bounds__(256) void shortconv_kernel(
 // The same for bfloat16 with 8 channels (16 bytes) per thread and the window kept in registers:
 // a prompt portion is a pass over 3 + 1 values per (row, channel), bound by memory traffic.
 // K is a template parameter (2..4, what LFM2 checkpoints use); other lengths take the kernel above.
-constexpr int TLV = 16;  // rows per tile (>= K - 1)
+constexpr int TLV = 8;   // rows per tile (>= K - 1)
+constexpr int RU = 4;    // rows whose loads are in flight together
 
 __device__ __forceinline__ void unpack8(const uint4& raw, float* f) {
   const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
@@ -119,26 +120,46 @@ __global__ __launch_bounds__(64) void shortconv_bf16x8_kernel(
   float win[K][8];  // win[j]: B * x of row t - (K-1) + j
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) bx_at(t0 - (K - 1) + j, win[j + 1]);
-  for (int t = t0; t < t_end; ++t) {
+  for (int tg = t0; tg < t_end; tg += RU) {
+    // the loads of RU rows first, then their arithmetic: a wave is alone with its rows' latency
+    uint4 rb[RU], rx[RU], rc[RU];
 #pragma unroll
-    for (int j = 0; j < K - 1; ++j)
-#pragma unroll
-      for (int i = 0; i < 8; ++i) win[j][i] = win[j + 1][i];
-    bx_at(t, win[K - 1]);
-    float cg[8];
-    unpack8(*(const uint4*)(bcx + (size_t)(row0 + t) * ld + C + c0), cg);
-    uint32_t ow[4];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float acc = 0.f;
-#pragma unroll
-      for (int j = 0; j < K; ++j) acc = fmaf(w[i][j], win[j][i], acc);
-      acc += b[i];
-      const uint32_t bits = (uint32_t)__builtin_bit_cast(unsigned short, (bf16)(cg[i] * acc));
-      if (i % 2 == 0) ow[i / 2] = bits;
-      else ow[i / 2] |= bits << 16;
+    for (int u = 0; u < RU; ++u) {
+      rb[u] = rx[u] = rc[u] = make_uint4(0, 0, 0, 0);
+      if (tg + u < t_end) {
+        const bf16* row = bcx + (size_t)(row0 + tg + u) * ld + c0;
+        rb[u] = *(const uint4*)row;
+        rc[u] = *(const uint4*)(row + C);
+        rx[u] = *(const uint4*)(row + 2 * C);
+      }
     }
-    *(uint4*)(y + (size_t)(row0 + t) * C + c0) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+#pragma unroll
+    for (int u = 0; u < RU; ++u) {
+      const int t = tg + u;
+      if (t >= t_end) break;
+#pragma unroll
+      for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) win[j][i] = win[j + 1][i];
+      float bv[8], xv[8], cg[8];
+      unpack8(rb[u], bv);
+      unpack8(rx[u], xv);
+      unpack8(rc[u], cg);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) win[K - 1][i] = bv[i] * xv[i];
+      uint32_t ow[4];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < K; ++j) acc = fmaf(w[i][j], win[j][i], acc);
+        acc += b[i];
+        const uint32_t bits = (uint32_t)__builtin_bit_cast(unsigned short, (bf16)(cg[i] * acc));
+        if (i % 2 == 0) ow[i / 2] = bits;
+        else ow[i / 2] |= bits << 16;
+      }
+      *(uint4*)(y + (size_t)(row0 + t) * C + c0) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+    }
   }
   if (tile == 0) {
     // new[s] = window[q + s] reads old[q + s] (an index above s), so ascending s is safe

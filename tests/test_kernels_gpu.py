@@ -41,7 +41,7 @@ def test_embed(table_dtype):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("hidden", [48, 200, 2048, 5000])
+@pytest.mark.parametrize("hidden", [48, 70, 200, 2048, 5000, 20000])   # 70 and 20000: the element-wise kernel
 def test_add_rmsnorm(dtype, hidden):
     from gibbs_amd import ops
     x = rnd(7, hidden, scale=3.0)
