@@ -12,6 +12,12 @@ model entry inherits the defaults; the keys that mean something here:
     batch           requests decoded side by side (default 1)
     dtype           "bfloat16" (default) or "float32"
     min_tok_s       the run fails (exit status 3) if decode is slower
+    workload        "decode" (default: the protocol below) or "serve": `requests` prompts of
+                    `prefill_tokens` seeded ids each are submitted at once to the continuous-batching
+                    scheduler and generate `decode_tokens` tokens each (greedy, no EOS), with
+                    `max_requests` live at a time (default: all), prompts cut into portions of at
+                    most `chunk` tokens (default: none) under `max_batch_tokens` (default 2048) per
+                    step; the row reports generated and prompt tokens a second over the whole run
 
 Protocol (/root/reference/src/bench.rs:241-322): prompts are seeded synthetic ids (the reference
 cycles an encoded sentence to length, :255-259; without tokenizers on this path the ids are drawn
@@ -44,7 +50,7 @@ def _slug(name: str) -> str:
     return re.sub(r"[^a-z0-9]+", "_", name.lower()).strip("_")
 
 
-def _load(entry: Dict, base: str):
+def _load(entry: Dict, base: str, batch: int = 0, ctx: int = 0):
     import torch
 
     from .config import config_from_dict
@@ -52,7 +58,9 @@ def _load(entry: Dict, base: str):
     from .parts import DecoderModel
     from .weights import random_weights_on_device
     ident = entry["id"]
-    batch, ctx = int(entry["batch"]), int(entry["prefill_tokens"]) + int(entry["decode_tokens"]) * (int(entry["runs"]) + 1) + WARMUP_STEPS + 64
+    if not batch:
+        batch = int(entry["batch"])
+        ctx = int(entry["prefill_tokens"]) + int(entry["decode_tokens"]) * (int(entry["runs"]) + 1) + WARMUP_STEPS + 64
     if ident.startswith("random:"):
         path = os.path.join(base, ident[len("random:"):])
         with open(path) as f:
@@ -119,6 +127,43 @@ def measure(entry: Dict, base: str) -> Dict:
                                        / roofline.PEAK_FLOPS[entry["dtype"]], 4)}
 
 
+def serve(entry: Dict, base: str) -> Dict:
+    """Many requests through the scheduler: what a step holds is the scheduler's decision (prompt
+    portions beside decoded tokens, bursts of captured decode steps when only decoding is left)."""
+    import numpy as np
+    import torch
+
+    from .engine import Generator
+    from .sampling import SamplingParams
+    n_req, n_prompt, n_decode = int(entry.get("requests", 8)), int(entry["prefill_tokens"]), int(entry["decode_tokens"])
+    live = int(entry.get("max_requests", n_req))
+    engine = _load(entry, base, batch=live, ctx=-(-(n_prompt + n_decode + 1) // 64) * 64)
+    rng = np.random.default_rng(0)
+    chunk = entry.get("chunk")
+    gen = Generator(engine, max_batch_tokens=int(entry.get("max_batch_tokens", 2048)), chunk=int(chunk) if chunk else None)
+    params = SamplingParams(temperature=0.0, max_new_tokens=n_decode, ignore_eos=True)
+    warm = gen.submit(rng.integers(0, engine.spec.vocab, size=min(n_prompt, 64)).tolist(),
+                      SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True))
+    gen.run()                                                # compiles nothing, but warms libraries and captures
+    assert warm is not None
+    gen.stats = type(gen.stats)()
+    rids = [gen.submit(rng.integers(0, engine.spec.vocab, size=n_prompt).tolist(), params) for _ in range(n_req)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    results = gen.run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    done = [results[r] for r in rids if r in results and not results[r].error]
+    generated = sum(len(r.tokens) for r in done)
+    st = gen.stats
+    return {"model": entry["name"], "workload": "serve", "dtype": entry["dtype"], "requests": n_req, "live": live,
+            "prompt_tokens": n_prompt, "decode_tokens": n_decode, "chunk": chunk,
+            "finished": len(done), "wall_ms": round(1e3 * wall, 2),
+            "decode_tok_s": round(generated / wall, 1), "prompt_tok_s": round(n_req * n_prompt / wall, 1),
+            "steps_prefill_ms": round(1e3 * st.prefill_seconds, 2), "steps_decode_ms": round(1e3 * st.decode_seconds, 2),
+            "prefill_tok_s": round(st.prefill_tok_s, 1), "decode_only_tok_s": round(st.decode_tok_s, 1)}
+
+
 def run_suite(path: str) -> int:
     """Runs every model of the suite; returns the process's exit status."""
     try:
@@ -143,7 +188,7 @@ def run_suite(path: str) -> int:
         ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
         entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
         try:
-            row = measure(entry, base)
+            row = serve(entry, base) if entry.get("workload", "decode") == "serve" else measure(entry, base)
         except Exception as e:     # one model's failure is reported; the others still run (bench.rs:751)
             print(f"gibbs --bench: {entry['name']}: {type(e).__name__}: {e}", file=sys.stderr)
             failed = True
@@ -156,8 +201,9 @@ def run_suite(path: str) -> int:
     for row in rows:
         print(f"METRIC {_slug(row['model'])}_tok_s={row['decode_tok_s']}")
         print(f"METRIC {_slug(row['model'])}_prefill_tok_s={row['prefill_tok_s']}")
-    if rows:
-        geo = math.exp(sum(math.log(max(r["roofline_pct"], 1e-9)) for r in rows) / len(rows))
+    pcts = [r["roofline_pct"] for r in rows if "roofline_pct" in r]
+    if pcts:
+        geo = math.exp(sum(math.log(max(p, 1e-9)) for p in pcts) / len(pcts))
         print(f"METRIC geomean_roofline_pct={geo:.2f}")
     for line in missed:
         print(f"gibbs --bench: {line}", file=sys.stderr)

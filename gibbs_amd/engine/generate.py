@@ -46,6 +46,11 @@ class GenerationStats:
         return self.decode_tokens / max(self.decode_seconds, 1e-9)
 
 
+# a burst shorter than this does not get a decode loop (and captured graphs) of its own: requests
+# that finish one after another would otherwise have a loop made for every batch size on the way down
+MIN_STEPS_FOR_NEW_LOOP = 8
+
+
 class Generator:
     def __init__(self, engine: Engine, *, max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
                  eos_token_ids: Optional[Sequence[int]] = None, decode_burst: int = 16):
@@ -86,6 +91,8 @@ class Generator:
         key = (len(seqs), greedy)
         try:
             loop = self._loops.get(key)
+            if loop is None and n < MIN_STEPS_FOR_NEW_LOOP:
+                return None                                 # capturing graphs for so few steps costs more than it saves
             if loop is None:
                 loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index)
             elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:

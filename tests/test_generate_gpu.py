@@ -309,12 +309,16 @@ def test_bench_suite_through_the_command_line(dirs, tmp_path):
     (tmp_path / "cfg.json").write_text(json.dumps(H.TINY["C"]))
     suite = {"defaults": {"prefill_tokens": 40, "decode_tokens": 8, "runs": 2},
              "models": [{"id": dirs["A"], "name": "Tiny A", "dtype": "float32"},
-                        {"id": "random:cfg.json", "batch": 3}]}
+                        {"id": "random:cfg.json", "batch": 3},
+                        {"id": dirs["B"], "name": "served", "workload": "serve", "requests": 5, "max_requests": 3,
+                         "prefill_tokens": 21, "decode_tokens": 12, "chunk": 8, "max_batch_tokens": 16}]}
     (tmp_path / "suite.json").write_text(json.dumps(suite))
     p = run("--bench", str(tmp_path / "suite.json"))
     assert p.returncode == 0, p.stderr[-2000:]
     rows = [json.loads(l) for l in p.stdout.splitlines() if l.startswith("{")]
-    assert [r["model"] for r in rows] == ["Tiny A", "cfg"] and rows[1]["batch"] == 3
+    assert [r["model"] for r in rows] == ["Tiny A", "cfg", "served"] and rows[1]["batch"] == 3
+    served = rows.pop()
+    assert served["finished"] == 5 and served["live"] == 3 and served["decode_tok_s"] > 0 and served["prompt_tok_s"] > 0
     for r in rows:
         assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0 and 0 < r["roofline_pct"] < 100
         assert abs(r["roofline_tok_s"] * r["bytes_per_token"] - r["ceiling_gbps"] * 1e9) < 1e-3 * r["ceiling_gbps"] * 1e9
