@@ -21,7 +21,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# BASELINE.json configs[2]: the LFM2-1.2B shape
+# the LFM2-1.2B shape (Liquid's 1.2B model: 16 layers, 6 of them attention)
 SHAPE = dict(
     architectures=["Lfm2ForCausalLM"], model_type="lfm2", hidden_size=2048, num_hidden_layers=16,
     full_attn_idxs=[2, 5, 8, 10, 12, 14], num_attention_heads=32, num_key_value_heads=8, head_dim=64,

@@ -4,11 +4,13 @@
 // A workgroup takes 64 consecutive query rows of one request and one query head; each of its 4
 // waves owns 16 of the rows.  Keys are walked in tiles of 64 aligned to absolute key index (so a
 // row's sequence of operations does not depend on how the prompt was cut).  Per tile:
-//   K tile -> LDS as stored ([key][d]): it is the B operand of S = Q K^T as it lies
-//   V tile -> LDS transposed ([d][key]): the B operand of O += P V must be contiguous along keys
-//   S (16 x 64 per wave) = v_mfma_f32_16x16x32_bf16 over d;  scale, mask by position;
-//   online softmax per row (row maxima by shuffles over the 16 lanes that share a row);
-//   P -> bfloat16 -> the wave's LDS patch -> back as the A operand;  O += P V.
+//   K tile -> LDS as stored ([key][d]);  V tile -> LDS transposed ([d][key], keys of a group of 32
+//   in the order the product below wants them);
+//   scores transposed, S^T (64 keys x 16 rows per wave) = K Q^T by v_mfma_f32_16x16x32_bf16 over d:
+//   a lane then holds 16 scores of ONE query row (lane % 16), so that the online softmax needs no
+//   exchange between lanes except two steps over the 4 lanes that share the row, and exp(S - m)
+//   is, as it lies in the registers, the B operand of O^T += V^T P^T (the contraction runs over
+//   the keys in any order, as long as V^T is read in the same one): P never goes through LDS.
 // Keys come from the request's pages through its block table; row n sees keys lo .. pos[n]
 // (lo = max(0, pos - window + 1), window 0 = all).  The step's own keys were written to the pages
 // before this kernel runs.  Head sizes: multiples of 16 up to 128.
@@ -23,24 +25,19 @@ constexpr int BN = 64;   // keys per tile
 constexpr int LDP = BN + 8;
 constexpr int SEG_PAGES = 1024;  // page ids kept in LDS at a time (a segment of the request's block table)
 
-// Maximum / sum over the 16 lanes of a row (the lanes that hold one query row's scores), every lane
-// getting the result: data-parallel-primitive moves (swap in pairs, in quads, mirror the half row,
-// mirror the row) instead of LDS permutes, which sit on the critical path of every key tile.
-template <int CTRL>
-__device__ __forceinline__ float dpp_move(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+// Maximum / sum over the 4 lanes that hold one query row's scores (lanes l, l ^ 16, l ^ 32, l ^ 48),
+// every lane getting the result: two lane-swap instructions each (rows of 16 lanes, halves of 32).
+__device__ __forceinline__ float row4_max(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
-__device__ __forceinline__ float row16_max(float v) {
-  v = fmaxf(v, dpp_move<0xB1>(v));
-  v = fmaxf(v, dpp_move<0x4E>(v));
-  v = fmaxf(v, dpp_move<0x141>(v));
-  return fmaxf(v, dpp_move<0x140>(v));
-}
-__device__ __forceinline__ float row16_sum(float v) {
-  v += dpp_move<0xB1>(v);
-  v += dpp_move<0x4E>(v);
-  v += dpp_move<0x141>(v);
-  return v + dpp_move<0x140>(v);
+__device__ __forceinline__ float row4_sum(float v) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 struct PrefillArgs {
@@ -65,7 +62,6 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   constexpr int LDK = HD + 8;
   __shared__ bf16 sK[BN][LDK];
   __shared__ bf16 sVT[HD][LDP];
-  __shared__ bf16 sP[4][16][LDP];
   __shared__ int s_pages[SEG_PAGES];
 
   // which request and which 64 rows of it
@@ -110,17 +106,12 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
                 ? *(const bf16x8*)(q + (size_t)(n0 + my_row) * a.ldq + (size_t)head * HD + d)
                 : zero8;
   }
-  // rows this lane owns in S and O: wave*16 + g*4 + i
-  int pos_i[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) pos_i[i] = p0 + min(wave * 16 + g * 4 + i, rows_here - 1);
+  // the query row this lane owns in S^T and O^T: wave*16 + lr
+  const int pos_row = p0 + min(wave * 16 + lr, rows_here - 1);
 
-  float m[4], l[4];
-  floatx4 o[DT];
-#pragma unroll
-  // a finite stand-in for 'no key seen yet': exp2(x - m) is then 0 for masked scores and for the
-  // first rescale, with no special cases on the path of every score
-  for (int i = 0; i < 4; ++i) { m[i] = -1e30f; l[i] = 0.f; }
+  // a finite stand-in for 'no key seen yet': exp2 of anything minus it is 0, with no special cases
+  float m = -1e30f, l = 0.f;   // maximum of the raw scores; sum of this lane's share of the row
+  floatx4 o[DT];               // O^T: d = t*16 + g*4 + i of row lr
 #pragma unroll
   for (int t = 0; t < DT; ++t) o[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 
@@ -167,13 +158,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
       const int c = tid + i * 256;
       if (c >= (BN / 2) * (HD / 8)) continue;
       const int kp = c % (BN / 2), d = (c / (BN / 2)) * 8;
+      // key k of a group of 32 (k = b*16 + q*4 + j) lies at q*8 + b*4 + j: the 8 keys that a lane of
+      // the product O^T += V^T P^T holds side by side (4 of each half of the group)
+      const int k2 = 2 * kp, kin = k2 % 32;
+      const int vpos = k2 - kin + ((kin % 16) / 4) * 8 + (kin / 16) * 4 + kin % 4;
       const uint32_t w0[4] = {vreg0[i].x, vreg0[i].y, vreg0[i].z, vreg0[i].w};
       const uint32_t w1[4] = {vreg1[i].x, vreg1[i].y, vreg1[i].z, vreg1[i].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         // elements d+2j and d+2j+1 of both keys
-        *(uint32_t*)&sVT[d + 2 * j][2 * kp] = (w0[j] & 0xffffu) | (w1[j] << 16);
-        *(uint32_t*)&sVT[d + 2 * j + 1][2 * kp] = (w0[j] >> 16) | (w1[j] & 0xffff0000u);
+        *(uint32_t*)&sVT[d + 2 * j][vpos] = (w0[j] & 0xffffu) | (w1[j] << 16);
+        *(uint32_t*)&sVT[d + 2 * j + 1][vpos] = (w0[j] >> 16) | (w1[j] & 0xffff0000u);
       }
     }
   };
@@ -206,7 +201,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     // a wave whose rows see none of this tile's keys has nothing to do (it still takes part in the barriers)
     if (key0 > wave_last || key0 + BN <= wave_first_key) continue;
 
-    // S = Q K^T: 4 sub-tiles of 16 keys
+    // S^T = K Q^T: 4 sub-tiles of 16 keys; this lane gets S[row lr][key c*16 + g*4 + i]
     floatx4 s4[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -215,72 +210,75 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
       for (int s = 0; s < DS; ++s) {
         const int d = s * 32 + g * 8;
         const bf16x8 kf = d < HD ? *(const bf16x8*)&sK[c * 16 + lr][d] : zero8;
-        s4[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[s], kf, s4[c], 0, 0, 0);
+        s4[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[s], s4[c], 0, 0, 0);
       }
     }
-    // scale, mask, row maxima: this lane holds S[row g*4+i][key c*16+lr]
+    // mask by position, row maximum (of the raw scores: the scale is positive)
     const bool need_mask = key0 + BN - 1 > p0 + wave * 16 || a.window > 0;
-    float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-      const int key = key0 + c * 16 + lr;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = s4[c][i] * scale2;  // scores in units of log2: exp(s) = exp2(s * log2 e)
+        float v = s4[c][i];
         if (need_mask) {
-          const bool vis = key <= pos_i[i] && (a.window == 0 || key > pos_i[i] - a.window);
+          const int key = key0 + c * 16 + g * 4 + i;
+          const bool vis = key <= pos_row && (a.window == 0 || key > pos_row - a.window);
           v = vis ? v : -INFINITY;
+          s4[c][i] = v;
         }
-        s4[c][i] = v;
-        mx[i] = fmaxf(mx[i], v);
+        mx = fmaxf(mx, v);
       }
     }
-    float keep[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      mx[i] = row16_max(mx[i]);
-      const float m_new = fmaxf(m[i], mx[i]);
-      keep[i] = __builtin_amdgcn_exp2f(m[i] - m_new);
-      m[i] = m_new;
-      l[i] *= keep[i];
-    }
-    // P = exp(S - m) -> bfloat16 -> the wave's patch of LDS
+    mx = row4_max(mx);
+    const float m_new = fmaxf(m, mx);
+    const float keep = __builtin_amdgcn_exp2f((m - m_new) * scale2);
+    const float shift = -m_new * scale2;
+    m = m_new;
+    l *= keep;
+    // P^T = exp(S^T - m) in units of log2 (exp(s) = exp2(s * log2 e)), as B operands: element e of
+    // step kk is key (2 kk + e / 4) * 16 + g * 4 + e % 4
+    bf16x8 pf[2];
 #pragma unroll
     for (int c = 0; c < 4; ++c)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = __builtin_amdgcn_exp2f(s4[c][i] - m[i]);
-        l[i] += p;
-        sP[wave][g * 4 + i][c * 16 + lr] = (bf16)p;
+        const float p = __builtin_amdgcn_exp2f(fmaf(s4[c][i], scale2, shift));
+        l += p;
+        pf[c / 2][(c % 2) * 4 + i] = (bf16)p;
       }
 #pragma unroll
     for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] *= keep[i];
-    // the wave reads back what its own lanes wrote: LDS operations of a wave complete in order
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    // O += P V: k runs over the 64 keys in 2 steps of 32
+      for (int i = 0; i < 4; ++i) o[t][i] *= keep;
+    // O^T += V^T P^T: k runs over the 64 keys in 2 steps of 32
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      const bf16x8 pf = *(const bf16x8*)&sP[wave][lr][kk * 32 + g * 8];
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
         const bf16x8 vf = *(const bf16x8*)&sVT[t * 16 + lr][kk * 32 + g * 8];
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[t], 0, 0, 0);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[t], 0, 0, 0);
       }
     }
   }
 
-  // row sums over the 16 lanes that share the rows; store
+  // row sum over the 4 lanes that share the row; store d = t*16 + g*4 .. +4 of row lr
+  l = row4_sum(l);
+  const int row = wave * 16 + lr;
+  if (row < rows_here) {
+    const float inv = 1.0f / l;
+    bf16* dst = out + (size_t)(n0 + row) * a.ldo + (size_t)head * HD + g * 4;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    l[i] = row16_sum(l[i]);
-    const int row = wave * 16 + g * 4 + i;
-    if (row >= rows_here) continue;
-    const float inv = 1.0f / l[i];
-    bf16* dst = out + (size_t)(n0 + row) * a.ldo + (size_t)head * HD;
+    for (int t = 0; t < DT; ++t) {
+      typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+      const bf16x4 v = {(bf16)(o[t][0] * inv), (bf16)(o[t][1] * inv), (bf16)(o[t][2] * inv), (bf16)(o[t][3] * inv)};
+      if (a.ldo % 4 == 0) {
+        *(bf16x4*)(dst + t * 16) = v;
+      } else {
 #pragma unroll
-    for (int t = 0; t < DT; ++t) dst[t * 16 + lr] = (bf16)(o[t][i] * inv);
+        for (int i = 0; i < 4; ++i) dst[t * 16 + i] = v[i];
+      }
+    }
   }
 }
 }  // namespace

@@ -127,7 +127,7 @@ def test_reference_golden_vector_through_the_engine(dirs, dtype):
 
 
 def test_seeded_temperature_sampling(dirs):
-    """BASELINE's Tiny B workload: four requests (5, 11, 17, 29 tokens), prompt portions of 8,
+    """The Tiny B workload: four requests (5, 11, 17, 29 tokens), prompt portions of 8,
     temperature 0.8 from a fixed seed.  Every token equals what the plain sampler draws from the
     plain logits of the same history with the same draw."""
     from gibbs_amd import Engine, Generator, SamplingParams
