@@ -52,7 +52,9 @@ struct PrefillArgs {
   int window;
 };
 
-template <int DT>  // head size = 16 * DT
+// DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
+// integer division costs dozens of instructions, several times per thread and tile).
+template <int DT, bool POW2>
 __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __restrict__ q,
                                                                 const bf16* __restrict__ kpages,
                                                                 const bf16* __restrict__ vpages, bf16* __restrict__ out,
@@ -85,11 +87,10 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   const int p0 = a.ctx[r] + row_in_req0;             // its absolute position
   const int rows_here = min(BM, qlen - row_in_req0);
   const int* table = a.table + (size_t)r * a.max_pages;
-  // (page, slot) of a key: shifts when the page size is a power of two (integer division costs
-  // dozens of instructions, several times per thread and tile); page ids come from a segment of
-  // the block table held in LDS, so that a tile's loads do not wait for a table load first
+  // (page, slot) of a key; page ids come from a segment of the block table held in LDS, so that a
+  // tile's loads do not wait for a table load first
   int seg_first_page = 0;
-  auto logical_page = [&](int ak) -> int { return a.page_shift >= 0 ? ak >> a.page_shift : ak / a.page_size; };
+  auto logical_page = [&](int ak) -> int { return POW2 ? ak >> a.page_shift : ak / a.page_size; };
   auto page_row = [&](const bf16* pages, int ak) -> const bf16* {
     const int lp = logical_page(ak);
     return pages + (((size_t)s_pages[lp - seg_first_page] * a.nkv + kvh) * a.page_size + (ak - lp * a.page_size)) * HD;
@@ -106,8 +107,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
                 ? *(const bf16x8*)(q + (size_t)(n0 + my_row) * a.ldq + (size_t)head * HD + d)
                 : zero8;
   }
-  // the query row this lane owns in S^T and O^T: wave*16 + lr
+  // the query row this lane owns in S^T and O^T: wave*16 + lr; it sees keys above lo_row up to pos_row
   const int pos_row = p0 + min(wave * 16 + lr, rows_here - 1);
+  const int lo_row = a.window > 0 ? pos_row - a.window : -1;
 
   // a finite stand-in for 'no key seen yet': exp2 of anything minus it is 0, with no special cases
   float m = -1e30f, l = 0.f;   // maximum of the raw scores; sum of this lane's share of the row
@@ -223,7 +225,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
         float v = s4[c][i];
         if (need_mask) {
           const int key = key0 + c * 16 + g * 4 + i;
-          const bool vis = key <= pos_row && (a.window == 0 || key > pos_row - a.window);
+          const bool vis = (key <= pos_row) & (key > lo_row);
           v = vis ? v : -INFINITY;
           s4[c][i] = v;
         }
@@ -281,6 +283,11 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     }
   }
 }
+template <int DT>
+void launch_prefill(dim3 grid, hipStream_t stream, const bf16* q, const bf16* k, const bf16* v, bf16* out, const PrefillArgs& a) {
+  if (a.page_shift >= 0) attention_prefill_kernel<DT, true><<<grid, 256, 0, stream>>>(q, k, v, out, a);
+  else attention_prefill_kernel<DT, false><<<grid, 256, 0, stream>>>(q, k, v, out, a);
+}
 }  // namespace
 
 // q: [N, >= nh*hd] bfloat16 (row stride ldq), rows of request r are cu[r] .. cu[r+1] at positions
@@ -303,14 +310,14 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;
   switch (hd / 16) {
-    case 1: attention_prefill_kernel<1><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 2: attention_prefill_kernel<2><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 3: attention_prefill_kernel<3><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 4: attention_prefill_kernel<4><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 5: attention_prefill_kernel<5><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 6: attention_prefill_kernel<6><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    case 7: attention_prefill_kernel<7><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
-    default: attention_prefill_kernel<8><<<grid, 256, 0, stream>>>(qq, kk, vv, oo, a); break;
+    case 1: launch_prefill<1>(grid, stream, qq, kk, vv, oo, a); break;
+    case 2: launch_prefill<2>(grid, stream, qq, kk, vv, oo, a); break;
+    case 3: launch_prefill<3>(grid, stream, qq, kk, vv, oo, a); break;
+    case 4: launch_prefill<4>(grid, stream, qq, kk, vv, oo, a); break;
+    case 5: launch_prefill<5>(grid, stream, qq, kk, vv, oo, a); break;
+    case 6: launch_prefill<6>(grid, stream, qq, kk, vv, oo, a); break;
+    case 7: launch_prefill<7>(grid, stream, qq, kk, vv, oo, a); break;
+    default: launch_prefill<8>(grid, stream, qq, kk, vv, oo, a); break;
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
 }
