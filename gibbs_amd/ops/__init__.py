@@ -2,7 +2,6 @@
 what the kernel and its grid assume, then queues the kernel on the current stream."""
 from __future__ import annotations
 
-import os
 from typing import Optional
 
 import torch
@@ -248,9 +247,10 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
     o = w.shape[0]
     assert stream_x.dtype == torch.float32 and stream_x.shape == (n, o) and stream_x.is_contiguous()
     assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, o) and mirror.is_contiguous()
-    if n > 32 and not os.environ.get("GIBBS_RESIDUAL_DIRECT"):
-        # many rows: every workgroup re-reads x_in, so workgroups take 64 features each and the chip is
-        # filled by cutting k instead; the partial sums are added to the stream by a second kernel
+    if n > 32 and i >= 4096:
+        # many rows and a long inner size: every workgroup re-reads x_in, so workgroups take 64 features
+        # each and the chip is filled by cutting k instead; the partial sums are added to the stream by
+        # a second kernel (measured at 33 to 64 rows: 17 against 24 us at k = 8192, 12 against 9 at 2048)
         parts = gemm_skinny(x_in, w, torch.float32, skinny_splits(o, i, want_blocks=256, features=64, min_k=256))
         residual_add(stream_x, parts if parts.dim() == 3 else parts[None], mirror)
         return
