@@ -142,7 +142,7 @@ def main() -> int:
 
     cfg = engine.config
     line = {
-        "metric": "decode tok/s at batch 8 (LFM2-1.2B shape, 2,048-token prompts, context 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B shape, 2,048-token prompts, context 4096)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
