@@ -301,7 +301,7 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
                            rotary_dim: int, variant: str, window: Optional[int] = None,
                            max_seq: int = 0, n_splits: Optional[int] = None,
                            out: Optional[torch.Tensor] = None, cos_sin: Optional[torch.Tensor] = None,
-                           waves: Optional[int] = None) -> torch.Tensor:
+                           waves: Optional[int] = None, kind: str = "auto") -> torch.Tensor:
     """Decode attention straight from the raw fused projection qkv[N, (nh + 2 nkv) hd] of N decoded
     tokens: q/k norm and rotation, the write of the new key and value to their pages, attention over
     split keys in one kernel (followed by the merge of the slices).  `cos_sin` as in `qk_rope_kv`."""
@@ -323,7 +323,7 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
         if rotary_dim % 16:
             raise KernelError(f"attention_decode_fused: rotary_dim {rotary_dim} must be a multiple of 16")
     if n_splits is None or waves is None:
-        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind)
         n_splits = auto_splits if n_splits is None else n_splits
         waves = auto_waves if waves is None else waves
     partial = None
@@ -336,7 +336,7 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
          ptr(q_gain), ptr(k_gain), float(eps), ptr(inv_freq), rotary_dim, ROPE_VARIANTS[variant], ptr(cos_sin),
          table_len, ptr(pos), ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
          qkv.stride(0) if n_rows > 1 else qkv.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves),
-         stream())
+         DECODE_KINDS[kind], int(max_seq), stream())
     return out
 
 
@@ -453,23 +453,29 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
     return out
 
 
-def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int) -> tuple:
+# how the decode attention walks its keys: chosen by the kernel, on the vector units, on the matrix cores
+DECODE_KINDS = {"auto": 0, "valu": 1, "mfma": 2}
+
+
+def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, kind: str = "auto") -> tuple:
     """(key slices per (row, kv head), waves per workgroup) for the decode attention.  Few rows:
-    enough slices of at least 64 keys to give each of the 256 compute units two workgroups of 4
-    waves.  Rows and heads that fill the chip by themselves: no slices, 8 waves (measured at batch
-    1 to 64 and 2,048 to 8,192 keys; a slice costs every wave its own prologue and final fold)."""
+    enough slices to give each of the 256 compute units two workgroups of 4 waves, but at least 64
+    keys to a slice (128 on the matrix cores: a tile of 32 for every wave).  Rows and heads that fill
+    the chip by themselves: no slices (a slice costs every wave its own prologue and final fold), 8
+    waves on the vector units, 4 on the matrix cores (measured at batch 1 to 64, 2,048 to 8,192 keys)."""
+    matrix = kind != "valu" and hd > 0 and hd % 16 == 0 and hd <= 128
     gt = 8 if group >= 8 else (4 if group > 2 else group)
     per_split = n_rows * nkv * -(-group // gt)
     if per_split >= 256:
-        return 1, 8
+        return 1, (4 if matrix else 8)
     want = -(-512 // per_split)
-    return max(1, min(want, max_seq // 64, 256)), 4
+    return max(1, min(want, max_seq // (128 if matrix else 64), 256)), 4
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                      vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
                      scale: float, window: Optional[int] = None, max_seq: int = 0, n_splits: Optional[int] = None,
-                     out: Optional[torch.Tensor] = None, waves: Optional[int] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, waves: Optional[int] = None, kind: str = "auto") -> torch.Tensor:
     """bfloat16 paged attention for rows with few queries and long caches (decoded tokens): the
     keys of each (row, kv head) are cut into `n_splits` slices that run as workgroups of their own
     and are merged afterwards.  Same operands and result as `attention_plain`."""
@@ -484,7 +490,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     assert table.dim() == 2 and table.shape[0] >= n_req
     _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
     if n_splits is None or waves is None:
-        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq)
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind)
         n_splits = auto_splits if n_splits is None else n_splits
         waves = auto_waves if waves is None else waves
     partial = None
@@ -495,7 +501,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
     call("gibbs_attention_decode", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(pos), ptr(row_req),
          ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
-         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves), stream())
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), n_splits, int(waves), DECODE_KINDS[kind], int(max_seq), stream())
     return out
 
 

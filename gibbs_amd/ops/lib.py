@@ -44,7 +44,7 @@ _SIGNATURES = {
                           c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p],
     "gibbs_attention_decode_fused": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_float, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                     c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_void_p],
+                                     c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_shortconv": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
                         c_int, c_int, c_int, c_int, c_int, c_void_p],
@@ -57,7 +57,7 @@ _SIGNATURES = {
     "gibbs_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
-                               c_int, c_void_p],
+                               c_int, c_int, c_int, c_void_p],
     "gibbs_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],

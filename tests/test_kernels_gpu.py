@@ -273,11 +273,12 @@ def test_attention_plain_paged(dtype, nh, nkv, hd, page, window):
         at += len(ps)
 
 
+@pytest.mark.parametrize("kind", ["valu", "mfma"])
 @pytest.mark.parametrize("n_splits,waves", [(1, 4), (1, 8), (3, 8), (16, 4), (None, None)])
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
                                                    (32, 8, 64, 16, None), (16, 2, 128, 16, None), (2, 2, 256, 64, 100),
-                                                   (24, 2, 32, 16, None)])
-def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves):
+                                                   (24, 2, 32, 16, None), (3, 1, 24, 16, None)])
+def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves, kind):
     """The key-splitting kernel against the float64 reference and against the plain kernel, for
     rows of different lengths (one key, a page edge, hundreds of keys) in one call."""
     from gibbs_amd import ops
@@ -288,8 +289,13 @@ def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves)
     pos, row_req = i32(positions), i32([0, 1, 2, 3])
     q = rnd(4, nh * hd, dtype=dtype, seed=9)
     scale = 1 / math.sqrt(hd)
+    if kind == "mfma" and (hd % 16 or hd > 128):
+        with pytest.raises(ops.KernelError, match="matrix-core"):
+            ops.attention_decode(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window, max_seq=700,
+                                 n_splits=n_splits, waves=waves, kind=kind)
+        return
     out = ops.attention_decode(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window, max_seq=700,
-                               n_splits=n_splits, waves=waves)
+                               n_splits=n_splits, waves=waves, kind=kind)
     plain = ops.attention_plain(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window)
     for r in range(4):
         want = attention_reference(q[r:r + 1].view(1, nh, hd), ks[r], vs[r], [positions[r]], scale, window)
@@ -537,11 +543,12 @@ def test_embed_and_residual_mirror():
     close(out, F.rms_norm(x.double(), (72,), None, 1e-5), torch.bfloat16, "gain-free norm")
 
 
+@pytest.mark.parametrize("kind", ["valu", "mfma"])
 @pytest.mark.parametrize("n_splits,table_len,waves", [(1, 0, 8), (4, 20, 4), (None, 1024, None)])   # rows at 699 and 32 beyond a table of 20
 @pytest.mark.parametrize("variant", ["half_split", "interleaved"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,page,window", [(4, 2, 16, 16, 16, None), (32, 8, 64, 64, 16, None), (6, 1, 48, 32, 8, None),
                                                        (5, 5, 80, 80, 32, 37), (16, 2, 128, 128, 16, None), (24, 2, 32, 32, 16, None)])
-def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_splits, table_len, waves):
+def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_splits, table_len, waves, kind):
     """The fused decode attention against the separate kernels: same pages afterwards, same output,
     for rows at a page's first slot, its last slot, position 0 and far into the cache."""
     from gibbs_amd import ops
@@ -562,7 +569,7 @@ def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_split
     kp1, vp1 = kp.clone(), vp.clone()
     got = ops.attention_decode_fused(qkv, n, nh, nkv, hd, kp1, vp1, table, n, pos, row_req, scale, q_gain=qg,
                                      k_gain=kg, eps=1e-6, inv_freq=inv, rotary_dim=rot, variant=variant,
-                                     window=window, max_seq=700, n_splits=n_splits, waves=waves,
+                                     window=window, max_seq=700, n_splits=n_splits, waves=waves, kind=kind,
                                      cos_sin=ops.rope_table(inv, table_len) if table_len else None)
     close(kp1, kp2, dtype, "new keys in the pages", bf16=8e-3)
     assert torch.equal(vp1, vp2)
