@@ -4,13 +4,13 @@
 // A workgroup takes 64 consecutive query rows of one request and one query head; each of its 4
 // waves owns 16 of the rows.  Keys are walked in tiles of 64 aligned to absolute key index (so a
 // row's sequence of operations does not depend on how the prompt was cut).  Per tile:
-//   K tile -> LDS as stored ([key][d]);  V tile -> LDS transposed ([d][key], keys of a group of 32
-//   in the order the product below wants them);
+//   K and V tiles -> LDS as stored ([key][d]);
 //   scores transposed, S^T (64 keys x 16 rows per wave) = K Q^T by v_mfma_f32_16x16x32_bf16 over d:
 //   a lane then holds 16 scores of ONE query row (lane % 16), so that the online softmax needs no
 //   exchange between lanes except two steps over the 4 lanes that share the row, and exp(S - m)
 //   is, as it lies in the registers, the B operand of O^T += V^T P^T (the contraction runs over
 //   the keys in any order, as long as V^T is read in the same one): P never goes through LDS.
+//   V^T comes from the V tile as it was stored, through the transposing LDS read of gfx950.
 // Keys come from the request's pages through its block table; row n sees keys lo .. pos[n]
 // (lo = max(0, pos - window + 1), window 0 = all).  The step's own keys were written to the pages
 // before this kernel runs.  Head sizes: multiples of 16 up to 128.
@@ -19,10 +19,11 @@
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
 
 constexpr int BM = 64;   // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
-constexpr int LDP = BN + 8;
 constexpr int SEG_PAGES = 1024;  // page ids kept in LDS at a time (a segment of the request's block table)
 
 // Maximum / sum over the 4 lanes that hold one query row's scores (lanes l, l ^ 16, l ^ 32, l ^ 48),
@@ -38,6 +39,14 @@ __device__ __forceinline__ float row4_sum(float v) {
   v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
   auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+// 4 x 4 elements of a row-major 16-bit matrix in LDS, transposed: of the 16 lanes of a row of lanes, lane j
+// passes the address of 4 consecutive elements and receives element j % 4 of the lanes j / 4, j / 4 + 4,
+// j / 4 + 8, j / 4 + 12 (ds_read_b64_tr_b16).  With lane j pointing at V[key j / 4][d0 + 4 (j % 4)] it
+// receives V[key 0..3][d0 + j]: the keys run along the register, as the matrix instruction wants them.
+__device__ __forceinline__ short4v lds_read_transposed(const bf16* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)p);
 }
 
 struct PrefillArgs {
@@ -63,7 +72,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   constexpr int DS = (DT + 1) / 2;  // steps of 32 over d
   constexpr int LDK = HD + 8;
   __shared__ bf16 sK[BN][LDK];
-  __shared__ bf16 sVT[HD][LDP];
+  __shared__ bf16 sV[BN][LDK];
   __shared__ int s_pages[SEG_PAGES];
 
   // which request and which 64 rows of it
@@ -125,26 +134,17 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
 
   // One tile ahead: the next tile's keys and values travel from memory to registers while the
   // matrix cores work on the current tile, and go to LDS once everyone is done with it.
-  constexpr int KCH = (BN * (HD / 8) + 255) / 256;        // 16-byte chunks of K per thread and tile
-  constexpr int VCH = ((BN / 2) * (HD / 8) + 255) / 256;  // pairs of V chunks per thread and tile
-  uint4 kreg[KCH], vreg0[VCH], vreg1[VCH];
+  constexpr int KCH = (BN * (HD / 8) + 255) / 256;        // 16-byte chunks of K (and of V) per thread and tile
+  uint4 kreg[KCH], vreg[KCH];
   auto load_tile = [&](int key0) {
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = tid + i * 256;
       const int key = c / (HD / 8), d = (c % (HD / 8)) * 8;
-      kreg[i] = make_uint4(0, 0, 0, 0);
-      if (c < BN * (HD / 8) && key0 + key <= last_pos) kreg[i] = *(const uint4*)(page_row(kpages, key0 + key) + d);
-    }
-#pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + i * 256;
-      const int kp = c % (BN / 2), d = (c / (BN / 2)) * 8;
-      const int ak = key0 + 2 * kp;
-      vreg0[i] = vreg1[i] = make_uint4(0, 0, 0, 0);
-      if (c < (BN / 2) * (HD / 8)) {
-        if (ak <= last_pos) vreg0[i] = *(const uint4*)(page_row(vpages, ak) + d);
-        if (ak + 1 <= last_pos) vreg1[i] = *(const uint4*)(page_row(vpages, ak + 1) + d);
+      kreg[i] = vreg[i] = make_uint4(0, 0, 0, 0);
+      if (c < BN * (HD / 8) && key0 + key <= last_pos) {
+        kreg[i] = *(const uint4*)(page_row(kpages, key0 + key) + d);
+        vreg[i] = *(const uint4*)(page_row(vpages, key0 + key) + d);
       }
     }
   };
@@ -152,25 +152,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
       const int c = tid + i * 256;
-      if (c < BN * (HD / 8)) *(uint4*)&sK[c / (HD / 8)][(c % (HD / 8)) * 8] = kreg[i];
-    }
-    // V transposed: a thread holds two neighbouring keys x 8 d and writes 8 packed pairs
-#pragma unroll
-    for (int i = 0; i < VCH; ++i) {
-      const int c = tid + i * 256;
-      if (c >= (BN / 2) * (HD / 8)) continue;
-      const int kp = c % (BN / 2), d = (c / (BN / 2)) * 8;
-      // key k of a group of 32 (k = b*16 + q*4 + j) lies at q*8 + b*4 + j: the 8 keys that a lane of
-      // the product O^T += V^T P^T holds side by side (4 of each half of the group)
-      const int k2 = 2 * kp, kin = k2 % 32;
-      const int vpos = k2 - kin + ((kin % 16) / 4) * 8 + (kin / 16) * 4 + kin % 4;
-      const uint32_t w0[4] = {vreg0[i].x, vreg0[i].y, vreg0[i].z, vreg0[i].w};
-      const uint32_t w1[4] = {vreg1[i].x, vreg1[i].y, vreg1[i].z, vreg1[i].w};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        // elements d+2j and d+2j+1 of both keys
-        *(uint32_t*)&sVT[d + 2 * j][vpos] = (w0[j] & 0xffffu) | (w1[j] << 16);
-        *(uint32_t*)&sVT[d + 2 * j + 1][vpos] = (w0[j] >> 16) | (w1[j] & 0xffff0000u);
+      if (c < BN * (HD / 8)) {
+        *(uint4*)&sK[c / (HD / 8)][(c % (HD / 8)) * 8] = kreg[i];
+        *(uint4*)&sV[c / (HD / 8)][(c % (HD / 8)) * 8] = vreg[i];
       }
     }
   };
@@ -258,8 +242,11 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
-        const bf16x8 vf = *(const bf16x8*)&sVT[t * 16 + lr][kk * 32 + g * 8];
-        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[kk], o[t], 0, 0, 0);
+        // V^T of d = t*16 + lr, the 8 keys of pf[kk]: two transposing reads of 4 keys each
+        const short4v v0 = lds_read_transposed(&sV[(2 * kk) * 16 + g * 4 + lr / 4][t * 16 + 4 * (lr % 4)]);
+        const short4v v1 = lds_read_transposed(&sV[(2 * kk + 1) * 16 + g * 4 + lr / 4][t * 16 + 4 * (lr % 4)]);
+        const short8v both = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+        o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, both), pf[kk], o[t], 0, 0, 0);
       }
     }
   }
