@@ -323,7 +323,7 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
         if rotary_dim % 16:
             raise KernelError(f"attention_decode_fused: rotary_dim {rotary_dim} must be a multiple of 16")
     if n_splits is None or waves is None:
-        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind)
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind, page_size)
         n_splits = auto_splits if n_splits is None else n_splits
         waves = auto_waves if waves is None else waves
     partial = None
@@ -457,19 +457,26 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
 DECODE_KINDS = {"auto": 0, "valu": 1, "mfma": 2}
 
 
-def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, kind: str = "auto") -> tuple:
+MATRIX_SLICE_PAGES = 510   # page ids of a key slice that the matrix-core walk keeps in LDS
+
+
+def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, kind: str = "auto",
+                  page_size: int = 16) -> tuple:
     """(key slices per (row, kv head), waves per workgroup) for the decode attention.  Few rows:
     enough slices to give each of the 256 compute units two workgroups of 4 waves, but at least 64
     keys to a slice (128 on the matrix cores: a tile of 32 for every wave).  Rows and heads that fill
     the chip by themselves: no slices (a slice costs every wave its own prologue and final fold), 8
-    waves on the vector units, 4 on the matrix cores (measured at batch 1 to 64, 2,048 to 8,192 keys)."""
+    waves on the vector units, 4 on the matrix cores (measured at batch 1 to 64, 2,048 to 8,192 keys).
+    The matrix-core walk keeps the page ids of a whole slice in LDS: caches longer than that are cut
+    into as many slices as it takes."""
     matrix = kind != "valu" and hd > 0 and hd % 16 == 0 and hd <= 128
     gt = 8 if group >= 8 else (4 if group > 2 else group)
     per_split = n_rows * nkv * -(-group // gt)
+    least = max(1, -(-max_seq // (MATRIX_SLICE_PAGES * page_size - 256))) if matrix else 1
     if per_split >= 256:
-        return 1, (4 if matrix else 8)
+        return least, (4 if matrix else 8)
     want = -(-512 // per_split)
-    return max(1, min(want, max_seq // (128 if matrix else 64), 256)), 4
+    return max(least, min(want, max_seq // (128 if matrix else 64), 256)), 4
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
@@ -490,7 +497,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     assert table.dim() == 2 and table.shape[0] >= n_req
     _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
     if n_splits is None or waves is None:
-        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind)
+        auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind, page_size)
         n_splits = auto_splits if n_splits is None else n_splits
         waves = auto_waves if waves is None else waves
     partial = None

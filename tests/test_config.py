@@ -94,7 +94,7 @@ def test_round_trip_and_spec(name):
     assert all(l.ffn.params["inter"] == c.intermediate_size for l in spec.layers)
 
 
-def test_baseline_shapes():
+def test_1p2b_shape_and_parameter_count():
     c = config_from_dict(dict(architectures=["Lfm2ForCausalLM"], hidden_size=2048, num_hidden_layers=16,
                               num_attention_heads=32, num_key_value_heads=8, vocab_size=65536, block_ff_dim=12288,
                               block_auto_adjust_ff_dim=True, block_ffn_dim_multiplier=1.0, conv_L_cache=3,
