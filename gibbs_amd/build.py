@@ -1,4 +1,5 @@
-"""Builds the HIP kernels for gfx950 into one shared library and finds it again.
+"""Builds the HIP kernels for gfx950 into one shared library and finds it again; and the host
+runtime (cache accounting and step staging, plain C++) into a second one.
 
 The library lives in-tree (`gibbs_amd/_lib/libgibbs_hip.so`) beside a stamp of the sources it
 was built from.  `ensure_built()` returns the library if the stamp fits the sources; otherwise
@@ -25,6 +26,11 @@ ARCH = "gfx950"
 # not know the feature; that is harmless).
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+
+
+HOST_SRC = os.path.join(CSRC, "host")
+HOST_LIB_NAME = "libgibbs_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wall"]
 
 
 class BuildError(RuntimeError):
@@ -62,8 +68,8 @@ def _lib_dirs() -> list[str]:
     return [os.path.join(HERE, "_lib"), tmp]
 
 
-def _is_current(lib_dir: str, stamp: str) -> bool:
-    lib, st = os.path.join(lib_dir, LIB_NAME), os.path.join(lib_dir, LIB_NAME + ".stamp")
+def _is_current(lib_dir: str, stamp: str, name: str = LIB_NAME) -> bool:
+    lib, st = os.path.join(lib_dir, name), os.path.join(lib_dir, name + ".stamp")
     if not (os.path.isfile(lib) and os.path.isfile(st)):
         return False
     with open(st) as f:
@@ -127,6 +133,59 @@ def build(verbose: bool = True) -> str:
     return os.path.join(lib_dir, LIB_NAME)
 
 
+def host_sources() -> list[str]:
+    return sorted(glob.glob(os.path.join(HOST_SRC, "*.cpp")))
+
+
+def _host_stamp() -> str:
+    h = hashlib.sha256()
+    for path in host_sources():
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()
+
+
+def host_compiler() -> str | None:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"), hipcc()):
+        if cand and os.path.isfile(cand) and os.access(cand, os.X_OK):
+            return cand
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compiles the host runtime (no GPU code) into its library; always compiles."""
+    cxx = host_compiler()
+    if cxx is None:
+        raise BuildError("no C++ compiler found: the host runtime cannot be built (set CXX)")
+    lib_dir = next((d for d in _lib_dirs() if _writable(d)), None)
+    if lib_dir is None:
+        raise BuildError(f"no writable folder for the host runtime among {_lib_dirs()}")
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())
+    tmp_lib = os.path.join(lib_dir, f".{HOST_LIB_NAME}.{os.getpid()}")
+    t0 = time.time()
+    proc = subprocess.run([cxx, *HOST_FLAGS, *host_sources(), "-o", tmp_lib], capture_output=True, text=True, env=env)
+    if proc.returncode != 0:
+        raise BuildError(f"compiling the host runtime failed:\n{proc.stderr[-4000:]}")
+    os.replace(tmp_lib, os.path.join(lib_dir, HOST_LIB_NAME))
+    with open(os.path.join(lib_dir, HOST_LIB_NAME + ".stamp"), "w") as f:
+        f.write(_host_stamp())
+    if verbose:
+        _say(f"built {os.path.join(lib_dir, HOST_LIB_NAME)} ({time.time() - t0:.1f}s)")
+    return os.path.join(lib_dir, HOST_LIB_NAME)
+
+
+def ensure_host_built(verbose: bool = True) -> str:
+    """The path of a host runtime library that fits its sources; builds it when there is none."""
+    stamp = _host_stamp()
+    for d in _lib_dirs():
+        if _is_current(d, stamp, HOST_LIB_NAME):
+            return os.path.join(d, HOST_LIB_NAME)
+    return build_host(verbose=verbose)
+
+
 def ensure_built(verbose: bool = True) -> str:
     """The path of a library that fits the sources; builds it when there is none."""
     stamp = _stamp()
@@ -142,4 +201,5 @@ def ensure_built(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
+    build_host()
     build()

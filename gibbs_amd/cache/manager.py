@@ -18,26 +18,36 @@ a page holds.  The reference returns blocks on the same events
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 
+from . import host
 from .needs import CacheNeed, StateNeed
-from .pages import PageError, PagePool
+from .pages import PageError
 
 NO_PAGE = -1
 
 
-@dataclass
-class _Request:
-    slot: int
-    tokens: int = 0                                         # positions whose keys/state are cached
-    pages: Dict[int, List[int]] = field(default_factory=dict)   # group -> logical page -> id or NO_PAGE
+class _PoolView:
+    """What the rest of the package asks of a group's pool."""
+
+    def __init__(self, manager: "CacheManager", group: int, num_pages: int):
+        self._manager, self._group, self.num_pages = manager, group, num_pages
+
+    @property
+    def n_free(self) -> int:
+        return self._manager.free_pages(self._group)
+
+    @property
+    def n_held(self) -> int:
+        return self.num_pages - self.n_free
 
 
 class CacheManager:
-    """Host-side accounting.  Device tensors hang on `DeviceCache`, which reads this."""
+    """Host-side accounting, kept by the native core (csrc/host/cache_core.cpp); this class maps
+    request ids to the core's slots and turns its failure codes into exceptions.  Device tensors
+    hang on `DeviceCache`, which reads this."""
 
     def __init__(self, needs: Sequence[Optional[CacheNeed]], states: Sequence[Sequence[StateNeed]],
                  page_size: int, num_pages: int, max_requests: int):
@@ -59,7 +69,8 @@ class CacheManager:
             g = self.group_needs.index(need)
             self.group_layers[g].append(i)
             self.layer_group[i] = g
-        self.pools = [PagePool(num_pages) for _ in self.group_needs]
+        if self.group_needs and num_pages <= 0:
+            raise ValueError(f"a page pool needs at least one page, not {num_pages}")
         # state layout of a slot: (layer, name) -> (offset, shape), in float32 elements
         self.state_layout: Dict[Tuple[int, str], Tuple[int, Tuple[int, ...]]] = {}
         off = 0
@@ -70,131 +81,130 @@ class CacheManager:
                 self.state_layout[(i, s.name)] = (off, tuple(s.shape))
                 off += s.numel
         self.slot_floats = off
-        self._free_slots = list(range(max_requests - 1, -1, -1))
-        self._requests: Dict[Hashable, _Request] = {}
-        self.fresh_slots: List[int] = []            # slots taken since the device last cleared them
+        self._lib = host.library()
+        windows = host.ints([int(n.window or 0) for n in self.group_needs])
+        self._core = self._lib.gibbs_cache_create(len(self.group_needs), windows, page_size, max(1, num_pages),
+                                                  max_requests)
+        if not self._core:
+            raise ValueError("the cache core refused its sizes")
+        self.pools = [_PoolView(self, g, num_pages) for g in range(len(self.group_needs))]
+        self._slots: Dict[Hashable, int] = {}
+        self._needed = host.ints([0] * len(self.group_needs))
+
+    def __del__(self):
+        if getattr(self, "_core", None):
+            self._lib.gibbs_cache_destroy(self._core)
+            self._core = None
+
+    def _raise(self, code: int, rid: Hashable = None):
+        text = host.last_error()
+        if rid is not None:
+            text = f"request {rid!r}: {text}"
+        if code == host.ERR_PAGE:
+            raise PageError(text)
+        raise ValueError(text)
 
     # ------------------------------------------------------------------ queries
     @property
     def n_groups(self) -> int:
         return len(self.group_needs)
 
+    @property
+    def core(self):
+        """The native core (for the step staging of the engine)."""
+        return self._core
+
     def __contains__(self, rid: Hashable) -> bool:
-        return rid in self._requests
+        return rid in self._slots
 
     def live(self) -> List[Hashable]:
-        return list(self._requests)
+        return list(self._slots)
 
     def tokens(self, rid: Hashable) -> int:
-        return self._requests[rid].tokens
+        return self._lib.gibbs_cache_tokens(self._core, self._slots[rid])
 
     def slot(self, rid: Hashable) -> int:
-        return self._requests[rid].slot
+        return self._slots[rid]
 
     def free_pages(self, group: int = 0) -> int:
-        return self.pools[group].n_free
+        return self._lib.gibbs_cache_free_pages(self._core, group)
 
     def free_slots(self) -> int:
-        return len(self._free_slots)
+        return self._lib.gibbs_cache_free_slots(self._core)
 
     def pages_for(self, n_tokens: int) -> int:
         return -(-n_tokens // self.page_size)
 
     def pages_needed(self, rid: Hashable, n_new: int) -> List[int]:
         """Per group: pages that `reserve(rid, n_new)` would have to take."""
-        r = self._requests[rid]
-        want = self.pages_for(r.tokens + n_new)
-        return [max(0, want - len(r.pages[g])) for g in range(self.n_groups)]
+        self._lib.gibbs_cache_pages_needed(self._core, self._slots[rid], n_new, self._needed)
+        return list(self._needed[:self.n_groups])
 
     # ------------------------------------------------------------------ life of a request
     def admit(self, rid: Hashable) -> bool:
         """Gives the request a slot (cleared before the next step); False if none is free."""
-        if rid in self._requests:
+        if rid in self._slots:
             raise KeyError(f"request {rid!r} is already live")
-        if not self._free_slots:
+        slot = self._lib.gibbs_cache_admit(self._core)
+        if slot < 0:
             return False
-        slot = self._free_slots.pop()
-        self._requests[rid] = _Request(slot, 0, {g: [] for g in range(self.n_groups)})
-        self.fresh_slots.append(slot)
+        self._slots[rid] = slot
         return True
 
     def reserve(self, rid: Hashable, n_new: int) -> bool:
         """Pages for the next `n_new` positions in every group; all or nothing."""
-        r = self._requests[rid]
-        need = self.pages_needed(rid, n_new)
-        if any(n > self.pools[g].n_free for g, n in enumerate(need)):
+        code = self._lib.gibbs_cache_reserve(self._core, self._slots[rid], n_new)
+        if code == host.ERR_NO_ROOM:
             return False
-        for g, n in enumerate(need):
-            r.pages[g].extend(self.pools[g].allocate(n))
+        if code < 0:
+            self._raise(code, rid)
         return True
 
     def commit(self, rid: Hashable, n_new: int) -> None:
         """`n_new` more positions are cached now.  A window group gives back every page that
         no later query can see: page j holds positions [j*ps, (j+1)*ps), the next query is at
         position >= tokens and sees keys > tokens - window."""
-        r = self._requests[rid]
-        if self.pages_for(r.tokens + n_new) > min((len(p) for p in r.pages.values()), default=1 << 60):
-            raise PageError(f"request {rid!r}: commit of {n_new} tokens beyond its reserved pages")
-        r.tokens += n_new
-        for g, need in enumerate(self.group_needs):
-            if need.window is None:
-                continue
-            first_visible = r.tokens - need.window + 1
-            passed = max(0, first_visible // self.page_size)
-            pages = r.pages[g]
-            gone = [p for p in pages[:passed] if p != NO_PAGE]
-            if gone:
-                self.pools[g].release(gone)
-                for j in range(min(passed, len(pages))):
-                    pages[j] = NO_PAGE
+        code = self._lib.gibbs_cache_commit(self._core, self._slots[rid], n_new)
+        if code < 0:
+            self._raise(code, rid)
 
     def release(self, rid: Hashable) -> None:
         """Gives back every page and the slot of a request that ended."""
-        r = self._requests.pop(rid)
-        for g, pages in r.pages.items():
-            self.pools[g].release([p for p in pages if p != NO_PAGE])
-        self._free_slots.append(r.slot)
+        slot = self._slots.pop(rid)
+        code = self._lib.gibbs_cache_release(self._core, slot)
+        if code < 0:
+            self._raise(code, rid)
 
     # ------------------------------------------------------------------ what kernels read
+    def slots_of(self, rids: Sequence[Hashable]):
+        return host.ints([self._slots[r] for r in rids])
+
     def table_width(self, rids: Sequence[Hashable], group: int) -> int:
-        return max((len(self._requests[r].pages[group]) for r in rids), default=0)
+        return max(0, self._lib.gibbs_cache_table_width(self._core, self.slots_of(rids), len(rids), group))
 
     def block_table(self, rids: Sequence[Hashable], group: int, width: Optional[int] = None) -> np.ndarray:
         """int32 [len(rids), width]: page id of logical page j of each request (NO_PAGE beyond
         its pages and for pages a window has passed)."""
         width = max(1, self.table_width(rids, group)) if width is None else width
-        out = np.full((len(rids), width), NO_PAGE, dtype=np.int32)
-        for i, rid in enumerate(rids):
-            pages = self._requests[rid].pages[group]
-            if len(pages) > width:
-                raise ValueError(f"request {rid!r} holds {len(pages)} pages, table width is {width}")
-            out[i, :len(pages)] = pages
+        out = np.empty((len(rids), width), dtype=np.int32)
+        code = self._lib.gibbs_cache_block_table(self._core, self.slots_of(rids), len(rids), group, width,
+                                                 out.ctypes.data)
+        if code < 0:
+            self._raise(code)
         return out
 
     def take_fresh_slots(self) -> List[int]:
-        out, self.fresh_slots = self.fresh_slots, []
-        return out
+        out = host.ints([0] * self.max_requests)
+        n = self._lib.gibbs_cache_take_fresh_slots(self._core, out, self.max_requests)
+        return list(out[:n])
 
     # ------------------------------------------------------------------ invariants (tests)
     def check(self) -> None:
-        """No page lost, held twice or free while held; no slot shared."""
-        for g, pool in enumerate(self.pools):
-            owners: Dict[int, Hashable] = {}
-            for rid, r in self._requests.items():
-                for p in r.pages[g]:
-                    if p == NO_PAGE:
-                        continue
-                    if p in owners:
-                        raise PageError(f"group {g}: page {p} held by {owners[p]!r} and {rid!r}")
-                    if not pool.is_held(p):
-                        raise PageError(f"group {g}: page {p} of {rid!r} is on the free list")
-                    owners[p] = rid
-            if len(owners) != pool.n_held:
-                raise PageError(f"group {g}: {pool.n_held} pages held, {len(owners)} owned: a page was lost")
-            if len(set(pool._free)) != len(pool._free):
-                raise PageError(f"group {g}: a page is on the free list twice")
-        slots = [r.slot for r in self._requests.values()]
-        if len(set(slots)) != len(slots) or set(slots) & set(self._free_slots):
-            raise PageError("a slot is shared or free while held")
-        if len(slots) + len(self._free_slots) != self.max_requests:
+        """No page lost, held twice or free while held; no slot shared or lost."""
+        code = self._lib.gibbs_cache_check(self._core)
+        if code < 0:
+            self._raise(code)
+        if len(set(self._slots.values())) != len(self._slots):
+            raise PageError("two requests share a slot")
+        if len(self._slots) + self.free_slots() != self.max_requests:
             raise PageError("a slot was lost")

@@ -5,10 +5,14 @@ a free list that allocation pops and release pushes), without its reference coun
 prefix tree: a page here belongs to at most one request.  Unlike the reference, whose block
 ids are bookkeeping only (/root/reference/src/scheduler/mod.rs:215), these ids index real
 device pages that the attention kernels read through a block table.
+
+The pool itself is native code (csrc/host/cache_core.cpp); this class is its handle.
 """
 from __future__ import annotations
 
 from typing import Iterable, List, Optional
+
+from . import host
 
 
 class PageError(RuntimeError):
@@ -20,37 +24,34 @@ class PagePool:
         if num_pages <= 0:
             raise ValueError(f"a page pool needs at least one page, not {num_pages}")
         self.num_pages = num_pages
-        # LIFO: a page that was just given back is the next to be used again.
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))
-        self._held = [False] * num_pages
+        self._lib = host.library()
+        self._pool = self._lib.gibbs_pool_create(num_pages)
+
+    def __del__(self):
+        if getattr(self, "_pool", None):
+            self._lib.gibbs_pool_destroy(self._pool)
+            self._pool = None
 
     @property
     def n_free(self) -> int:
-        return len(self._free)
+        return self._lib.gibbs_pool_free(self._pool)
 
     @property
     def n_held(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.n_free
 
     def allocate(self, n: int) -> Optional[List[int]]:
         """`n` pages, or None (and nothing taken) if fewer are free."""
         if n < 0:
             raise ValueError("cannot allocate a negative number of pages")
-        if n > len(self._free):
-            return None
-        out = [self._free.pop() for _ in range(n)]
-        for p in out:
-            self._held[p] = True
-        return out
+        out = host.ints([0] * n)
+        got = self._lib.gibbs_pool_allocate(self._pool, n, out)
+        return None if got < 0 else list(out[:n])
 
     def release(self, pages: Iterable[int]) -> None:
-        for p in pages:
-            if not 0 <= p < self.num_pages:
-                raise PageError(f"page {p} is not of this pool (0..{self.num_pages - 1})")
-            if not self._held[p]:
-                raise PageError(f"page {p} freed twice or never held")
-            self._held[p] = False
-            self._free.append(p)
+        pages = list(pages)
+        if self._lib.gibbs_pool_release(self._pool, host.ints(pages), len(pages)) < 0:
+            raise PageError(host.last_error())
 
     def is_held(self, page: int) -> bool:
-        return self._held[page]
+        return bool(self._lib.gibbs_pool_is_held(self._pool, page))

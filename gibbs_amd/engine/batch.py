@@ -7,6 +7,7 @@ as rows cu[r] .. cu[r+1] of every activation.  Prompt portions (q_len > 1) and d
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass, field
 from typing import Hashable, List, Optional, Sequence
 
@@ -69,6 +70,32 @@ class BatchStager:
             self._host[i] = torch.empty(cap, dtype=torch.int32, pin_memory=True)
             self._dev[i] = torch.empty(cap, dtype=torch.int32, device=self.device)
         return i, self._host[i], self._dev[i]
+
+    def stage_native(self, lib, core, operands, info, widths: Sequence[int], n_logits: int) -> StepBatch:
+        """The host runtime packs the step (entries as `operands` of `gibbs_cache_fill_step`, sizes as
+        `info` from its reservation) straight into the pinned buffer; one copy takes it to the device."""
+        n, slots_ptr, q_len_ptr = operands[0], operands[1], operands[2]
+        total = int(info[0])
+        i, host_buf, dev = self._buffers(total)
+        offsets = (ctypes.c_long * (9 + len(widths)))()
+        if lib.gibbs_cache_fill_step(core, *operands, info, host_buf.data_ptr(), offsets) < 0:
+            raise RuntimeError(lib.gibbs_host_last_error().decode(errors="replace"))
+        dev[:total].copy_(host_buf[:total], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._events[i] = ev
+        view = host_buf.numpy()
+        q_lens = np.ctypeslib.as_array(ctypes.cast(q_len_ptr, ctypes.POINTER(ctypes.c_int)), (n,)).tolist()
+        rows = sum(q_lens)
+        sizes = [rows, rows, rows, n + 1, n, n, n_logits] + [n * w for w in widths]
+        sec = [dev[int(o):int(o) + size] for o, size in zip(offsets, sizes)]
+        return StepBatch(
+            n_rows=rows, n_req=n, n_logits=n_logits,
+            ids=sec[0], pos=sec[1], row_req=sec[2], cu=sec[3], ctx=sec[4], slot=sec[5], logit_rows=sec[6],
+            tables=[t.view(n, w) for t, w in zip(sec[7:], widths)],
+            q_lens=q_lens, ctx_lens=view[int(offsets[4]):int(offsets[4]) + n].tolist(),
+            slots=view[int(offsets[5]):int(offsets[5]) + n].tolist(),
+            max_q=int(offsets[7 + len(widths)]), max_seq=int(offsets[8 + len(widths)]))
 
     def stage(self, ids: np.ndarray, pos: np.ndarray, row_req: np.ndarray, cu: np.ndarray, ctx: np.ndarray,
               slot: np.ndarray, logit_rows: np.ndarray, tables: Sequence[np.ndarray]) -> StepBatch:

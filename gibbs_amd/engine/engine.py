@@ -9,13 +9,15 @@ the reference's (lm.rs:528-544): no empty token list, no position beyond the con
 """
 from __future__ import annotations
 
+import ctypes
+import itertools
 import os
 from typing import Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 import torch
 
-from ..cache import CacheManager, DeviceCache
+from ..cache import CacheManager, DeviceCache, host
 from ..config import config_from_dict, read_config_json
 from ..config.base import ArchConfig
 from ..ops.lib import KernelError, library
@@ -88,63 +90,51 @@ class Engine:
 
     # ------------------------------------------------------------------ the step function
     def prepare(self, entries: Sequence[Entry]) -> StepBatch:
-        """Checks the entries, takes slots and pages for them and stages the batch's metadata."""
+        """Checks the entries, takes slots and pages for them (all or nothing for the whole step)
+        and stages the batch's metadata.  The checks, the page accounting and the packing of the
+        staging buffer run in the host runtime (csrc/host/cache_core.cpp)."""
         if not entries:
             raise StepError("a step needs at least one entry")
-        seen = set()
-        vocab = self.spec.vocab
-        token_arrays = []
-        for e in entries:
-            if e.rid in seen:
-                raise StepError(f"request {e.rid!r} appears twice in one step")
-            seen.add(e.rid)
-            if len(e.tokens) == 0:
-                raise StepError(f"request {e.rid!r}: no tokens")
-            toks = np.asarray(e.tokens, dtype=np.int64)
-            token_arrays.append(toks)
-            if toks.min() < 0 or toks.max() >= vocab:
-                bad = int(toks[(toks < 0) | (toks >= vocab)][0])
-                raise StepError(f"request {e.rid!r}: token id {bad} outside the vocabulary (0..{vocab - 1})")
-            if any(not 0 <= w < len(e.tokens) for w in e.want):
-                raise StepError(f"request {e.rid!r}: wanted place outside its {len(e.tokens)} tokens")
-            before = self.cache.tokens(e.rid) if e.rid in self.cache else 0
-            if before + len(e.tokens) > self.ctx_limit:
-                raise StepError(f"request {e.rid!r}: {before + len(e.tokens)} tokens exceed the context limit {self.ctx_limit}")
-        # slots and pages: all or nothing for the whole step
-        admitted, reserved = [], []
+        cache, lib = self.cache, host.library()
+        n = len(entries)
+        if len({e.rid for e in entries}) != n:
+            twice = next(e.rid for i, e in enumerate(entries) if any(o.rid == e.rid for o in entries[:i]))
+            raise StepError(f"request {twice!r} appears twice in one step")
+        admitted = []
         try:
             for e in entries:
-                if e.rid not in self.cache:
-                    if not self.cache.admit(e.rid):
-                        raise OutOfPages(f"no free slot for request {e.rid!r} ({self.cache.max_requests} live)")
+                if e.rid not in cache:
+                    if not cache.admit(e.rid):
+                        raise OutOfPages(f"no free slot for request {e.rid!r} ({cache.max_requests} live)")
                     admitted.append(e.rid)
-            need = [0] * self.cache.n_groups
-            for e in entries:
-                for g, n in enumerate(self.cache.pages_needed(e.rid, len(e.tokens))):
-                    need[g] += n
-            for g, n in enumerate(need):
-                if n > self.cache.free_pages(g):
-                    raise OutOfPages(f"the step needs {n} pages of cache group {g}, {self.cache.free_pages(g)} are free")
-            for e in entries:
-                assert self.cache.reserve(e.rid, len(e.tokens))
-        except OutOfPages:
+            slots = np.fromiter((cache.slot(e.rid) for e in entries), dtype=np.int32, count=n)
+            q_len = np.fromiter((len(e.tokens) for e in entries), dtype=np.int32, count=n)
+            try:
+                tokens = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int32,
+                                     count=int(q_len.sum()))
+            except (OverflowError, TypeError, ValueError) as exc:
+                raise StepError(f"token ids must be integers that fit 32 bits: {exc}") from None
+            want_cu = np.zeros(n + 1, dtype=np.int32)
+            np.cumsum([len(e.want) for e in entries], out=want_cu[1:])
+            want = np.fromiter(itertools.chain.from_iterable(e.want for e in entries), dtype=np.int32,
+                               count=int(want_cu[-1]))
+            info = (ctypes.c_long * (1 + cache.n_groups))()
+            bad = ctypes.c_int(0)
+            operands = (n, slots.ctypes.data, q_len.ctypes.data, tokens.ctypes.data, want_cu.ctypes.data,
+                        want.ctypes.data)
+            code = lib.gibbs_cache_reserve_step(cache.core, *operands, self.spec.vocab, self.ctx_limit, info,
+                                                ctypes.byref(bad))
+            if code == host.ERR_NO_ROOM:
+                raise OutOfPages(host.last_error())
+            if code < 0:
+                raise StepError(f"request {entries[bad.value].rid!r}: {host.last_error()}")
+        except (OutOfPages, StepError):
             for rid in admitted:
-                self.cache.release(rid)
+                cache.release(rid)
             raise
-
-        rids = [e.rid for e in entries]
-        q_lens = np.array([len(e.tokens) for e in entries], dtype=np.int32)
-        cu = np.zeros(len(entries) + 1, dtype=np.int32)
-        np.cumsum(q_lens, out=cu[1:])
-        ctx = np.array([self.cache.tokens(r) for r in rids], dtype=np.int32)
-        slot = np.array([self.cache.slot(r) for r in rids], dtype=np.int32)
-        ids = np.concatenate(token_arrays).astype(np.int32)
-        row_req = np.repeat(np.arange(len(entries), dtype=np.int32), q_lens)
-        pos = (np.arange(ids.size, dtype=np.int32) - cu[:-1][row_req]) + ctx[row_req]
-        logit_rows = np.array([cu[i] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int32)
-        tables = [self.cache.block_table(rids, g) for g in range(self.cache.n_groups)]
         self.device_cache.clear_fresh_slots()
-        return self._stager.stage(ids, pos.astype(np.int32), row_req, cu, ctx, slot, logit_rows, tables)
+        widths = [int(info[1 + g]) for g in range(cache.n_groups)]
+        return self._stager.stage_native(lib, cache.core, operands, info, widths, int(want_cu[-1]))
 
     def step(self, entries: Sequence[Entry]) -> Optional[torch.Tensor]:
         """Runs one batch; returns float32 logits [wanted places, vocab] in the order of the

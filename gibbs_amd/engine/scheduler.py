@@ -52,7 +52,7 @@ class FinishReason(Enum):           # scheduler/mod.rs:450-458
     ERROR = "error"
 
 
-@dataclass
+@dataclass(eq=False)         # a request is itself: membership tests compare identity, not token lists
 class Sequence:
     id: Hashable
     prompt_tokens: List[int]
@@ -67,6 +67,19 @@ class Sequence:
     @property
     def tokens(self) -> List[int]:
         return self.prompt_tokens + self.output_tokens
+
+    @property
+    def n_tokens(self) -> int:
+        return len(self.prompt_tokens) + len(self.output_tokens)
+
+    def span(self, at: int, n: int) -> List[int]:
+        """tokens[at : at + n] without joining the two lists."""
+        p = len(self.prompt_tokens)
+        if at >= p:
+            return self.output_tokens[at - p:at - p + n]
+        if at + n <= p:
+            return self.prompt_tokens[at:at + n]
+        return self.prompt_tokens[at:] + self.output_tokens[:at + n - p]
 
 
 @dataclass
@@ -185,7 +198,7 @@ class ContinuousBatchScheduler:
                 self._finish(seq, FinishReason.LENGTH)              # scheduler/mod.rs:1357-1359
                 finished.append(seq.id)
                 continue
-            total = len(seq.tokens)
+            total = seq.n_tokens
             if self.cache.pages_for(total + 1) > min((p.num_pages for p in self.cache.pools), default=1 << 60):
                 self.waiting.popleft()
                 self._finish(seq, FinishReason.ERROR,
@@ -260,8 +273,8 @@ class ContinuousBatchScheduler:
         prefill_tokens = decode_tokens = 0
         for seq, n in plan:
             at = self._computed(seq)
-            toks = seq.tokens[at:at + n]
-            last = at + n == len(seq.tokens)
+            toks = seq.span(at, n)
+            last = at + n == seq.n_tokens
             entries.append(Entry(seq.id, toks, [n - 1] if last else []))
             if last:
                 draws.append(Draw(seq.params, seq.id, len(seq.output_tokens)))
@@ -291,7 +304,7 @@ class ContinuousBatchScheduler:
                 seq.output_tokens.append(int(tok))
                 emitted.append((seq.id, int(tok)))
                 if (len(seq.output_tokens) >= seq.params.max_new_tokens
-                        or len(seq.tokens) >= self.context_len):
+                        or seq.n_tokens >= self.context_len):
                     self._finish(seq, FinishReason.LENGTH)
                     finished.append(seq.id)
         return StepOutput(entries, emitted, finished, preempted, prefill_tokens, decode_tokens,
@@ -308,7 +321,7 @@ class ContinuousBatchScheduler:
         if any(s.state != SequenceState.DECODING or self._remaining(s) != 1 for s in self.active):
             return None
         seqs = sorted(self.active, key=lambda s: s.submitted)
-        n = min(cap, min(min(s.params.max_new_tokens - len(s.output_tokens), self.context_len - len(s.tokens))
+        n = min(cap, min(min(s.params.max_new_tokens - len(s.output_tokens), self.context_len - s.n_tokens)
                          for s in seqs))
         return (seqs, n) if n >= 1 else None
 
@@ -327,7 +340,7 @@ class ContinuousBatchScheduler:
                 seq.output_tokens.append(int(tok))
                 emitted.append((seq.id, int(tok)))
                 if (len(seq.output_tokens) >= seq.params.max_new_tokens
-                        or len(seq.tokens) >= self.context_len):
+                        or seq.n_tokens >= self.context_len):
                     self._finish(seq, FinishReason.LENGTH)
                     finished.append(seq.id)
                     break
