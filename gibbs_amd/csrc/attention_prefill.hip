@@ -14,7 +14,12 @@
 // Keys come from the request's pages through its block table; row n sees keys lo .. pos[n]
 // (lo = max(0, pos - window + 1), window 0 = all).  The step's own keys were written to the pages
 // before this kernel runs.  Head sizes: multiples of 16 up to 128.
+//
+// Few rows over a long cache (a prompt portion late in a long prompt) give too few workgroups to fill
+// the chip: the key tiles of a workgroup's rows are then cut into n_splits slices that run as
+// workgroups of their own (grid z) and leave (max, sum, weighted values) for the merge kernel.
 #include "common.h"
+#include "attention_merge.h"
 
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -59,6 +64,7 @@ struct PrefillArgs {
   long ldq, ldo;
   float scale;
   int window;
+  int n_splits;    // slices of the key tiles (1: the workgroup writes the finished rows)
 };
 
 // DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
@@ -67,7 +73,7 @@ template <int DT, bool POW2>
 __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __restrict__ q,
                                                                 const bf16* __restrict__ kpages,
                                                                 const bf16* __restrict__ vpages, bf16* __restrict__ out,
-                                                                PrefillArgs a) {
+                                                                float* __restrict__ partial, PrefillArgs a) {
   constexpr int HD = 16 * DT;
   constexpr int DS = (DT + 1) / 2;  // steps of 32 over d
   constexpr int LDK = HD + 8;
@@ -170,15 +176,23 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     __syncthreads();
   };
 
-  const int kt_first = first_key / BN;
-  load_segment(kt_first * BN);
-  load_tile(kt_first * BN);
-  for (int kt = kt_first; kt * BN <= last_pos; ++kt) {
+  // this workgroup's slice of the key tiles first_key / BN .. last_pos / BN
+  int kt_first = first_key / BN, kt_stop = last_pos / BN + 1;
+  if (a.n_splits > 1) {
+    const int per = (kt_stop - kt_first + a.n_splits - 1) / a.n_splits;
+    kt_first += blockIdx.z * per;
+    kt_stop = min(kt_stop, kt_first + per);
+  }
+  if (kt_first < kt_stop) {
+    load_segment(kt_first * BN);
+    load_tile(kt_first * BN);
+  }
+  for (int kt = kt_first; kt < kt_stop; ++kt) {
     const int key0 = kt * BN;
     __syncthreads();  // everyone is done with the previous tile
     store_tile();
     __syncthreads();
-    if ((kt + 1) * BN <= last_pos) {
+    if (kt + 1 < kt_stop) {
       if (((kt + 1) * BN) % seg_keys == 0) load_segment((kt + 1) * BN);  // (uniform: everyone takes it)
       load_tile((kt + 1) * BN);
     }
@@ -254,6 +268,22 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   // row sum over the 4 lanes that share the row; store d = t*16 + g*4 .. +4 of row lr
   l = row4_sum(l);
   const int row = wave * 16 + lr;
+  if (a.n_splits > 1) {
+    // (max of the scaled scores, sum, weighted values) of this slice; a slice without keys leaves a
+    // maximum far below any score and zeros, which the merge weighs with exp(-huge) = 0
+    if (row < rows_here) {
+      float* ps = partial + (((size_t)(n0 + row) * a.nh + head) * a.n_splits + blockIdx.z) * (HD + 2);
+      if (g == 0) {
+        ps[0] = m * a.scale;
+        ps[1] = l;
+      }
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ps[2 + t * 16 + g * 4 + i] = o[t][i];
+    }
+    return;
+  }
   if (row < rows_here) {
     const float inv = 1.0f / l;
     bf16* dst = out + (size_t)(n0 + row) * a.ldo + (size_t)head * HD + g * 4;
@@ -271,18 +301,22 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   }
 }
 template <int DT>
-void launch_prefill(dim3 grid, hipStream_t stream, const bf16* q, const bf16* k, const bf16* v, bf16* out, const PrefillArgs& a) {
-  if (a.page_shift >= 0) attention_prefill_kernel<DT, true><<<grid, 256, 0, stream>>>(q, k, v, out, a);
-  else attention_prefill_kernel<DT, false><<<grid, 256, 0, stream>>>(q, k, v, out, a);
+void launch_prefill(dim3 grid, hipStream_t stream, const bf16* q, const bf16* k, const bf16* v, bf16* out, float* partial,
+                    const PrefillArgs& a) {
+  if (a.page_shift >= 0) attention_prefill_kernel<DT, true><<<grid, 256, 0, stream>>>(q, k, v, out, partial, a);
+  else attention_prefill_kernel<DT, false><<<grid, 256, 0, stream>>>(q, k, v, out, partial, a);
 }
 }  // namespace
 
 // q: [N, >= nh*hd] bfloat16 (row stride ldq), rows of request r are cu[r] .. cu[r+1] at positions
 // ctx[r] ..; pages: [num_pages, nkv, page_size, hd]; out: [N, nh*hd] (row stride ldo).
-GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out,
+// n_splits > 1: the key tiles of every workgroup's rows are cut into that many slices; partial is a
+// workspace of (first_row + n_rows) * nh * n_splits * (hd + 2) floats.  cu may start above 0 (the requests
+// of a step from some request on): first_row = cu[0] then, and n_rows counts the rows from there.
+GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
                                          const int* cu, const int* ctx, const int* table, int n_req, int max_pages,
                                          int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                         long ldo, float scale, int window, hipStream_t stream) {
+                                         long ldo, float scale, int window, int n_splits, int first_row, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && n_req >= 0 && nh > 0 && nkv > 0, "attention_prefill: bad sizes rows=%d requests=%d heads=%d kv=%d", n_rows, n_req, nh, nkv);
   GIBBS_REQUIRE(nh % nkv == 0, "attention_prefill: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd % 16 == 0 && hd >= 16 && hd <= 128, "attention_prefill: head size %d must be a multiple of 16 up to 128", hd);
@@ -290,21 +324,30 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
   GIBBS_REQUIRE(ldq >= (long)nh * hd && ldo >= (long)nh * hd, "attention_prefill: row strides shorter than heads * hd");
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention_prefill: bad cache geometry");
   GIBBS_REQUIRE(nh <= 65535, "attention_prefill: too many heads (%d)", nh);
+  GIBBS_REQUIRE(first_row >= 0, "attention_prefill: negative first row");
+  GIBBS_REQUIRE(n_splits >= 1 && n_splits <= 65535 && (n_splits == 1 || partial), "attention_prefill: %d key slices need a workspace", n_splits);
   if (n_rows == 0 || n_req == 0) return 0;
   const int page_shift = (page_size & (page_size - 1)) == 0 ? __builtin_ctz(page_size) : -1;
-  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window};
-  dim3 grid(ceil_div(n_rows, BM) + n_req, nh);
+  PrefillArgs a{cu, ctx, table, n_req, max_pages, page_size, num_pages, page_shift, nh, nkv, hd, ldq, ldo, scale, window, n_splits};
+  dim3 grid(ceil_div(n_rows, BM) + n_req, nh, n_splits);
   const bf16 *qq = (const bf16*)q, *kk = (const bf16*)kpages, *vv = (const bf16*)vpages;
   bf16* oo = (bf16*)out;
   switch (hd / 16) {
-    case 1: launch_prefill<1>(grid, stream, qq, kk, vv, oo, a); break;
-    case 2: launch_prefill<2>(grid, stream, qq, kk, vv, oo, a); break;
-    case 3: launch_prefill<3>(grid, stream, qq, kk, vv, oo, a); break;
-    case 4: launch_prefill<4>(grid, stream, qq, kk, vv, oo, a); break;
-    case 5: launch_prefill<5>(grid, stream, qq, kk, vv, oo, a); break;
-    case 6: launch_prefill<6>(grid, stream, qq, kk, vv, oo, a); break;
-    case 7: launch_prefill<7>(grid, stream, qq, kk, vv, oo, a); break;
-    default: launch_prefill<8>(grid, stream, qq, kk, vv, oo, a); break;
+    case 1: launch_prefill<1>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 2: launch_prefill<2>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 3: launch_prefill<3>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 4: launch_prefill<4>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 5: launch_prefill<5>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 6: launch_prefill<6>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    case 7: launch_prefill<7>(grid, stream, qq, kk, vv, oo, partial, a); break;
+    default: launch_prefill<8>(grid, stream, qq, kk, vv, oo, partial, a); break;
+  }
+  if (n_splits > 1) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return gibbs_fail("attention_prefill: %s", hipGetErrorString(e));
+    dim3 mgrid(n_rows, ceil_div(nh, 4));
+    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial + (size_t)first_row * nh * n_splits * (hd + 2),
+                                                      oo + (size_t)first_row * ldo, nh, hd, n_splits, ldo);
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
 }

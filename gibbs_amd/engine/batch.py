@@ -43,7 +43,17 @@ class StepBatch:
     slots: List[int] = field(default_factory=list)
     max_q: int = 0
     max_seq: int = 0
+    lead_single: int = 0         # requests at the head of the batch that bring one token each (decoded tokens)
     decode_graph: bool = False   # metadata lives in static buffers that a captured graph replays over
+
+
+def leading_single(q_lens: Sequence[int]) -> int:
+    n = 0
+    for q in q_lens:
+        if q != 1:
+            break
+        n += 1
+    return n
 
 
 class BatchStager:
@@ -95,7 +105,8 @@ class BatchStager:
             tables=[t.view(n, w) for t, w in zip(sec[7:], widths)],
             q_lens=q_lens, ctx_lens=view[int(offsets[4]):int(offsets[4]) + n].tolist(),
             slots=view[int(offsets[5]):int(offsets[5]) + n].tolist(),
-            max_q=int(offsets[7 + len(widths)]), max_seq=int(offsets[8 + len(widths)]))
+            max_q=int(offsets[7 + len(widths)]), max_seq=int(offsets[8 + len(widths)]),
+            lead_single=leading_single(q_lens))
 
     def stage(self, ids: np.ndarray, pos: np.ndarray, row_req: np.ndarray, cu: np.ndarray, ctx: np.ndarray,
               slot: np.ndarray, logit_rows: np.ndarray, tables: Sequence[np.ndarray]) -> StepBatch:
@@ -121,4 +132,5 @@ class BatchStager:
             ids=sec[0], pos=sec[1], row_req=sec[2], cu=sec[3], ctx=sec[4], slot=sec[5], logit_rows=sec[6],
             tables=[s.view(t.shape) for s, t in zip(sec[7:], tables)],
             q_lens=q_lens.tolist(), ctx_lens=ctx.tolist(), slots=slot.tolist(),
-            max_q=int(q_lens.max()) if n_req else 0, max_seq=int((ctx + q_lens).max()) if n_req else 0)
+            max_q=int(q_lens.max()) if n_req else 0, max_seq=int((ctx + q_lens).max()) if n_req else 0,
+            lead_single=leading_single(q_lens.tolist()))

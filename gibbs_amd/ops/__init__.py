@@ -512,12 +512,27 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     return out
 
 
+def prefill_splits(n_tiles: int, nh: int, max_seq: int, window: Optional[int] = None) -> int:
+    """Slices of the key tiles for the prompt attention: none while the query tiles and heads fill the
+    chip by themselves (about three workgroups per compute unit); else enough to get there, with at
+    least four tiles of 64 keys to a slice."""
+    blocks = max(1, n_tiles * nh)
+    keys = max_seq if not window else min(max_seq, int(window) + 64)
+    if blocks >= 768 or keys < 8 * 64:
+        return 1
+    return max(1, min(-(-1024 // blocks), keys // 256, 16))
+
+
 def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                       vpages: torch.Tensor, table: torch.Tensor, n_req: int, cu: torch.Tensor, ctx: torch.Tensor,
-                      scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                      max_seq: int = 0, n_splits: Optional[int] = None, first_req: int = 0,
+                      first_row: int = 0) -> torch.Tensor:
     """bfloat16 paged causal attention for prompt portions on the matrix cores: rows cu[r] .. cu[r+1]
     of request r sit at positions ctx[r] ..; same result as `attention_plain`.  Head sizes: multiples
-    of 16 up to 128."""
+    of 16 up to 128.  `max_seq`: a bound on the keys of any row, from which the number of key slices
+    is chosen (or `n_splits`).  `first_req`, `first_row`: only the requests from `first_req` on are
+    attended to (their rows start at `first_row`); the rows before are left as they are in `out`."""
     require_cuda(q, kpages, vpages, table, cu, ctx)
     if q.dtype != torch.bfloat16:
         raise KernelError("attention_prefill is the bfloat16 kernel; the float32 path uses attention_plain")
@@ -528,12 +543,19 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
     assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
     assert table.dim() == 2 and table.shape[0] >= n_req
     _i32(table, n_req, "block table"); _i32(cu, n_req + 1, "cu"); _i32(ctx, n_req, "ctx")
+    assert 0 <= first_req <= n_req and 0 <= first_row <= n_rows
     if out is None:
         out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
-    call("gibbs_attention_prefill", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(cu), ptr(ctx), ptr(table), n_req,
-         table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd, q.stride(0) if n_rows > 1 else q.shape[1], nh * hd,
-         float(scale), int(window or 0), stream())
+    rows, reqs = n_rows - first_row, n_req - first_req
+    if n_splits is None:
+        n_splits = prefill_splits(-(-rows // 64) + reqs // 2, nh, max_seq, window) if max_seq > 0 else 1
+    partial = None
+    if n_splits > 1:
+        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=q.device)
+    call("gibbs_attention_prefill", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(cu[first_req:]),
+         ptr(ctx[first_req:]), ptr(table[first_req:]), reqs, table.shape[1], page_size, num_pages, rows, nh, nkv, hd,
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), int(n_splits), int(first_row), stream())
     return out
 
 

@@ -21,6 +21,9 @@ from ..weights.loader import FLOAT32, TensorDecl, WeightStore
 from .base import Mixer, Runtime, build_position, register_mixer
 
 
+MIN_LEADING_DECODED = 2      # decoded tokens at the head of a mixed step that are worth a kernel of their own
+
+
 @register_mixer("attention")
 class AttentionMixer(Mixer):
     def __init__(self, spec, hidden, layer_index):
@@ -143,8 +146,17 @@ class AttentionMixer(Mixer):
         plain kernel."""
         bf16 = self.rt.act_dtype == torch.bfloat16
         if bf16 and batch.max_q > 1 and self.head_dim % 16 == 0 and self.head_dim <= 128:
+            # decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that
+            # splits their keys; a row of its own in the matrix-core kernel would walk its cache alone
+            lead = batch.lead_single if batch.lead_single >= MIN_LEADING_DECODED else 0
+            out = torch.empty((batch.n_rows, self.heads * self.head_dim), dtype=qkv.dtype, device=qkv.device)
+            if lead:
+                ops.attention_decode(qkv[:lead], lead, self.heads, self.kv_heads, self.head_dim, cache.kpages,
+                                     cache.vpages, table, batch.n_req, batch.pos[:lead], batch.row_req[:lead],
+                                     self.scale, self.window, max_seq=batch.max_seq, out=out[:lead])
             return ops.attention_prefill(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
-                                         cache.vpages, table, batch.n_req, batch.cu, batch.ctx, self.scale, self.window)
+                                         cache.vpages, table, batch.n_req, batch.cu, batch.ctx, self.scale, self.window,
+                                         out=out, max_seq=batch.max_seq, first_req=lead, first_row=lead)
         if bf16 and batch.max_q == 1 and self.head_dim % 8 == 0:
             return ops.attention_decode(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
                                         cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,

@@ -303,13 +303,15 @@ def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves,
     close(out, plain, dtype, "decode vs plain kernel", bf16=1e-2)
 
 
+@pytest.mark.parametrize("n_splits", [1, 3, 7])
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
                                                    (32, 8, 64, 16, None), (4, 2, 128, 16, None), (2, 2, 96, 64, 100),
                                                    (3, 1, 32, 16, 5)])
-def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window):
+def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window, n_splits):
     """Prompt portions on the matrix cores: a long portion after a cached context that ends off a
     tile edge, a whole short prompt, a 2-token portion, a single decoded row and a 65-row portion
-    that starts at position 0, all in one call."""
+    that starts at position 0, all in one call; with the key tiles whole or cut into slices (more
+    slices than the short requests have tiles: slices without keys)."""
     from gibbs_amd import ops
     dtype = torch.bfloat16
     seq_lens = [333, 9, 130, 77, 65]
@@ -320,7 +322,7 @@ def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window):
     n = int(cu[-1])
     q = rnd(n, nh * hd, dtype=dtype, seed=9)
     scale = 1 / math.sqrt(hd)
-    out = ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window)
+    out = ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window, n_splits=n_splits)
     pos = i32([c + t for c, ql in zip(ctx, q_lens) for t in range(ql)])
     row_req = i32([r for r, ql in enumerate(q_lens) for _ in range(ql)])
     plain = ops.attention_plain(q, n, nh, nkv, hd, kp, vp, table, 5, pos, row_req, scale, window)
@@ -329,6 +331,20 @@ def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window):
         want = attention_reference(q[rows].view(-1, nh, hd), ks[r], vs[r], list(range(ctx[r], seq_lens[r])), scale, window)
         close(out[rows].view(-1, nh, hd), want, dtype, f"prefill attention request {r}", bf16=1e-2)
     close(out, plain, dtype, "prefill vs plain kernel", bf16=1e-2)
+    # only the requests from the third on: the rows before them stay as they were
+    first_req, first_row = 2, int(cu[2])
+    part = torch.full_like(out, 7.0)
+    ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window, out=part,
+                          n_splits=n_splits, first_req=first_req, first_row=first_row)
+    assert torch.equal(part[first_row:], out[first_row:]) and (part[:first_row] == 7.0).all()
+
+
+def test_prefill_splits_choice():
+    from gibbs_amd.ops import prefill_splits
+    assert prefill_splits(32, 32, 2048) == 1                 # a whole 2,048-token prompt fills the chip
+    assert prefill_splits(8, 32, 8192) == 4                  # a portion of 512 late in a long prompt does not
+    assert prefill_splits(1, 4, 300) == 1 and prefill_splits(1, 4, 100000) == 16
+    assert prefill_splits(8, 32, 8192, window=128) == 1      # a window bounds the keys
 
 
 @pytest.mark.parametrize("dtype", DT)
