@@ -342,7 +342,7 @@ def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window, n_splits):
 def test_prefill_splits_choice():
     from gibbs_amd.ops import prefill_splits
     assert prefill_splits(32, 32, 2048) == 1                 # a whole 2,048-token prompt fills the chip
-    assert prefill_splits(8, 32, 8192) == 4                  # a portion of 512 late in a long prompt does not
+    assert prefill_splits(8, 32, 8192) == 8                  # a portion of 512 late in a long prompt does not
     assert prefill_splits(1, 4, 300) == 1 and prefill_splits(1, 4, 100000) == 16
     assert prefill_splits(8, 32, 8192, window=128) == 1      # a window bounds the keys
 
