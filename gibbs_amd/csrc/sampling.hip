@@ -34,6 +34,34 @@ __device__ __forceinline__ void block_best(float& v, int& i, float* sv, int* si)
     if (better(sv[w], si[w], v, i)) { v = sv[w]; i = si[w]; }
 }
 
+// Calls fn(value, index) for the elements of a row that fall to this thread: 16-byte loads over the
+// aligned middle of the row, single elements before and after it.
+template <typename F>
+__device__ __forceinline__ void walk_row(const float* row, int V, F fn) {
+  const int head = min(V, (int)(((16 - ((uintptr_t)row & 15)) & 15) / 4));
+  const int n4 = (V - head) / 4;
+  for (int i = threadIdx.x; i < head; i += THREADS) fn(row[i], i);
+  const float4* row4 = (const float4*)(row + head);
+  constexpr int AHEAD = 4;     // loads in flight per thread
+  for (int j0 = threadIdx.x; j0 < n4; j0 += AHEAD * THREADS) {
+    float4 v[AHEAD];
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a)
+      if (j0 + a * THREADS < n4) v[a] = row4[j0 + a * THREADS];
+#pragma unroll
+    for (int a = 0; a < AHEAD; ++a) {
+      const int j = j0 + a * THREADS;
+      if (j >= n4) break;
+      const int i = head + 4 * j;
+      fn(v[a].x, i);
+      fn(v[a].y, i + 1);
+      fn(v[a].z, i + 2);
+      fn(v[a].w, i + 3);
+    }
+  }
+  for (int i = head + 4 * n4 + threadIdx.x; i < V; i += THREADS) fn(row[i], i);
+}
+
 __global__ __launch_bounds__(THREADS) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V,
                                                          long ld) {
   __shared__ float sv[THREADS / WAVE];
@@ -41,45 +69,44 @@ __global__ __launch_bounds__(THREADS) void argmax_kernel(const float* __restrict
   const float* row = logits + (size_t)blockIdx.x * ld;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  // 16-byte loads over the aligned middle; NaN fails both comparisons in `better`
-  const int head = min(V, (int)(((16 - ((uintptr_t)row & 15)) & 15) / 4));
-  const int n4 = (V - head) / 4;
-  for (int i = threadIdx.x; i < head; i += THREADS)
-    if (better(row[i], i, bv, bi)) { bv = row[i]; bi = i; }
-  const float4* row4 = (const float4*)(row + head);
-  for (int j = threadIdx.x; j < n4; j += THREADS) {
-    const float4 v = row4[j];
-    const int i = head + 4 * j;
-    if (better(v.x, i, bv, bi)) { bv = v.x; bi = i; }
-    if (better(v.y, i + 1, bv, bi)) { bv = v.y; bi = i + 1; }
-    if (better(v.z, i + 2, bv, bi)) { bv = v.z; bi = i + 2; }
-    if (better(v.w, i + 3, bv, bi)) { bv = v.w; bi = i + 3; }
-  }
-  for (int i = head + 4 * n4 + threadIdx.x; i < V; i += THREADS)
-    if (better(row[i], i, bv, bi)) { bv = row[i]; bi = i; }
+  // NaN fails both comparisons in `better`
+  walk_row(row, V, [&](float v, int i) {
+    if (better(v, i, bv, bi)) { bv = v; bi = i; }
+  });
   block_best(bv, bi, sv, si);
   if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
 }
 
-__global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int* __restrict__ out, int V,
-                                                         long ld, const float* __restrict__ temperature,
-                                                         const float* __restrict__ top_p, const int* __restrict__ top_k,
-                                                         const float* __restrict__ u) {
-  __shared__ float sv[THREADS / WAVE];
-  __shared__ int si[THREADS / WAVE];
-  __shared__ float cand_v[MAX_K];
-  __shared__ int cand_i[MAX_K];
-  const int m = blockIdx.x;
-  const float* row = logits + (size_t)m * ld;
-  const float T = temperature[m];
-  const bool greedy = T <= 1e-4f;
-  int k = greedy ? 1 : top_k[m];
-  k = k < 1 ? 1 : (k > MAX_K ? MAX_K : k);
-  if (k > V) k = V;
-  // Round c finds the best element strictly after the previous pick in candidate order.
+// ---------------------------------------------------------------------------------------------- sampling
+// A candidate as one number: larger is better.  High half: the value's bits made monotone (negative
+// values flipped; -0 counted as +0, as the comparison of values does); low half: ~index, so that of
+// equal values the smaller index wins.  0 stands for "none" (no value maps to it; NaN is never a
+// candidate).
+typedef unsigned long long key64;
+constexpr int MAX_LIST = 2048;   // candidates above the threshold that are sorted exactly
+
+__device__ __forceinline__ unsigned ordered_bits(float v) {
+  const unsigned b = __float_as_uint(v == 0.f ? 0.f : v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ key64 make_key(float v, int i) {
+  return v != v ? 0ull : ((key64)ordered_bits(v) << 32) | (key64)(0xffffffffu - (unsigned)i);
+}
+__device__ __forceinline__ float key_value(key64 k) {
+  const unsigned o = (unsigned)(k >> 32);
+  return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
+}
+__device__ __forceinline__ int key_index(key64 k) { return (int)(0xffffffffu - (unsigned)k); }
+// Lane c's value, for a c that is the same in every lane (a scalar read, not a trip through LDS).
+__device__ __forceinline__ float lane_value(float v, int c) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), c));
+}
+
+// The k best candidates, one after the other: every round walks the whole row.  The way out when too
+// many values tie at the threshold for the list below (a row of equal logits).
+__device__ int top_k_by_rounds(const float* row, int V, int k, float* cand_v, int* cand_i, float* sv, int* si) {
   float pv = INFINITY;
-  int pi = -1;
-  int found = 0;
+  int pi = -1, found = 0;
   for (int c = 0; c < k; ++c) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
@@ -89,37 +116,132 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
       if (after && better(v, i, bv, bi)) { bv = v; bi = i; }
     }
     block_best(bv, bi, sv, si);
-    if (bi == 0x7fffffff) break;  // fewer than k finite candidates
+    if (bi == 0x7fffffff) break;  // fewer than k candidates
     if (threadIdx.x == 0) { cand_v[c] = bv; cand_i[c] = bi; }
     pv = bv; pi = bi; found = c + 1;
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  if (found == 0) { out[m] = 0; return; }
-  if (greedy) { out[m] = cand_i[0]; return; }
-  float probs[MAX_K];
+  return found;
+}
+
+// Two walks over the row instead of k.  First walk: every thread keeps the best of its elements.  The
+// ceil(k / 16)-th best of those in every wave, and the smallest of these over the 16 waves, is a value
+// that at least k elements of the row reach: a threshold at or below the k-th best value.  Second walk: the
+// elements that reach it (a few hundred for logits of a model) go to a list, which is ranked exactly.
+__global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict__ logits, int* __restrict__ out, int V,
+                                                         long ld, const float* __restrict__ temperature,
+                                                         const float* __restrict__ top_p, const int* __restrict__ top_k,
+                                                         const float* __restrict__ u) {
+  constexpr int WAVES = THREADS / WAVE;
+  __shared__ float sv[WAVES];
+  __shared__ int si[WAVES];
+  __shared__ float cand_v[MAX_K];
+  __shared__ int cand_i[MAX_K];
+  __shared__ unsigned wave_low[WAVES];
+  __shared__ key64 list[MAX_LIST];
+  __shared__ int s_count, s_valid;
+  const int m = blockIdx.x;
+  const float* row = logits + (size_t)m * ld;
+  const float T = temperature[m];
+  const bool greedy = T <= 1e-4f;
+  int k = greedy ? 1 : top_k[m];
+  k = k < 1 ? 1 : (k > MAX_K ? MAX_K : k);
+  if (k > V) k = V;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  if (threadIdx.x == 0) { s_count = 0; s_valid = 0; }
+
+  // first walk
+  unsigned mine = 0;         // the largest value of this thread's elements, as ordered bits (0: none)
+  int valid = 0;
+  walk_row(row, V, [&](float v, int i) {
+    const unsigned o = v != v ? 0u : ordered_bits(v);
+    valid += o != 0;
+    mine = max(mine, o);
+  });
+  // the ceil(k / 16)-th largest of the wave's threads, counting equal ones once (0: it has fewer): at
+  // least that many threads of the wave hold an element that reaches it
+  const int per_wave = (k + WAVES - 1) / WAVES;
+  unsigned rest = mine, nth = 0;
+  for (int c = 0; c < per_wave; ++c) {
+    nth = rest;
+#pragma unroll
+    for (int o = WAVE / 2; o > 0; o >>= 1) nth = max(nth, (unsigned)__shfl_xor((int)nth, o, WAVE));
+    if (rest == nth) rest = 0;
+  }
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) valid += __shfl_xor(valid, o, WAVE);
+  __syncthreads();
+  if (lane == 0) {
+    wave_low[wave] = nth;
+    atomicAdd(&s_valid, valid);
+  }
+  __syncthreads();
+  unsigned threshold = wave_low[0];                       // 0: every candidate passes
+  for (int w = 1; w < WAVES; ++w) threshold = min(threshold, wave_low[w]);
+  const int n_valid = s_valid;
+  int found = k < n_valid ? k : n_valid;
+  if (found == 0) {
+    if (threadIdx.x == 0) out[m] = 0;
+    return;
+  }
+
+  // second walk: everything at or above the threshold
+  walk_row(row, V, [&](float v, int i) {
+    if (v == v && ordered_bits(v) >= threshold) {
+      const int at = atomicAdd(&s_count, 1);
+      if (at < MAX_LIST) list[at] = make_key(v, i);
+    }
+  });
+  __syncthreads();
+  const int n = s_count;
+  if (n > MAX_LIST) {
+    found = top_k_by_rounds(row, V, k, cand_v, cand_i, sv, si);
+  } else {
+    // rank of every listed candidate = how many are better; keys differ, so ranks do
+    for (int j = threadIdx.x; j < n; j += THREADS) {
+      const key64 key = list[j];
+      int rank = 0;
+      for (int o = 0; o < n; ++o) rank += list[o] > key;
+      if (rank < found) {
+        cand_v[rank] = key_value(key);
+        cand_i[rank] = key_index(key);
+      }
+    }
+    __syncthreads();
+  }
+  // The draw, by the first wave: lane c holds candidate c; the sums run over the candidates one after
+  // the other (values passed from lane to lane), in the order a serial loop would add them.
+  if (wave != 0) return;
+  if (found == 0) {
+    if (lane == 0) out[m] = 0;
+    return;
+  }
+  if (greedy) {
+    if (lane == 0) out[m] = cand_i[0];
+    return;
+  }
   const float mx = cand_v[0] / T;
+  const float e = lane < found ? expf(cand_v[lane] / T - mx) : 0.f;
   float sum = 0.f;
-  for (int c = 0; c < found; ++c) { probs[c] = expf(cand_v[c] / T - mx); sum += probs[c]; }
-  const float denom = fmaxf(sum, 1e-12f);
+  for (int c = 0; c < found; ++c) sum += lane_value(e, c);
+  const float p = e / fmaxf(sum, 1e-12f);
   const float thresh = fminf(fmaxf(top_p[m], 0.01f), 1.0f);
   float cum = 0.f;
   int cut = found;
   for (int c = 0; c < found; ++c) {
-    probs[c] /= denom;
-    cum += probs[c];
+    cum += lane_value(p, c);
     if (cum >= thresh) { cut = c + 1; break; }
   }
   float kept = 0.f;
-  for (int c = 0; c < cut; ++c) kept += probs[c];
+  for (int c = 0; c < cut; ++c) kept += lane_value(p, c);
   const float r = u[m] * kept;
   cum = 0.f;
-  int pick = cand_i[cut - 1];
+  int pick = cut - 1;
   for (int c = 0; c < cut; ++c) {
-    cum += probs[c];
-    if (cum >= r) { pick = cand_i[c]; break; }
+    cum += lane_value(p, c);
+    if (cum >= r) { pick = c; break; }
   }
-  out[m] = pick;
+  if (lane == 0) out[m] = cand_i[pick];
 }
 }  // namespace
 

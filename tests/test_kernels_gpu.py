@@ -464,6 +464,39 @@ def test_sample_against_plain():
     assert g.tolist() == logits.argmax(-1).tolist()
 
 
+@pytest.mark.parametrize("V", [65536, 50001, 700])
+def test_sample_large_vocabulary_ties_and_specials(V):
+    """Top-k by two walks over the row: vocabularies beyond one element per thread, a thousand values tied
+    at the top (the smaller ids win), a row of equal logits (more ties than the candidate list holds),
+    NaN (never a candidate) and -inf among the values, and -0 beside +0 at the top (equal values)."""
+    from gibbs_amd import ops
+    from tests.plain import lfm2_plain as P
+    rng = np.random.default_rng(V)
+    rows = [rng.standard_normal(V).astype(np.float32) * 3 for _ in range(6)]
+    top = rows[1].max() + 1
+    rows[1][rng.choice(V, size=min(1000, V // 2), replace=False)] = top          # many ties at the top
+    rows[2][:] = 0.25                                                          # everything ties
+    rows[3][rng.choice(V, size=V // 3, replace=False)] = np.nan
+    rows[3][rng.choice(V, size=V // 4, replace=False)] = -np.inf
+    rows[4] = -np.abs(rows[4]) - 1
+    zeros = rng.choice(V, size=40, replace=False)
+    rows[4][zeros[:20]] = 0.0
+    rows[4][zeros[20:]] = -0.0
+    rows[5][:] = -np.inf                                                       # nothing above -inf: still candidates
+    rows[5][V // 2] = 1.0
+    logits = torch.tensor(np.stack(rows), device=DEV)
+    M = len(rows)
+    for temp, p, k in [(0.8, 0.9, 50), (1.3, 1.0, 64), (0.5, 0.97, 7)]:
+        u = rng.random(M).astype(np.float32)
+        got = ops.sample(logits, torch.full((M,), temp, device=DEV), torch.full((M,), p, device=DEV),
+                         i32([k] * M), torch.tensor(u, device=DEV)).tolist()
+        for m in range(M):
+            cand, probs = P.nucleus(rows[m], temp, k, p)
+            assert got[m] == P.draw(cand, probs, float(u[m])), f"row {m}, k {k}"
+    greedy = ops.sample(logits, torch.zeros(M, device=DEV), torch.ones(M, device=DEV), i32([50] * M), torch.zeros(M, device=DEV))
+    assert greedy.tolist() == [P.argmax_first(r) for r in rows] == ops.argmax(logits).tolist()
+
+
 # --------------------------------------------------------------------------- fused decode kernels
 def rms_scale(x, eps):
     return 1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + eps)
