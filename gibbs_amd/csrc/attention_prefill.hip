@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
     // the loads above are to be in flight during the arithmetic below, not sunk to their use
     __builtin_amdgcn_sched_barrier(0);
     // a wave whose rows see none of this tile's keys has nothing to do (it still takes part in the barriers)
-    if (key0 > wave_last || key0 + BN <= wave_first_key) continue;
+    if (key0 > wave_last || key0 + BN <= wave_first_key || wave * 16 >= rows_here) continue;   // (or it has no rows)
 
     // S^T = K Q^T: 4 sub-tiles of 16 keys; this lane gets S[row lr][key c*16 + g*4 + i]
     floatx4 s4[4];

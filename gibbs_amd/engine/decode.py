@@ -60,7 +60,7 @@ class DecodeLoop:
             n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
             cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
             tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
-            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=engine.ctx_limit, decode_graph=True)
+            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True)
         self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
         self.counter = torch.zeros(1, dtype=torch.int32, device=dev)
         if not self.greedy:
@@ -98,6 +98,13 @@ class DecodeLoop:
         self._fill_tables()
         self._dev.copy_(torch.from_numpy(h))
         self.batch.ctx_lens, self.batch.slots = lens.tolist(), h[self._sec[5]].tolist()
+        # The longest sequence the loop can reach before it is bound again: kernels choose their key
+        # slices by it, and a captured graph keeps that choice, so graphs captured for a shorter bound
+        # are dropped.  Powers of two, so that requests that grow do not have graphs captured often.
+        reach = min(engine.ctx_limit, int(lens.max()) + self.capacity)
+        if reach > self.batch.max_seq:
+            self.batch.max_seq = min(engine.ctx_limit, 1 << max(reach - 1, 1).bit_length())
+            self.graph = self.graph_many = None
         self.counter.zero_()
         self.steps_done = 0
         self.pending = 0
