@@ -122,3 +122,68 @@ def test_random_orders_keep_invariants(seed):
         m.release(rid)
     m.check()
     assert m.free_pages(0) == m.free_pages(1) == 30 and m.free_slots() == 4
+
+
+def test_native_step_staging_matches_a_plain_packing():
+    """The host runtime's packing of a step (ids, positions, row -> request, cu, ctx, slots, wanted rows,
+    block tables, every section on a 16-byte boundary) against the same arrays built here; a refused
+    step (bad token, wanted place, context limit, too few pages) changes nothing."""
+    import ctypes
+
+    from gibbs_amd.cache import host
+    lib = host.library()
+    m = CacheManager([FULL, None, WIN], [(), (StateNeed("s", (4,)),), ()], 8, 10, 4)
+    rng = random.Random(3)
+    for rid, n in (("a", 11), ("b", 3)):
+        assert m.admit(rid) and m.reserve(rid, n)
+        m.commit(rid, n)
+    assert m.admit("c")
+
+    def stage(entries, vocab=100, ctx_limit=64):
+        n = len(entries)
+        slots = np.array([m.slot(r) for r, _, _ in entries], dtype=np.int32)
+        q_len = np.array([len(t) for _, t, _ in entries], dtype=np.int32)
+        tokens = np.array([x for _, t, _ in entries for x in t], dtype=np.int32)
+        want_cu = np.concatenate([[0], np.cumsum([len(w) for _, _, w in entries])]).astype(np.int32)
+        want = np.array([x for _, _, w in entries for x in w], dtype=np.int32)
+        info = (ctypes.c_long * (1 + m.n_groups))()
+        bad = ctypes.c_int(-1)
+        ops = (n, slots.ctypes.data, q_len.ctypes.data, tokens.ctypes.data, want_cu.ctypes.data, want.ctypes.data)
+        code = lib.gibbs_cache_reserve_step(m.core, *ops, vocab, ctx_limit, info, ctypes.byref(bad))
+        if code < 0:
+            return code, bad.value, host.last_error()
+        out = np.full(int(info[0]), -7, dtype=np.int32)
+        offsets = (ctypes.c_long * (9 + m.n_groups))()
+        assert lib.gibbs_cache_fill_step(m.core, *ops, info, out.ctypes.data, offsets) == 0
+        return out, list(offsets), [int(info[1 + g]) for g in range(m.n_groups)]
+
+    before = (m.free_pages(0), m.free_pages(1))
+    assert stage([("a", [1, 2], [0]), ("b", [3, 100], [])])[:2] == (host.ERR_STEP, 1)          # token outside the vocabulary
+    assert stage([("a", [1, 2], [2])])[:2] == (host.ERR_STEP, 0)                                # wanted place outside
+    assert stage([("a", [1] * 54, [])])[0] == host.ERR_STEP                                     # 65 tokens > 64
+    assert stage([("a", [1], []), ("a", [2], [])])[:2] == (host.ERR_STEP, 1)                    # twice in one step
+    code, group, text = stage([("a", [1] * 30, []), ("c", [1] * 50, [])])
+    assert code == host.ERR_NO_ROOM and "pages" in text
+    assert (m.free_pages(0), m.free_pages(1)) == before and m.tokens("a") == 11
+    m.check()
+
+    entries = [("b", [7], [0]), ("a", [rng.randrange(100) for _ in range(9)], [0, 8]), ("c", [5, 6, 7], [])]
+    out, offsets, widths = stage(entries)
+    ctx = [3, 11, 0]
+    q = [1, 9, 3]
+    cu = np.concatenate([[0], np.cumsum(q)])
+    assert all(o % 4 == 0 for o in offsets[:7 + m.n_groups])
+    sec = lambda i, size: out[offsets[i]:offsets[i] + size].tolist()
+    assert sec(0, 13) == [x for _, t, _ in entries for x in t]
+    assert sec(1, 13) == [c + t for c, n in zip(ctx, q) for t in range(n)]
+    assert sec(2, 13) == [i for i, n in enumerate(q) for _ in range(n)]
+    assert sec(3, 4) == cu.tolist() and sec(4, 3) == ctx and sec(5, 3) == [m.slot(r) for r, _, _ in entries]
+    assert sec(6, 3) == [0, 1, 9]                                                               # b's row, rows of a's places 0 and 8
+    for g in range(m.n_groups):
+        table = np.array(sec(7 + g, 3 * widths[g])).reshape(3, widths[g])
+        assert (table == m.block_table([r for r, _, _ in entries], g, widths[g])).all()
+        assert widths[g] == m.pages_for(20)
+    assert offsets[7 + m.n_groups:9 + m.n_groups] == [9, 20]                                     # longest portion, longest sequence
+    for (r, t, _), n in zip(entries, q):
+        m.commit(r, n)
+    m.check()
