@@ -35,7 +35,7 @@ class PreNormBlock(Block):
             self.ffn.pack_matrices()
 
     def _fold(self, norm, part) -> bool:
-        if self.rt.act_dtype != torch.bfloat16:
+        if self.rt.act_dtype != torch.bfloat16 or os.environ.get("GIBBS_FOLD_GAINS", "1") == "0":
             return False
         if not (hasattr(norm, "fold_gain") and hasattr(part, "fold_input_gain")):
             return False
