@@ -169,6 +169,31 @@ def test_mixed_with_page_reuse(model_dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_decoded_tokens_at_the_head_of_a_mixed_step(model_dirs, name, dtype):
+    """Three requests that decode, then a prompt portion, then one more decoded token, in one step:
+    in bfloat16 the decoded tokens at the head take the decode attention kernel and the rest the
+    matrix-core kernel, each with its own slice of the batch's metadata; twice, so that the second
+    such step reads what the first one cached."""
+    d = model_dirs[name]
+    vocab = H.TINY[name]["vocab_size"]
+    seqs = {f"s{i}": H.tokens(40 + i, n, vocab) for i, n in enumerate([40, 23, 57, 75, 31])}
+    pre = {"s0": 30, "s1": 21, "s2": 50, "s3": 0, "s4": 29}
+    steps = [([(r, seqs[r][:n], [n - 1])], []) for r, n in pre.items() if n]
+    at = dict(pre)
+    for portion in (41, 34):
+        entries = []
+        for r in ("s0", "s1", "s2", "s3", "s4"):
+            n = portion if r == "s3" else 1
+            entries.append((r, seqs[r][at[r]:at[r] + n], list(range(n))))
+            at[r] += n
+        steps.append((entries, []))
+    got = run_steps(make_engine(d, dtype, max_tokens=512, max_requests=5), steps)
+    assert ("s3", 74) in got and ("s0", 31) in got
+    check(d, seqs, got, dtype, f"decoded tokens first {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding(model_dirs, dtype):
     d = model_dirs["A"]
     ids = H.tokens(9, 400, 256)
