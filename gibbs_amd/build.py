@@ -139,7 +139,7 @@ def host_sources() -> list[str]:
 
 def _host_stamp() -> str:
     h = hashlib.sha256()
-    for path in host_sources():
+    for path in host_sources() + sorted(glob.glob(os.path.join(HOST_SRC, "*.h"))):
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())

@@ -1,4 +1,4 @@
-"""Loads the host runtime (page accounting, block tables, step staging: plain C++) and declares
+"""Loads the host runtime (page accounting, block tables, step staging, the scheduler's decisions: plain C++) and declares
 its C interface.  Built at the first use when no current library is there; there is no Python
 twin of it."""
 from __future__ import annotations
@@ -39,6 +39,18 @@ _SIGNATURES = {
     "gibbs_cache_check": ([c_void_p], c_int),
     "gibbs_cache_reserve_step": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_long,
                                   _lp, _ip], c_int),
+    "gibbs_sched_create": ([c_void_p, c_long, c_long, c_long], c_void_p),
+    "gibbs_sched_destroy": ([c_void_p], None),
+    "gibbs_sched_submit": ([c_void_p, c_long, c_long, c_int], c_int),
+    "gibbs_sched_counts": ([c_void_p, _ip, _ip], c_int),
+    "gibbs_sched_list": ([c_void_p, c_int, _ip, c_int], c_int),
+    "gibbs_sched_query": ([c_void_p, c_int, _lp], c_int),
+    "gibbs_sched_events": ([c_void_p, _lp, c_long], c_long),
+    "gibbs_sched_plan": ([c_void_p, _lp, c_int, _lp, c_long, _lp], c_int),
+    "gibbs_sched_apply": ([c_void_p, c_int, _ip, _ip, _ip, _lp, c_long, _lp], c_int),
+    "gibbs_sched_fail_plan": ([c_void_p, _lp, c_long, _lp], c_int),
+    "gibbs_sched_burst_plan": ([c_void_p, c_long, _ip, c_int, _ip], c_long),
+    "gibbs_sched_apply_burst": ([c_void_p, c_int, c_int, _ip, _lp, c_long, _lp], c_int),
     "gibbs_cache_fill_step": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, _lp, c_void_p, _lp],
                               c_int),
 }

@@ -175,6 +175,16 @@ class CacheManager:
         if code < 0:
             self._raise(code, rid)
 
+    def adopt(self, rid: Hashable, slot: int) -> None:
+        """The native scheduler admitted `rid` into `slot` of the core: learn the name."""
+        if rid in self._slots:
+            raise KeyError(f"request {rid!r} is already live")
+        self._slots[rid] = slot
+
+    def forget(self, rid: Hashable) -> None:
+        """The native scheduler gave the request's slot and pages back."""
+        del self._slots[rid]
+
     # ------------------------------------------------------------------ what kernels read
     def slots_of(self, rids: Sequence[Hashable]):
         return host.ints([self._slots[r] for r in rids])

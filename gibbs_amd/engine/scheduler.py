@@ -22,16 +22,22 @@ prompt (state of fixed size cannot be rewound or swapped by position, so recompu
 only exact way).  A prompt portion that cannot get pages shrinks to what is free, or waits.  If
 no request can move at all, the youngest is preempted so that the oldest can.  A request that
 does not fit the whole pool alone fails with an error.
+
+The decisions themselves are native code (csrc/host/scheduler.cpp: it works on lengths and counts and
+takes slots and pages from the cache core directly); this module keeps the tokens, the sampling
+parameters and the results, builds the step's entries from the native plan, runs them and reports
+the sampled tokens back.
 """
 from __future__ import annotations
 
-import itertools
+import ctypes
 from collections import deque
 from dataclasses import dataclass, field
 from enum import Enum
 from typing import Callable, Deque, Dict, Hashable, List, Optional, Tuple
 from typing import Sequence as SeqOf
 
+from ..cache import host
 from ..cache.manager import CacheManager
 from ..sampling.sampler import Draw, SamplingParams
 from .batch import Entry
@@ -99,6 +105,10 @@ class StepOutput:
 Runner = Callable[[SeqOf[Entry], SeqOf[Draw]], List[int]]
 
 
+# what the native core reports back: (kind, request number, value)
+EV_ADMITTED, EV_RELEASED, EV_PREEMPTED, EV_STOP, EV_LENGTH, EV_TOO_LARGE, EV_POOL, EV_STEP_FAILED = range(1, 9)
+
+
 class ContinuousBatchScheduler:
     def __init__(self, cache: CacheManager, runner: Runner, *, context_len: int,
                  max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
@@ -114,11 +124,24 @@ class ContinuousBatchScheduler:
         self.max_batch_tokens = max_batch_tokens
         self.chunk = chunk
         self.eos = set(eos_token_ids)
-        self.waiting: Deque[Sequence] = deque()
-        self.active: List[Sequence] = []
         self.finished: Dict[Hashable, Sequence] = {}
-        self._counter = itertools.count()
         self.steps = 0
+        self._lib = host.library()
+        self._core = self._lib.gibbs_sched_create(cache.core, context_len, max_batch_tokens, chunk or 0)
+        if not self._core:
+            raise ValueError("the scheduler core refused its sizes")
+        self._seqs: List[Sequence] = []                     # by request number (the order of submission)
+        self._ids: Dict[Hashable, int] = {}                 # requests that have not finished
+        room = 3 * (8 * cache.max_requests + 64)
+        self._events = (ctypes.c_long * room)()
+        self._n_events = ctypes.c_long(0)
+        self._plan = (ctypes.c_long * (5 * cache.max_requests))()
+        self._numbers = (ctypes.c_int * cache.max_requests)()
+
+    def __del__(self):
+        if getattr(self, "_core", None):
+            self._lib.gibbs_sched_destroy(self._core)
+            self._core = None
 
     # ------------------------------------------------------------------ submitting
     def submit(self, prompt_tokens: SeqOf[int], params: Optional[SamplingParams] = None,
@@ -126,9 +149,9 @@ class ContinuousBatchScheduler:
         """Queues a request.  An empty prompt becomes [1] (scheduler/mod.rs:1005-1008);
         `max_new_tokens` is clamped to the room the context leaves (:953-955)."""
         params = params or SamplingParams()
-        order = next(self._counter)
+        order = len(self._seqs)
         rid = order if rid is None else rid
-        if rid in self.finished or any(s.id == rid for s in itertools.chain(self.waiting, self.active)):
+        if rid in self.finished or rid in self._ids:
             raise KeyError(f"request id {rid!r} is in use")
         prompt = [int(t) for t in prompt_tokens] or [1]
         if len(prompt) > self.context_len:
@@ -137,149 +160,93 @@ class ContinuousBatchScheduler:
         if params.max_new_tokens > room:
             params = SamplingParams(params.temperature, params.top_p, params.top_k, room, params.seed,
                                     params.ignore_eos)
-        self.waiting.append(Sequence(rid, prompt, params, order))
+        number = self._lib.gibbs_sched_submit(self._core, len(prompt), params.max_new_tokens, int(params.ignore_eos))
+        assert number == order
+        self._seqs.append(Sequence(rid, prompt, params, order))
+        self._ids[rid] = number
         return rid
 
+    # ------------------------------------------------------------------ what the core knows
+    def _listed(self, which: int) -> List[Sequence]:
+        out = (ctypes.c_int * max(1, len(self._ids)))()
+        n = self._lib.gibbs_sched_list(self._core, which, out, len(out))
+        return [self._seqs[out[i]] for i in range(n)]
+
+    @property
+    def waiting(self) -> Deque[Sequence]:
+        """The waiting queue, head first (a copy: the queue itself is the core's)."""
+        return deque(self._listed(0))
+
+    @property
+    def active(self) -> List[Sequence]:
+        return self._listed(1)
+
+    def _counts(self):
+        w, a = ctypes.c_int(0), ctypes.c_int(0)
+        self._lib.gibbs_sched_counts(self._core, ctypes.byref(w), ctypes.byref(a))
+        return w.value, a.value
+
     def has_work(self) -> bool:
-        return bool(self.waiting or self.active)
+        return any(self._counts())
 
-    # ------------------------------------------------------------------ helpers
-    def _computed(self, seq: Sequence) -> int:
-        return self.cache.tokens(seq.id) if seq.id in self.cache else 0
-
-    def _remaining(self, seq: Sequence) -> int:
-        """Tokens the request still has to feed: its whole remaining prompt, or 1 when it decodes."""
-        return len(seq.prompt_tokens) + len(seq.output_tokens) - self._computed(seq)
-
-    def _fits(self, rid: Hashable, n: int) -> bool:
-        need = self.cache.pages_needed(rid, n)
-        return all(k <= self.cache.free_pages(g) for g, k in enumerate(need))
-
-    def _largest_fit(self, rid: Hashable, n: int) -> int:
-        """The most tokens <= n whose pages are free now (the pages needed grow with n)."""
-        lo, hi = 0, n
-        while lo < hi:
-            mid = (lo + hi + 1) // 2
-            if self._fits(rid, mid):
-                lo = mid
+    def _book(self, error: Optional[str] = None):
+        """Applies the core's events of the last call to the requests and to the cache manager's names;
+        returns (finished ids, preempted ids) in the order they happened."""
+        finished, preempted = [], []
+        if 3 * self._n_events.value > len(self._events):          # more happened than the buffer holds: ask again
+            self._events = (ctypes.c_long * (3 * self._n_events.value))()
+            self._lib.gibbs_sched_events(self._core, self._events, len(self._events))
+        ev = self._events
+        for i in range(self._n_events.value):
+            kind, seq, value = ev[3 * i], self._seqs[ev[3 * i + 1]], ev[3 * i + 2]
+            if kind == EV_ADMITTED:
+                self.cache.adopt(seq.id, value)
+                seq.state = SequenceState.PREFILLING
+            elif kind == EV_RELEASED:
+                self.cache.forget(seq.id)
+            elif kind == EV_PREEMPTED:
+                seq.state = SequenceState.WAITING
+                seq.preemptions += 1
+                preempted.append(seq.id)
             else:
-                hi = mid - 1
-        return lo
-
-    def _finish(self, seq: Sequence, reason: FinishReason, error: Optional[str] = None) -> None:
-        seq.state, seq.finish_reason, seq.error = SequenceState.FINISHED, reason, error
-        if seq.id in self.cache:
-            self.cache.release(seq.id)
-        if seq in self.active:
-            self.active.remove(seq)
-        self.finished[seq.id] = seq
-
-    def _preempt(self, seq: Sequence) -> None:
-        """Frees everything the request holds; it will be recomputed from its tokens so far."""
-        self.cache.release(seq.id)
-        self.active.remove(seq)
-        seq.state = SequenceState.WAITING
-        seq.preemptions += 1
-        self.waiting.appendleft(seq)
+                seq.state = SequenceState.FINISHED
+                if kind == EV_STOP:
+                    seq.finish_reason = FinishReason.STOP
+                elif kind == EV_LENGTH:
+                    seq.finish_reason = FinishReason.LENGTH
+                else:
+                    seq.finish_reason = FinishReason.ERROR
+                    pool = min((p.num_pages for p in self.cache.pools), default=0)
+                    seq.error = {EV_TOO_LARGE: f"the request needs {value} pages, the pool has {pool}",
+                                 EV_POOL: "the cache pool is too small for this request"}.get(kind, error)
+                self.finished[seq.id] = seq
+                self._ids.pop(seq.id, None)
+                finished.append(seq.id)
+        return finished, preempted
 
     # ------------------------------------------------------------------ one step
     def step(self) -> StepOutput:
         self.steps += 1
-        budget = self.max_batch_tokens
-        cap = budget if self.chunk is None else min(budget, self.chunk)
-        preempted: List[Hashable] = []
-        finished: List[Hashable] = []
+        lib, n_ev = self._lib, ctypes.byref(self._n_events)
+        n_plan = lib.gibbs_sched_plan(self._core, self._plan, len(self._plan) // 5, self._events, len(self._events), n_ev)
+        if n_plan < 0:
+            raise RuntimeError(host.last_error())
+        finished, preempted = self._book()
 
-        # 1. admission: first in, first out; needs a slot and the pages of the first portion
-        while self.waiting:
-            seq = self.waiting[0]
-            if seq.params.max_new_tokens == 0 and not seq.output_tokens:
-                self.waiting.popleft()
-                self._finish(seq, FinishReason.LENGTH)              # scheduler/mod.rs:1357-1359
-                finished.append(seq.id)
-                continue
-            total = seq.n_tokens
-            if self.cache.pages_for(total + 1) > min((p.num_pages for p in self.cache.pools), default=1 << 60):
-                self.waiting.popleft()
-                self._finish(seq, FinishReason.ERROR,
-                             f"the request needs {self.cache.pages_for(total + 1)} pages, the pool has "
-                             f"{min(p.num_pages for p in self.cache.pools)}")
-                finished.append(seq.id)
-                continue
-            if not self.cache.admit(seq.id):
-                break
-            first = min(total, cap)
-            if not self.cache.reserve(seq.id, first):
-                self.cache.release(seq.id)
-                break
-            self.waiting.popleft()
-            seq.state = SequenceState.PREFILLING
-            self.active.append(seq)
-
-        # 2. order: decoders first, then shortest remaining prompt; the oldest prefilling request
-        #    keeps up to half the budget
-        def is_decoding(s: Sequence) -> bool:
-            return s.state == SequenceState.DECODING
-        self.active.sort(key=lambda s: (0 if is_decoding(s) else self._remaining(s), s.submitted))
-        prefilling = [s for s in self.active if not is_decoding(s)]
-        oldest = min(prefilling, key=lambda s: s.submitted, default=None)
-        reserved = min(self._remaining(oldest), -(-budget // 2)) if oldest is not None else 0
-
-        # 3. plan: pages first, so that the batch that runs is the batch that fits
-        plan: List[Tuple[Sequence, int]] = []
-        left = budget
-        for seq in list(self.active):
-            if seq not in self.active:
-                continue                                            # preempted meanwhile
-            if is_decoding(seq):
-                while not self._fits(seq.id, 1):
-                    victim = max(self.active, key=lambda s: s.submitted)
-                    plan = [(s, n) for s, n in plan if s is not victim]
-                    self._preempt(victim)
-                    preempted.append(victim.id)
-                    if victim is seq:
-                        break
-                if seq in self.active:
-                    assert self.cache.reserve(seq.id, 1)
-                    plan.append((seq, 1))
-                continue
-            if seq is oldest:
-                available, reserved = left, 0
-            else:
-                available = max(0, left - reserved)
-            n = min(self._remaining(seq), available, cap)
-            if n > 0 and not self._fits(seq.id, n):
-                n = self._largest_fit(seq.id, n)
-            if n <= 0:
-                continue                                            # budget or pages exhausted: next step
-            assert self.cache.reserve(seq.id, n)
-            plan.append((seq, n))
-            left -= n
-        if not plan and self.active:
-            # nothing can move: make room for the oldest by preempting the youngest
-            victim = max(self.active, key=lambda s: s.submitted)
-            if len(self.active) == 1:
-                self._finish(victim, FinishReason.ERROR, "the cache pool is too small for this request")
-                finished.append(victim.id)
-            else:
-                self._preempt(victim)
-                preempted.append(victim.id)
-
-        # 4. one batch: portions beside decoded tokens; logits at the last row of every request
-        #    that has fed all its tokens
+        # one batch: portions beside decoded tokens; logits at the last row of every request that has
+        # fed all its tokens
         entries: List[Entry] = []
         draws: List[Draw] = []
         sampled_for: List[Sequence] = []
         prefill_tokens = decode_tokens = 0
-        for seq, n in plan:
-            at = self._computed(seq)
-            toks = seq.span(at, n)
-            last = at + n == seq.n_tokens
-            entries.append(Entry(seq.id, toks, [n - 1] if last else []))
+        for i in range(n_plan):
+            number, at, n, last, decoding = self._plan[5 * i:5 * i + 5]
+            seq = self._seqs[number]
+            entries.append(Entry(seq.id, seq.span(at, n), [n - 1] if last else []))
             if last:
                 draws.append(Draw(seq.params, seq.id, len(seq.output_tokens)))
                 sampled_for.append(seq)
-            if is_decoding(seq):
+            if decoding:
                 decode_tokens += 1
             else:
                 prefill_tokens += n
@@ -288,27 +255,26 @@ class ContinuousBatchScheduler:
             try:
                 tokens = self.runner(entries, draws)
             except Exception as exc:                                # scheduler/mod.rs:1332-1340
-                for seq, _ in plan:
-                    self._finish(seq, FinishReason.ERROR, f"{type(exc).__name__}: {exc}")
-                    finished.append(seq.id)
-                return StepOutput(entries, [], finished, preempted, prefill_tokens, decode_tokens,
-                                  len(self.active), len(self.waiting))
+                lib.gibbs_sched_fail_plan(self._core, self._events, len(self._events), n_ev)
+                finished += self._book(f"{type(exc).__name__}: {exc}")[0]
+                waiting, active = self._counts()
+                return StepOutput(entries, [], finished, preempted, prefill_tokens, decode_tokens, active, waiting)
             assert len(tokens) == len(sampled_for)
-            # 5. emit and finish
-            for seq, tok in zip(sampled_for, tokens):
+            # emit and finish
+            k = len(tokens)
+            numbers = (ctypes.c_int * max(1, k))(*[s.submitted for s in sampled_for])
+            is_eos = (ctypes.c_int * max(1, k))(*[int(t in self.eos) for t in tokens])
+            took = (ctypes.c_int * max(1, k))()
+            if lib.gibbs_sched_apply(self._core, k, numbers, is_eos, took, self._events, len(self._events), n_ev) < 0:
+                raise RuntimeError(host.last_error())
+            for seq, tok, counts in zip(sampled_for, tokens, took):
                 seq.state = SequenceState.DECODING
-                if tok in self.eos and not seq.params.ignore_eos:
-                    self._finish(seq, FinishReason.STOP)            # the end token is not emitted
-                    finished.append(seq.id)
-                    continue
-                seq.output_tokens.append(int(tok))
-                emitted.append((seq.id, int(tok)))
-                if (len(seq.output_tokens) >= seq.params.max_new_tokens
-                        or seq.n_tokens >= self.context_len):
-                    self._finish(seq, FinishReason.LENGTH)
-                    finished.append(seq.id)
-        return StepOutput(entries, emitted, finished, preempted, prefill_tokens, decode_tokens,
-                          len(self.active), len(self.waiting))
+                if counts:
+                    seq.output_tokens.append(int(tok))
+                    emitted.append((seq.id, int(tok)))
+            finished += self._book()[0]
+        waiting, active = self._counts()
+        return StepOutput(entries, emitted, finished, preempted, prefill_tokens, decode_tokens, active, waiting)
 
     # ------------------------------------------------------------------ bursts of decode steps
     def burst_plan(self, cap: int) -> Optional[Tuple[List[Sequence], int]]:
@@ -316,14 +282,11 @@ class ContinuousBatchScheduler:
         back on the device without the host in between (a captured graph per step).  Returns the
         requests (oldest first) and how many steps all of them can still take, at most `cap`; None
         when a step has anything else to do."""
-        if self.waiting or not self.active:
+        n_out = ctypes.c_int(0)
+        n = self._lib.gibbs_sched_burst_plan(self._core, cap, self._numbers, len(self._numbers), ctypes.byref(n_out))
+        if n < 1:
             return None
-        if any(s.state != SequenceState.DECODING or self._remaining(s) != 1 for s in self.active):
-            return None
-        seqs = sorted(self.active, key=lambda s: s.submitted)
-        n = min(cap, min(min(s.params.max_new_tokens - len(s.output_tokens), self.context_len - s.n_tokens)
-                         for s in seqs))
-        return (seqs, n) if n >= 1 else None
+        return [self._seqs[self._numbers[i]] for i in range(n_out.value)], int(n)
 
     def apply_burst(self, seqs: List[Sequence], tokens: List[List[int]]) -> StepOutput:
         """Books the tokens that a burst sampled (tokens[i]: those of seqs[i], all already cached):
@@ -332,19 +295,16 @@ class ContinuousBatchScheduler:
         emitted: List[Tuple[Hashable, int]] = []
         finished: List[Hashable] = []
         for seq, toks in zip(seqs, tokens):
-            for tok in toks:
-                if tok in self.eos and not seq.params.ignore_eos:
-                    self._finish(seq, FinishReason.STOP)
-                    finished.append(seq.id)
-                    break
-                seq.output_tokens.append(int(tok))
-                emitted.append((seq.id, int(tok)))
-                if (len(seq.output_tokens) >= seq.params.max_new_tokens
-                        or seq.n_tokens >= self.context_len):
-                    self._finish(seq, FinishReason.LENGTH)
-                    finished.append(seq.id)
-                    break
-        return StepOutput([], emitted, finished, [], 0, len(emitted), len(self.active), len(self.waiting))
+            is_eos = (ctypes.c_int * max(1, len(toks)))(*[int(t in self.eos) for t in toks])
+            took = self._lib.gibbs_sched_apply_burst(self._core, seq.submitted, len(toks), is_eos, self._events,
+                                                     len(self._events), ctypes.byref(self._n_events))
+            if took < 0:
+                raise RuntimeError(host.last_error())
+            seq.output_tokens.extend(int(t) for t in toks[:took])
+            emitted.extend((seq.id, int(t)) for t in toks[:took])
+            finished += self._book()[0]
+        waiting, active = self._counts()
+        return StepOutput([], emitted, finished, [], 0, len(emitted), active, waiting)
 
     def run(self, on_step: Optional[Callable[[StepOutput], None]] = None) -> Dict[Hashable, Sequence]:
         """Steps until every submitted request has finished."""

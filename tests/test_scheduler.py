@@ -198,3 +198,16 @@ def test_temperature_draws_are_reproducible():
     assert u == [uniform(5, request_key("r"), i) for i in range(1000)]
     assert u[:10] != [uniform(6, request_key("r"), i) for i in range(10)]
     assert u[:10] != [uniform(5, request_key("q"), i) for i in range(10)]
+
+
+def test_many_requests_that_end_at_admission():
+    """More events in one step than the wrapper's buffer was made for (requests that may generate
+    nothing end as they reach the head of the queue)."""
+    s, model, cache = make(reqs=2)
+    rids = [s.submit([1, 2, 3], greedy(0)) for _ in range(200)]
+    last = s.submit([4, 5], greedy(1))
+    out = s.step()
+    assert out.finished[:200] == rids and all(s.finished[r].finish_reason == FinishReason.LENGTH for r in rids)
+    assert s.finished[last].output_tokens and not s.has_work()
+    assert cache.free_slots() == 2
+    cache.check()
