@@ -103,13 +103,17 @@ def measure(entry: Dict, base: str) -> Dict:
     loop = DecodeLoop(engine, rids, first)
     loop.run(WARMUP_STEPS)
     torch.cuda.synchronize()
-    wall, seq_lens = [], []
+    wall, gpu, seq_lens = [], [], []
     for _ in range(runs):
         seq_lens.append([engine.cached_tokens(r) + n_decode // 2 for r in rids])
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
+        begin.record()
         loop.run(n_decode)
+        end.record()
         torch.cuda.synchronize()
         wall.append(time.perf_counter() - t0)
+        gpu.append(begin.elapsed_time(end) * 1e-3)
     mid = wall.index(_median(wall))
     decode_s = wall[mid]
     step_bytes = roofline.decode_bytes(engine, seq_lens[mid])
@@ -121,7 +125,12 @@ def measure(entry: Dict, base: str) -> Dict:
             "bytes_per_token": int(step_bytes // batch), "ceiling_gbps": roofline.HBM_BYTES_PER_S / 1e9,
             "decode_tok_s": round(tok_s, 1), "roofline_tok_s": round(roof, 1),
             "roofline_pct": round(100.0 * tok_s / roof, 2), "wall_ms": round(1e3 * decode_s, 3),
-            "ms_per_step": round(1e3 * decode_s / n_decode, 4), "prefill_tokens": n_prompt,
+            "ms_per_step": round(1e3 * decode_s / n_decode, 4),
+            # per decode step, as the reference's rows have them (src/bench.rs:92-106): the time between the
+            # first and the last of the run's launches on the device, what is left of the wall time, and
+            # the time the step's bytes take at the ceiling
+            "gpu_ms": round(1e3 * gpu[mid] / n_decode, 4), "host_ms": round(1e3 * (decode_s - gpu[mid]) / n_decode, 4),
+            "weights_ms": round(1e3 * step_bytes / roofline.HBM_BYTES_PER_S, 4), "prefill_tokens": n_prompt,
             "prefill_tok_s": round(n_prompt / prefill_s, 1),
             "prefill_peak_frac": round(roofline.prefill_flops(engine, n_prompt) / prefill_s
                                        / roofline.PEAK_FLOPS[entry["dtype"]], 4)}
