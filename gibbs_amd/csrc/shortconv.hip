@@ -80,13 +80,21 @@ template <int K>
 __global__ __launch_bounds__(64) void shortconv_bf16x8_kernel(
     const bf16* __restrict__ bcx, const float* __restrict__ taps, const float* __restrict__ bias,
     float* __restrict__ state, long slot_stride, const int* __restrict__ cu, const int* __restrict__ ctx,
-    const int* __restrict__ slot, bf16* __restrict__ y, int n_req, int C) {
+    const int* __restrict__ slot, bf16* __restrict__ y, int n_req, int C, int one_row_each) {
   int tile = blockIdx.y, r = 0, q = 0;
-  for (; r < n_req; ++r) {
-    q = cu[r + 1] - cu[r];
-    const int t = (q + TLV - 1) / TLV;
-    if (tile < t) break;
-    tile -= t;
+  // as many rows as requests: if every request brings one row (decoded tokens only), tile i is
+  // request i and there is no walk over the requests; any other split of the rows takes the walk
+  if (one_row_each && tile < n_req && cu[tile] == tile && cu[tile + 1] == tile + 1) {
+    r = tile;
+    q = 1;
+    tile = 0;
+  } else {
+    for (; r < n_req; ++r) {
+      q = cu[r + 1] - cu[r];
+      const int t = (q + TLV - 1) / TLV;
+      if (tile < t) break;
+      tile -= t;
+    }
   }
   if (r >= n_req) return;
   const int c0 = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
@@ -190,9 +198,10 @@ GIBBS_EXPORT int gibbs_shortconv(const void* bcx, const float* taps, const float
     GIBBS_REQUIRE(vgrid.y <= 65535, "shortconv: too many row tiles (%d)", (int)vgrid.y);
     const bf16* in = (const bf16*)bcx;
     bf16* out = (bf16*)y;
-    if (K == 2) shortconv_bf16x8_kernel<2><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
-    else if (K == 3) shortconv_bf16x8_kernel<3><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
-    else shortconv_bf16x8_kernel<4><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C);
+    const int one = n_rows == n_req;
+    if (K == 2) shortconv_bf16x8_kernel<2><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
+    else if (K == 3) shortconv_bf16x8_kernel<3><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
+    else shortconv_bf16x8_kernel<4><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
   } else if (dtype == GIBBS_BF16)
     shortconv_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)bcx, taps, bias, state, slot_stride, cu, ctx,
                                                      slot, (bf16*)y, n_req, C, K);
