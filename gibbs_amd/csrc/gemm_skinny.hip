@@ -93,7 +93,12 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
     for (int u = 0; u < U; ++u) read_slot[u] = r * CH + ((u * 4 + g - r * U / 4) & (CH - 1));
   }
-  for (int k = k_begin; k < k_end; k += 32 * U) {
+  // every workgroup of a k slice reads the same rows of X: workgroup b starts b iterations into its
+  // waves' ranges and wraps around, so that they do not ask the same L2 channels at the same time
+  const int n_iter = (k_end - k_begin + 32 * U - 1) / (32 * U);
+  const int first_iter = (STAGE && n_iter > 0) ? (int)(blockIdx.x % n_iter) : 0;
+  for (int it = 0; it < n_iter; ++it) {
+    const int k = k_begin + ((it + first_iter) % n_iter) * 32 * U;
     bf16x8 a[U][FT], b[U][NT];
     if (STAGE) {
       bf16x8 sv[NT][LPT];

@@ -34,6 +34,7 @@ enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_GLU = 2, EPI_CONV = 3 };
 constexpr int MAX_TAPS = 8;
 
 struct FusedArgs {
+  int rotate;     // 1: workgroups start at different k (see the kernel)
   const bf16* W;
   int packed;        // W is in tile order
   int ktiles;        // packed: 32-k tiles per 16-row tile
@@ -186,7 +187,13 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
     for (int u = 0; u < U; ++u) read_slot[u] = r * CH + ((u * 4 + g - r * U / 4) & (CH - 1));
   }
-  for (int k = k_begin; k < k_end; k += 32 * U) {
+  // Every workgroup reads the same rows of X: started at the same k, all of them would ask the same L2
+  // channels for the same lines at the same time.  Workgroup b starts b iterations into its waves'
+  // ranges and wraps around (the order of a feature's additions is fixed by its workgroup).
+  const int n_iter = (k_end - k_begin + 32 * U - 1) / (32 * U);
+  const int first_iter = (STAGE && n_iter > 0 && a.rotate) ? (int)(blockIdx.x % n_iter) : 0;
+  for (int it = 0; it < n_iter; ++it) {
+    const int k = k_begin + ((it + first_iter) % n_iter) * 32 * U;
     bf16x8 av[U][FT][RG], bv[U][NT];
     if (STAGE) {
       bf16x8 sv[NT][LPT];
@@ -414,6 +421,8 @@ int check_common(const char* what, const void* X, const void* W, int N, int O, i
 
 // A row stride of 0 says that W is in tile order (pack_weight).
 void note_layout(FusedArgs& a) {
+  static const int rotate = getenv("GIBBS_SKINNY_ROTATE") ? atoi(getenv("GIBBS_SKINNY_ROTATE")) : 1;   // for measurements
+  a.rotate = rotate;
   if (a.ldw != 0) return;
   a.packed = 1;
   a.ktiles = ceil_div(a.I, 32);
