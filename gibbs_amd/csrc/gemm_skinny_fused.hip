@@ -385,7 +385,7 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
     }
   }
   // few features: halve the rows per workgroup so that every compute unit gets one
-  if (NT <= 2 && a.O / 16 < rows8_below) {
+  if ((NT <= 2 || EPI == EPI_CONV) && a.O / 16 < rows8_below) {
     gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
   } else {
     gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
