@@ -328,7 +328,7 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
         waves = auto_waves if waves is None else waves
     partial = None
     if n_splits > 1:
-        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=qkv.device)
+        partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=qkv.device)
     if out is None:
         out = torch.empty((n_rows, nh * hd), dtype=qkv.dtype, device=qkv.device)
     assert out.shape == (n_rows, nh * hd) and out.dtype == qkv.dtype and out.is_contiguous()
@@ -457,6 +457,11 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
 DECODE_KINDS = {"auto": 0, "valu": 1, "mfma": 2}
 
 
+def slices_workspace(n_rows: int, nh: int, hd: int, n_splits: int) -> int:
+    """Floats that the key slices of an attention call leave for the merge kernel."""
+    return int(library().gibbs_attention_decode_workspace(n_rows, nh, hd, n_splits))
+
+
 MATRIX_SLICE_PAGES = 510   # page ids of a key slice that the matrix-core walk keeps in LDS
 
 
@@ -502,7 +507,7 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
         waves = auto_waves if waves is None else waves
     partial = None
     if n_splits > 1:
-        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=q.device)
+        partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=q.device)
     if out is None:
         out = torch.empty((n_rows, nh * hd), dtype=q.dtype, device=q.device)
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
@@ -553,7 +558,7 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
         n_splits = prefill_splits(-(-rows // 64) + reqs // 2, nh, max_seq, window) if max_seq > 0 else 1
     partial = None
     if n_splits > 1:
-        partial = torch.empty(n_rows * nh * n_splits * (hd + 2), dtype=torch.float32, device=q.device)
+        partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=q.device)
     call("gibbs_attention_prefill", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(cu[first_req:]),
          ptr(ctx[first_req:]), ptr(table[first_req:]), reqs, table.shape[1], page_size, num_pages, rows, nh, nkv, hd,
          q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), int(n_splits), int(first_row), stream())

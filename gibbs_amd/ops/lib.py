@@ -81,6 +81,8 @@ def library() -> ctypes.CDLL:
                     fn = getattr(lib, name)
                     fn.argtypes = argtypes
                     fn.restype = c_int
+                lib.gibbs_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
+                lib.gibbs_attention_decode_workspace.restype = c_long
                 _lib = lib
     return _lib
 
