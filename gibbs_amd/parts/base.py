@@ -21,7 +21,7 @@ runs norm + part + residual add for a step of single decoded tokens in a few fus
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence, Type
 
 import torch
@@ -37,6 +37,7 @@ class Runtime:
     device: torch.device
     act_dtype: torch.dtype          # activations and cache pages: bfloat16, or float32 for the 32-bit path
     max_positions: int = 0          # positions a request can reach (tables over positions are sized by it); 0: unknown
+    shared: Dict = field(default_factory=dict)   # what parts of one model derive once and share (tables)
 
 
 @dataclass

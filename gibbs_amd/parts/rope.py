@@ -51,6 +51,9 @@ class RotaryPosition(PositionEncoding):
 
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
         self.rt = rt
-        self.inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)
         n_pos = min(int(rt.max_positions), MAX_TABLE_POSITIONS)
-        self.cos_sin = ops.rope_table(self.inv_freq, n_pos) if n_pos > 0 else None
+        key = ("rope", self.rotary_dim, self.theta, self.precision, n_pos)
+        if key not in rt.shared:        # the layers of a model that have the same encoding share one table
+            inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)
+            rt.shared[key] = (inv_freq, ops.rope_table(inv_freq, n_pos) if n_pos > 0 else None)
+        self.inv_freq, self.cos_sin = rt.shared[key]
