@@ -12,7 +12,8 @@
 // When pages run out (the reference goes on without them, :1296-1299, :1397-1400): a decoding request
 // that cannot get its next page preempts the youngest running request, which returns to the head of
 // the queue to be recomputed; a prompt portion shrinks to what is free or waits; if nothing can move
-// the youngest is preempted; a request larger than the pool fails.
+// the youngest is preempted; admission leaves the running requests the page of their next token; a
+// request larger than the pool fails.
 #include <deque>
 
 #include "cache_core.h"
@@ -194,7 +195,13 @@ HOST_EXPORT int gibbs_sched_plan(void* sched, long* plan, int plan_cap, long* ev
   const long budget = s->budget;
   const long cap = s->chunk > 0 ? std::min(budget, s->chunk) : budget;
 
-  // 1. admission: first in, first out; needs a slot and the pages of the first portion
+  // 1. admission: first in, first out; needs a slot and the pages of the first portion, beside the
+  //    page that every running request needs for its next token.  (Without that margin a request that
+  //    was preempted to make room takes the freed page back at once, fills it, is preempted again, and
+  //    the running requests that wait for a page never move.)
+  std::vector<long> margin(c->n_groups(), 0);
+  for (int id : s->active)
+    for (int g = 0; g < c->n_groups(); ++g) margin[g] += c->pages_needed(c->requests[s->seqs[id].slot], 1, g);
   while (!s->waiting.empty()) {
     const int id = s->waiting.front();
     Seq& q = s->seqs[id];
@@ -213,7 +220,10 @@ HOST_EXPORT int gibbs_sched_plan(void* sched, long* plan, int plan_cap, long* ev
     }
     const int slot = gibbs_cache_admit(c);
     if (slot < 0) break;
-    if (gibbs_cache_reserve(c, slot, std::min(total, cap)) < 0) {
+    bool room = true;
+    for (int g = 0; g < c->n_groups(); ++g)
+      room = room && c->pages_needed(c->requests[slot], std::min(total, cap), g) + margin[g] <= c->pools[g].n_free();
+    if (!room || gibbs_cache_reserve(c, slot, std::min(total, cap)) < 0) {
       gibbs_cache_release(c, slot);
       break;
     }

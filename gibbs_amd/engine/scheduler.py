@@ -20,7 +20,9 @@ takes it from the youngest running request, which is preempted: its pages and sl
 it returns to the front of the waiting queue with all its tokens so far, to be recomputed as a
 prompt (state of fixed size cannot be rewound or swapped by position, so recomputation is the
 only exact way).  A prompt portion that cannot get pages shrinks to what is free, or waits.  If
-no request can move at all, the youngest is preempted so that the oldest can.  A request that
+no request can move at all, the youngest is preempted so that the oldest can.  Admission leaves,
+beside the pages of the newcomer's first portion, the page that every running request needs for
+its next token: a preempted request must not take the freed page straight back.  A request that
 does not fit the whole pool alone fails with an error.
 
 The decisions themselves are native code (csrc/host/scheduler.cpp: it works on lengths and counts and

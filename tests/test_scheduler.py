@@ -211,3 +211,54 @@ def test_many_requests_that_end_at_admission():
     assert s.finished[last].output_tokens and not s.has_work()
     assert cache.free_slots() == 2
     cache.check()
+
+
+def test_preempted_request_does_not_take_the_freed_page_back():
+    """Two running requests wait at a page's edge for a page; the youngest, preempted to make room,
+    must not take the freed page back at its next admission (it would fill it, be preempted again,
+    and the two would wait for ever)."""
+    lens, news = [2, 1, 50, 26, 40, 3, 1], [0, 6, 2, 2, 1, 2, 0]
+    s, model, cache = make(pages=4, reqs=3, ps=16, budget=3, chunk=16)
+    rids = [s.submit([7 + i] * n, greedy(m)) for i, (n, m) in enumerate(zip(lens, news))]
+    steps = 0
+    while s.has_work():
+        s.step()
+        cache.check()
+        steps += 1
+        assert steps < 400, "the scheduler does not get on"
+    assert [len(s.finished[r].output_tokens) for r in rids] == news
+    assert cache.free_pages() == 4 and cache.free_slots() == 3
+
+
+def test_random_workloads_always_finish_with_the_tokens_of_a_run_alone():
+    """Random pools, budgets and requests, the pool never smaller than the largest request needs:
+    every request ends with the tokens it gets alone, nothing is lost, and the number of steps
+    stays within what one token per step would take many times over."""
+    import random
+    for case in range(300):
+        rng = random.Random(case)
+        ps = rng.choice([2, 4, 16])
+        n = rng.randint(1, 8)
+        lens = [rng.choice([1, 2, rng.randint(3, 60)]) for _ in range(n)]
+        news = [rng.choice([0, 1, rng.randint(2, 30)]) for _ in range(n)]
+        most = max(-(-(a + b) // ps) for a, b in zip(lens, news))
+        pages = rng.randint(most, most + rng.choice([0, 1, 3, 20]))
+        reqs = rng.randint(1, 5)
+        budget = rng.choice([1, 2, 3, 8, 64])
+        chunk = rng.choice([None, 1, 5, 16])
+        s, model, cache = make(pages=pages, reqs=reqs, ps=ps, budget=budget, chunk=chunk)
+        prompts = [[rng.randint(0, 99) for _ in range(a)] for a in lens]
+        rids = [s.submit(p, greedy(m)) for p, m in zip(prompts, news)]
+        steps, bound = 0, 50 * (sum(lens) + sum(news)) + 100
+        while s.has_work():
+            s.step()
+            steps += 1
+            assert steps < bound, f"case {case}: no end after {steps} steps"
+        cache.check()
+        assert cache.free_pages() == pages and cache.free_slots() == reqs, f"case {case}"
+        for rid, p, m in zip(rids, prompts, news):
+            got = s.finished[rid]
+            assert got.error is None and len(got.output_tokens) == m, f"case {case}: request {rid}: {got.error}"
+            s2, _, _ = make(pages=64, ps=16)
+            r2 = s2.submit(p, greedy(m))
+            assert s2.run()[r2].output_tokens == got.output_tokens, f"case {case}: request {rid}"
