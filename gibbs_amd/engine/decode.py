@@ -8,6 +8,8 @@ steps of a `run` are reserved, and the block tables uploaded, before the first o
 """
 from __future__ import annotations
 
+import contextlib
+import gc
 from typing import Hashable, List, Optional, Sequence
 
 import numpy as np
@@ -23,6 +25,23 @@ from .engine import Engine, OutOfPages, StepError
 # steps per launch of the longer captured graph (a launch costs the host and the queue about as much
 # as four kernels of a step)
 UNROLL = 8
+
+
+@contextlib.contextmanager
+def capture(graph: "torch.cuda.CUDAGraph"):
+    """Captures into `graph` with Python's cycle collector switched off.  The collector may run at
+    any allocation; if it then destroys the graphs of a loop that was dropped earlier (a loop, its
+    engine and its batch hold each other), a capturing stream refuses the call and the error, raised
+    from a destructor, ends the process.  What can be collected is collected before the capture."""
+    gc.collect()
+    was_enabled = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield
+    finally:
+        if was_enabled:
+            gc.enable()
 
 
 class DecodeLoop:
@@ -178,7 +197,7 @@ class DecodeLoop:
                 self.u.copy_(self.u_all[self.steps_done])
             g = torch.cuda.CUDAGraph()
             torch.cuda.synchronize()
-            with torch.cuda.graph(g):
+            with capture(g):
                 self._step()
             self.graph = g                                  # the capture itself ran nothing
         left = n_steps
@@ -186,7 +205,7 @@ class DecodeLoop:
             if self.graph_many is None:
                 g = torch.cuda.CUDAGraph()
                 torch.cuda.synchronize()
-                with torch.cuda.graph(g):
+                with capture(g):
                     for _ in range(UNROLL):
                         self._step()
                 self.graph_many = g

@@ -224,6 +224,34 @@ def test_decode_loop_graph_replays_match_eager(dirs, dtype):
     assert loop.tokens() == got
 
 
+def test_dropped_loops_are_collected_before_a_capture(dirs):
+    """A decode loop that was dropped while something still points at it in a cycle is garbage that
+    only Python's collector frees; the collector must not get to its graphs while another loop
+    captures (a capturing stream refuses the destruction of a graph)."""
+    import gc
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.engine.decode import DecodeLoop
+    d = dirs["A"]
+    prompt = H.tokens(3, 12, 256)
+    def loop_of(eng, rid):
+        first = int(eng.step([Entry(rid, prompt, [len(prompt) - 1])]).argmax(-1).item())
+        loop = DecodeLoop(eng, [rid], [first])
+        loop.run(9)
+        return loop
+    eng = Engine(d, dtype="bfloat16", max_tokens=512, max_requests=4)
+    old = loop_of(eng, "old")
+    want = old.tokens()
+    old.cycle = old                       # garbage that reference counting alone does not free
+    del old
+    threshold = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)             # the collector now runs at almost every allocation
+    try:
+        new = loop_of(eng, "new")
+    finally:
+        gc.set_threshold(*threshold)
+    assert new.tokens() == want and gc.isenabled()
+
+
 def trace_lines(steps):
     return "".join(json.dumps({"step": i, "entries": [{"id": r, "tokens": t, "want": w} for r, t, w in e], "end": end}) + "\n"
                    for i, (e, end) in enumerate(steps))
