@@ -51,8 +51,19 @@ TINY_D = {
     "conv_L_cache": 5, "conv_bias": False, "rope_theta": 10000.0, "norm_eps": 1e-5,
     "max_position_embeddings": 512,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
-GAIN_STD = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1}
+# Medium M: the serving shapes in small: heads of 64, grouping 4:1, every size aligned, so that the
+# engine takes its fast kernels (matrix-core attention for prompts and decoding, packed weights, the
+# library product above 64 rows) on sequences long enough for key slices and many pages.
+MEDIUM_M = {
+    "architectures": ["Lfm2ForCausalLM"], "model_type": "lfm2",
+    "num_hidden_layers": 4, "layer_types": ["conv", "full_attention", "conv", "full_attention"],
+    "hidden_size": 512, "num_attention_heads": 8, "num_key_value_heads": 2, "head_dim": 64,
+    "block_ff_dim": 1536, "block_auto_adjust_ff_dim": False, "vocab_size": 4096, "tie_embedding": True,
+    "conv_L_cache": 3, "conv_bias": False, "rope_theta": 1000000.0, "norm_eps": 1e-5,
+    "max_position_embeddings": 8192,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "M": MEDIUM_M}
+GAIN_STD = {"A": 0.0, "B": 0.1, "C": 0.1, "D": 0.1, "M": 0.1}
 
 
 def make_model_dir(folder: str, name: str, seed: int = 0, std: float = 0.1, dtype: str = "bfloat16") -> str:

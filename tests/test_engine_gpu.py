@@ -203,6 +203,37 @@ def test_long_decoding(model_dirs, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_medium_model_long_sequences(tmp_path_factory, dtype):
+    """Heads of 64 and aligned sizes (the fast kernels, packed weights, the library product above 64
+    rows) on sequences of up to 2,209 tokens: portions of changing size up to 2,048 beside another
+    request's portions and decoded tokens, the last tokens one by one over many pages and key slices."""
+    d = H.make_model_dir(str(tmp_path_factory.mktemp("medium")), "M", seed=5, std=0.05)
+    rng = np.random.default_rng(3)
+    seqs = {"long": H.tokens(31, 2209, 4096), "mid": H.tokens(32, 563, 4096), "short": H.tokens(33, 70, 4096)}
+    tail = {"long": 24, "mid": 40, "short": 8}
+    at = {r: 0 for r in seqs}
+    steps = []
+    while at:
+        entries, ends = [], []
+        for r in list(at):
+            left = len(seqs[r]) - at[r]
+            n = 1 if left <= tail[r] else min(left - tail[r], int(rng.choice([2, 16, 65, 128, 512, 2048])))
+            want = sorted({0, n // 2, n - 1})
+            entries.append((r, seqs[r][at[r]:at[r] + n], want))
+            at[r] += n
+            if at[r] == len(seqs[r]):
+                ends.append(r)
+                del at[r]
+        entries.sort(key=lambda e: len(e[1]) != 1)      # decoded tokens at the head, as the scheduler puts them
+        steps.append((entries, ends))
+    eng = make_engine(d, dtype, max_tokens=3072, max_requests=3, page_size=16)
+    got = run_steps(eng, steps)
+    check(d, seqs, got, dtype, f"medium {dtype}", against_whole=False)
+    eng.cache.check()
+    assert eng.cache.free_pages() == eng.cache.pools[0].num_pages
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_first_tokens(model_dirs, name, dtype):
     """Positions 0, 1, 2 fed one by one: empty history in the convolution and a single key."""
