@@ -258,6 +258,87 @@ def test_layer_order_and_shared_cache(name, dtype, tmp_path):
     H.assert_close(np.concatenate(got), want, name, "hand-built spec")
 
 
+def window_spec(hidden=40, vocab=83, window=20):
+    """Layer 0 attends to all keys, layer 1 to a window of them (other head counts, so a cache group of
+    its own), layer 2 is a short convolution."""
+    from gibbs_amd.config import FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec
+    rope = PositionSpec("rope", {"theta": 1e4, "rotary_dim": 16, "precision": "f32"})
+    layers = []
+    for i, kind in enumerate(["full", "window", "short_conv"]):
+        p = f"l{i}"
+        if kind == "short_conv":
+            mixer = MixerSpec("short_conv", {"width": hidden, "kernel": 3, "bias": False},
+                              {"in_proj": f"{p}.in", "conv": f"{p}.taps", "out_proj": f"{p}.out"})
+        else:
+            heads, kv = (4, 2) if kind == "full" else (3, 1)
+            mixer = MixerSpec("attention", {"heads": heads, "kv_heads": kv, "head_dim": 16, "scale": 0.25, "qk_norm": "before",
+                                            "qk_norm_eps": 1e-5, "window": window if kind == "window" else None},
+                              {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o",
+                               "q_norm": f"{p}.qn", "k_norm": f"{p}.kn"}, rope)
+        ffn = FeedForwardSpec("glu", {"inter": 56, "activation": "silu"}, {"gate": f"{p}.w1", "up": f"{p}.w3", "down": f"{p}.w2"})
+        layers.append(LayerSpec(p, "pre_norm", NormSpec("rms", 1e-5, f"{p}.n1"), mixer, NormSpec("rms", 1e-5, f"{p}.n2"), ffn))
+    return ModelSpec("Windowed", hidden, vocab, tuple(layers), (0, 1, 2), "emb", NormSpec("rms", 1e-5, "fn"), None, 512)
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
+    """A model whose layers need different caches: all keys in one group, a window of 20 in another.
+    Three requests through the engine, portions beside decoded tokens, in a pool of 24 pages of 8
+    tokens per group: the window group hands out 29 pages over the run, so pages that a window has
+    passed are in use again while their first owner still runs; the logits equal the plain model's."""
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import random_tensor
+    spec = window_spec()
+    decls = DecoderModel(spec).tensor_decls()
+    tensors = {d.name: random_tensor(d, 9, torch.bfloat16, std=0.15, gain_std=0.1) for d in decls}
+
+    class Windowed(ArchConfig):
+        def model_spec(self):
+            return spec
+    ws = store({k: v.float().numpy() for k, v in tensors.items()}, decls, dtype)
+    eng = Engine(config=Windowed(), weights=ws, dtype=name, max_tokens=24 * 8, max_requests=2, page_size=8)
+    cm = eng.cache
+    assert cm.n_groups == 2 and cm.group_layers == [[0], [1]]
+    win = 1                                                     # the window's group
+    seqs = {"a": H.tokens(1, 150, spec.vocab), "b": H.tokens(2, 40, spec.vocab), "c": H.tokens(3, 40, spec.vocab)}
+    plain = {r: plain_spec_forward(spec, {k: v.double().numpy() for k, v in tensors.items()}, ids) for r, ids in seqs.items()}
+    got = {r: [] for r in seqs}
+    at = {r: 0 for r in seqs}
+    owners, used_again = {}, 0                                   # page of the window group -> (request, index in its table)
+    def step(parts):
+        nonlocal used_again
+        entries = [Entry(r, seqs[r][at[r]:at[r] + n], list(range(n))) for r, n in parts]
+        rows = eng.step(entries).cpu().numpy()
+        i = 0
+        for r, n in parts:
+            got[r].append(rows[i:i + n]); i += n; at[r] += n
+            table = cm.block_table([r], win)[0]
+            held = [(j, int(pg)) for j, pg in enumerate(table) if pg >= 0]
+            assert len(held) <= 20 // 8 + 2, f"request {r} holds {len(held)} pages of the window group"
+            for j, pg in held:
+                if pg in owners and owners[pg] != (r, j):
+                    used_again += 1
+                owners[pg] = (r, j)
+            if at[r] == len(seqs[r]):
+                eng.release(r)
+        cm.check()
+    step([("a", 37)])
+    step([("a", 1), ("b", 9)])
+    for _ in range(15):
+        step([("a", 1), ("b", 2)])
+    step([("a", 40), ("b", 1)])                                 # b ends (40 tokens)
+    step([("a", 2), ("c", 33)])
+    for _ in range(7):
+        step([("a", 1), ("c", 1)])                              # c ends
+    step([("a", 150 - at["a"])])
+    assert not any(r in cm for r in seqs) and all(cm.free_pages(g) == 24 for g in range(2))
+    assert used_again >= 5, "the pool was meant to be so small that pages a window has passed are used again"
+    for r in seqs:
+        H.assert_close(np.concatenate(got[r]), plain[r], name, f"windowed model request {r}")
+
+
 # --------------------------------------------------------------------------- a toy mixer with its own state
 def register_toy():
     """An exponential moving average over time of a projection of the input: state [hidden] per
