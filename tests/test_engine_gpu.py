@@ -234,6 +234,33 @@ def test_medium_model_long_sequences(tmp_path_factory, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_sequence_past_one_segment_of_page_ids(tmp_path_factory, dtype):
+    """4,400 tokens in pages of 8: more than the 512 page ids that the attention kernels keep in LDS
+    at a time, so prompt portions and decoded tokens late in the sequence walk a second segment (or
+    are cut into more key slices); a short request rides along."""
+    d = H.make_model_dir(str(tmp_path_factory.mktemp("medium")), "M", seed=6, std=0.05)
+    seqs = {"long": H.tokens(41, 4400, 4096), "other": H.tokens(42, 90, 4096)}
+    at = {"long": 0, "other": 0}
+    cuts = [2048, 2000, 130, 64, 17, 2]
+    steps = []
+    while at["long"] < 4400:
+        left = 4400 - at["long"]
+        n = min(cuts.pop(0), left - 40) if cuts and left > 40 else 1
+        want = sorted({0, n // 2} | set(range(max(0, n - 4), n)))
+        entries = [("long", seqs["long"][at["long"]:at["long"] + n], want)]
+        at["long"] += n
+        if at["other"] < 90:
+            m = 1 if at["other"] >= 60 else 30
+            entries.insert(0 if m == 1 else 1, ("other", seqs["other"][at["other"]:at["other"] + m], [m - 1]))
+            at["other"] += m
+        steps.append((entries, []))
+    eng = make_engine(d, dtype, max_tokens=4608, max_requests=2, page_size=8)
+    got = run_steps(eng, steps)
+    assert ("long", 4399) in got and sum(1 for r, p in got if r == "long" and p > 4096) >= 50
+    check(d, seqs, got, dtype, f"past one segment {dtype}", against_whole=False)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_first_tokens(model_dirs, name, dtype):
     """Positions 0, 1, 2 fed one by one: empty history in the convolution and a single key."""
