@@ -35,6 +35,8 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--temperature", type=float, default=None, help="sampling temperature (one-shot default 0.7; <= 1e-4 is greedy)")
     ap.add_argument("--top-p", type=float, default=None, help="nucleus cut (default 0.9)")
     ap.add_argument("--top-k", type=int, default=50, help="candidates (default 50, at most 64)")
+    ap.add_argument("--repetition-penalty", type=float, default=1.0,
+                    help="penalty on the tokens among the last 64 (default 1.0: none, as the reference's scheduler passes)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "fp32"])
     ap.add_argument("--random-weights", metavar="CONFIG_JSON",
                     help="write a model folder with random weights from this config.json into --model, then go on")
@@ -162,7 +164,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     temperature = 0.7 if args.temperature is None else args.temperature       # main.rs:744-749
     gen = Generator(engine, max_batch_tokens=args.max_batch_tokens, chunk=args.chunk)
     rid = gen.submit(prompt, SamplingParams(temperature, args.top_p, args.top_k, max_tokens, args.seed,
-                                            args.ignore_eos or tok is None))
+                                            args.ignore_eos or tok is None, args.repetition_penalty))
     result = gen.run()[rid]
     st = gen.stats
     print(f"⚡ Prefill: {st.prefill_tokens} tokens in {st.prefill_seconds * 1e3:.2f}ms ({st.prefill_tok_s:.1f} tok/s)")

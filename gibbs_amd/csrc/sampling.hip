@@ -245,6 +245,50 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
 }
 }  // namespace
 
+// Repetition penalty of the reference's sampler, applied to the logits in place before a row is
+// sampled.  A token that occurs c times among the row's recent tokens (the reference passes the last
+// 64 of prompt and output): greedy rows (/root/reference/src/runtime/lm.rs:1089-1105): c times
+// v = v > 0 ? v / penalty : v * penalty, then v -= 1.5 c; sampled rows (:1176-1189): c times
+// v = (v > 0 ? v / penalty : v * penalty) - 1.5.  Rows whose penalty is <= 1 are left alone (:1072,
+// :1163).  One workgroup of R threads per row; the first thread that holds a token does its update.
+__global__ void repetition_penalty_kernel(float* __restrict__ logits, long ld, int V, const int* __restrict__ recent,
+                                          int R, const float* __restrict__ penalty,
+                                          const float* __restrict__ temperature) {
+  extern __shared__ int s_recent[];
+  const int m = blockIdx.x, j = threadIdx.x;
+  const float p = penalty[m];
+  if (!(p > 1.0f)) return;
+  const int t = recent[(size_t)m * R + j];
+  s_recent[j] = t;
+  __syncthreads();
+  if (t < 0 || t >= V) return;
+  int count = 0;
+  for (int i = 0; i < R; ++i) {
+    if (s_recent[i] == t) {
+      if (i < j) return;          // an earlier thread holds this token
+      count += 1;
+    }
+  }
+  float v = logits[(size_t)m * ld + t];
+  if (temperature[m] <= 1e-4f) {
+    for (int c = 0; c < count; ++c) v = v > 0.f ? v / p : v * p;
+    v -= 1.5f * (float)count;
+  } else {
+    for (int c = 0; c < count; ++c) v = (v > 0.f ? v / p : v * p) - 1.5f;
+  }
+  logits[(size_t)m * ld + t] = v;
+}
+
+// recent: [M, R] token ids (negative: none), R <= 1024; penalty, temperature: [M].
+GIBBS_EXPORT int gibbs_repetition_penalty(float* logits, int M, int V, long ld, const int* recent, int R,
+                                          const float* penalty, const float* temperature, hipStream_t stream) {
+  GIBBS_REQUIRE(M >= 0 && V > 0 && ld >= V, "repetition_penalty: bad sizes M=%d V=%d ld=%ld", M, V, ld);
+  GIBBS_REQUIRE(R >= 1 && R <= 1024, "repetition_penalty: %d recent tokens a row outside 1..1024", R);
+  if (M == 0) return 0;
+  repetition_penalty_kernel<<<M, R, R * sizeof(int), stream>>>(logits, ld, V, recent, R, penalty, temperature);
+  GIBBS_LAUNCH_STATUS("repetition_penalty");
+}
+
 GIBBS_EXPORT int gibbs_argmax(const float* logits, int* out, int M, int V, long ld, hipStream_t stream) {
   GIBBS_REQUIRE(M >= 0 && V > 0 && ld >= V, "argmax: bad sizes M=%d V=%d ld=%ld", M, V, ld);
   if (M == 0) return 0;

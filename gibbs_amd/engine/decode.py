@@ -104,6 +104,8 @@ class DecodeLoop:
         self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * b
         if self.greedy != all(p.greedy for p in self.params):
             raise StepError("a decode loop is captured either for greedy or for sampled requests")
+        if any(p.penalises for p in self.params):
+            raise StepError("a repetition penalty reads the recent tokens on the host: such requests step through the scheduler")
         self.index = list(first_index) if first_index is not None else [0] * b
         h = self._host
         h[self._sec[0]] = np.asarray(last_tokens, dtype=np.int32)

@@ -86,6 +86,8 @@ class Generator:
         greedy = all(p.greedy for p in params)
         if not greedy and not all(not p.greedy for p in params):
             return None                                     # mixed greedy and sampled: step by step
+        if any(p.penalises for p in params):
+            return None                                     # the penalty reads the recent tokens on the host
         last = [s.output_tokens[-1] for s in seqs]
         index = [len(s.output_tokens) for s in seqs]
         key = (len(seqs), greedy)
@@ -139,10 +141,10 @@ class Generator:
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_tokens: int = 64,
              temperature: Optional[float] = None, top_p: Optional[float] = None, top_k: int = 50, seed: int = 0,
              ignore_eos: bool = False, max_batch_tokens: int = MAX_PREFILL_CHUNK,
-             chunk: Optional[int] = None, decode_burst: int = 16) -> List[Generation]:
+             chunk: Optional[int] = None, decode_burst: int = 16, repetition_penalty: float = 1.0) -> List[Generation]:
     """Generates a continuation of every prompt (lists of token ids), batched continuously."""
     gen = Generator(engine, max_batch_tokens=max_batch_tokens, chunk=chunk, decode_burst=decode_burst)
-    params = SamplingParams(temperature, top_p, top_k, max_tokens, seed, ignore_eos)
+    params = SamplingParams(temperature, top_p, top_k, max_tokens, seed, ignore_eos, repetition_penalty)
     rids = [gen.submit(p, params) for p in prompts]
     results = gen.run()
     return [results[r] for r in rids]

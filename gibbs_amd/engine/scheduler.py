@@ -41,7 +41,7 @@ from typing import Sequence as SeqOf
 
 from ..cache import host
 from ..cache.manager import CacheManager
-from ..sampling.sampler import Draw, SamplingParams
+from ..sampling.sampler import RECENT_TOKENS, Draw, SamplingParams
 from .batch import Entry
 
 MAX_PREFILL_CHUNK = 2048            # most prompt tokens one step prefills (scheduler/mod.rs:341)
@@ -246,7 +246,8 @@ class ContinuousBatchScheduler:
             seq = self._seqs[number]
             entries.append(Entry(seq.id, seq.span(at, n), [n - 1] if last else []))
             if last:
-                draws.append(Draw(seq.params, seq.id, len(seq.output_tokens)))
+                recent = seq.tokens[-RECENT_TOKENS:] if seq.params.penalises else ()
+                draws.append(Draw(seq.params, seq.id, len(seq.output_tokens), recent))
                 sampled_for.append(seq)
             if decoding:
                 decode_tokens += 1

@@ -577,6 +577,22 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     return out
 
 
+def repetition_penalty(logits: torch.Tensor, recent: torch.Tensor, penalty: torch.Tensor,
+                       temperature: torch.Tensor) -> torch.Tensor:
+    """Penalises, in place, the logits of the tokens in `recent` [M, R] (int32, negative: none) by the
+    reference's rule for greedy rows (temperature <= 1e-4) or sampled rows; rows with penalty <= 1
+    are left alone."""
+    require_cuda(logits, recent, penalty, temperature)
+    m, v = logits.shape
+    assert logits.dtype == torch.float32 and logits.stride(1) == 1
+    assert recent.dtype == torch.int32 and recent.dim() == 2 and recent.shape[0] == m and recent.is_contiguous()
+    for t in (penalty, temperature):
+        assert t.dtype == torch.float32 and t.numel() >= m and t.is_contiguous()
+    call("gibbs_repetition_penalty", ptr(logits), m, v, logits.stride(0) if m > 1 else v, ptr(recent), recent.shape[1],
+         ptr(penalty), ptr(temperature), stream())
+    return logits
+
+
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor, top_k: torch.Tensor,
            u: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row: top-k, softmax at the row's temperature, top-p cut, draw with u in [0, 1)."""

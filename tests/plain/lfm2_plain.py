@@ -285,6 +285,32 @@ def nucleus(logits, temperature: float, top_k: int, top_p: float):
     return cand[:cut], probs[:cut]
 
 
+def repetition_penalty(logits, recent, penalty: float, greedy: bool) -> np.ndarray:
+    """The logits as the reference's sampler sees them with a repetition penalty > 1 over the
+    recent tokens: a token that occurs c times is, c times over, divided by the penalty if its
+    value is positive and multiplied by it if not.  The greedy rule then takes 1.5 c off
+    (src/runtime/lm.rs:1089-1105); the sampling rule takes 1.5 off after each of the c steps, so a
+    value can change sign on the way (src/runtime/lm.rs:1176-1189).  A penalty <= 1 or no recent
+    tokens change nothing (src/runtime/lm.rs:1072, :1163)."""
+    out = np.array(logits, dtype=np.float32)
+    if not penalty > 1.0 or len(recent) == 0:
+        return out
+    p = np.float32(penalty)
+    for tok in sorted(set(int(t) for t in recent)):
+        if not 0 <= tok < len(out):
+            continue
+        c = sum(1 for t in recent if int(t) == tok)
+        v = out[tok]
+        for _ in range(c):
+            v = np.float32(v / p) if v > 0 else np.float32(v * p)
+            if not greedy:
+                v = np.float32(v - np.float32(1.5))
+        if greedy:
+            v = np.float32(v - np.float32(c) * np.float32(1.5))
+        out[tok] = v
+    return out
+
+
 def draw(cand, probs, u: float) -> int:
     """Pick the first candidate whose cumulative probability reaches u * sum(probs)
     (src/runtime/lm.rs:1137-1145)."""

@@ -150,6 +150,37 @@ def test_seeded_temperature_sampling(dirs):
             assert t == P.draw(cand, probs, uniform(7, request_key(rid), i)), f"request {rid} token {i}"
 
 
+def test_repetition_penalty_in_generation(dirs):
+    """Greedy and sampled requests with a repetition penalty beside a request without one: every
+    token is what the plain rule picks from the plain logits of the same history, with the last 64
+    tokens of prompt and output as the recent ones; the penalty changes the greedy continuation."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    from gibbs_amd.sampling import request_key, uniform
+    d = dirs["A"]
+    prompts = [H.tokens(50 + i, n, 256) for i, n in enumerate([70, 9, 30])]
+    params = [SamplingParams(temperature=0.0, max_new_tokens=24, repetition_penalty=1.7, ignore_eos=True),
+              SamplingParams(temperature=0.9, max_new_tokens=24, repetition_penalty=1.3, seed=11, ignore_eos=True),
+              SamplingParams(temperature=0.0, max_new_tokens=24, ignore_eos=True)]
+    eng = Engine(d, dtype="float32", max_tokens=1024, max_requests=4)
+    gen = Generator(eng, max_batch_tokens=32, chunk=16)
+    rids = [gen.submit(p, q) for p, q in zip(prompts, params)]
+    res = gen.run()
+    for rid, p, q in zip(rids, prompts, params):
+        out = res[rid].tokens
+        logits = H.plain_logits(d, p + out)
+        for i, t in enumerate(out):
+            row = P.repetition_penalty(logits[len(p) - 1 + i], (p + out[:i])[-64:], q.repetition_penalty, q.greedy)
+            if q.greedy:
+                best = P.argmax_first(row)
+                assert t == best or row[t] >= row[best] - 1e-4, f"request {rid} token {i}"
+            else:
+                cand, probs = P.nucleus(row, 0.9, 50, 0.9)
+                assert t == P.draw(cand, probs, uniform(11, request_key(rid), i)), f"request {rid} token {i}"
+    plain = plain_greedy(d, prompts[0], 24)
+    assert res[rids[0]].tokens != plain, "a penalty of 1.7 was meant to change the greedy continuation"
+    assert res[rids[2]].tokens == plain_greedy(d, prompts[2], 24)
+
+
 def test_continuous_batching_under_page_pressure(dirs):
     """A pool so small that running requests collide: the youngest is preempted and recomputed, and
     every request still gets exactly the tokens it gets alone."""

@@ -462,6 +462,35 @@ def test_sample_against_plain():
     assert g.tolist() == logits.argmax(-1).tolist()
 
 
+@pytest.mark.parametrize("V,R", [(700, 64), (65536 + 37, 64), (97, 5)])
+def test_repetition_penalty(V, R):
+    """The kernel against the plain rule, row by row: greedy and sampled rows, tokens seen once and
+    several times, positive and negative logits, ids outside the vocabulary and empty places in the
+    list, rows without a penalty (left alone bit for bit)."""
+    from gibbs_amd import ops
+    from tests.plain import lfm2_plain as P
+    rng = np.random.default_rng(V + R)
+    M = 7
+    logits = rnd(M, V, scale=3.0, seed=V)
+    recent = rng.integers(0, min(V, 12), size=(M, R)).astype(np.int32)       # few distinct ids: many repeats
+    recent[1, R // 2:] = -1                                                      # a short history
+    recent[2, 0] = V + 5                                                         # an id outside the vocabulary
+    recent[3] = rng.integers(0, V, size=R)
+    recent[6] = -1                                                               # nothing recent
+    penalty = np.array([1.3, 2.0, 1.1, 1.5, 1.0, 0.7, 1.8], dtype=np.float32)  # 1.0 and below: none
+    temp = np.array([0.0, 0.8, 1e-4, 1.2, 0.0, 0.9, 0.7], dtype=np.float32)
+    before = logits.clone()
+    got = ops.repetition_penalty(logits, i32(recent), torch.tensor(penalty, device=DEV), torch.tensor(temp, device=DEV))
+    assert got.data_ptr() == logits.data_ptr()
+    got = got.cpu().numpy()
+    for m in range(M):
+        want = P.repetition_penalty(before[m].cpu().numpy(), [t for t in recent[m] if t >= 0], float(penalty[m]),
+                                    greedy=bool(temp[m] <= 1e-4))
+        assert np.array_equal(got[m], want), f"row {m}: {np.abs(got[m] - want).max()}"
+    assert np.array_equal(got[4], before[4].cpu().numpy()) and np.array_equal(got[6], before[6].cpu().numpy())
+    assert not np.array_equal(got[0], before[0].cpu().numpy())
+
+
 @pytest.mark.parametrize("V", [65536, 50001, 700])
 def test_sample_large_vocabulary_ties_and_specials(V):
     """Top-k by two walks over the row: vocabularies beyond one element per thread, a thousand values tied

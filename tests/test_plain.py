@@ -197,3 +197,20 @@ def test_nucleus_against_full_sort():
     assert P.draw([4, 9, 2], np.array([0.5, 0.3, 0.2], dtype=np.float32), 0.0) == 4
     assert P.draw([4, 9, 2], np.array([0.5, 0.3, 0.2], dtype=np.float32), 0.6) == 9
     assert P.draw([4, 9, 2], np.array([0.5, 0.3, 0.2], dtype=np.float32), 0.999) == 2
+
+
+def test_repetition_penalty_rules():
+    """Worked by hand from the reference's two loops (src/runtime/lm.rs:1089-1105, :1176-1189): the
+    greedy rule divides c times and then subtracts 1.5 c; the sampling rule subtracts 1.5 after every
+    division, so 4.0 seen twice at penalty 2 becomes 4/2/2 - 3 = -2 when greedy and
+    (4/2 - 1.5)/2 - 1.5 = -1.25 when sampled; values that are not positive are multiplied."""
+    logits = [4.0, -1.0, 0.5, 3.0, 0.0]
+    recent = [0, 1, 0, 4, 99]                                  # 99: outside the vocabulary, ignored
+    g = P.repetition_penalty(logits, recent, 2.0, greedy=True)
+    s = P.repetition_penalty(logits, recent, 2.0, greedy=False)
+    assert g.tolist() == [-2.0, -3.5, 0.5, 3.0, -1.5]
+    assert s.tolist() == [-1.25, -3.5, 0.5, 3.0, -1.5]
+    assert P.repetition_penalty(logits, recent, 1.0, greedy=True).tolist() == logits
+    assert P.repetition_penalty(logits, [], 2.0, greedy=False).tolist() == logits
+    # the best token, seen before, loses to the runner-up; unseen, it stays the best whatever the penalty
+    assert P.argmax_first(g) == 3 and P.argmax_first(P.repetition_penalty(logits, [1, 2], 5.0, True)) == 0
