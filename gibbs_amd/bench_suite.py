@@ -149,7 +149,8 @@ def serve(entry: Dict, base: str) -> Dict:
     engine = _load(entry, base, batch=live, ctx=-(-(n_prompt + n_decode + 1) // 64) * 64)
     rng = np.random.default_rng(0)
     chunk = entry.get("chunk")
-    gen = Generator(engine, max_batch_tokens=int(entry.get("max_batch_tokens", 2048)), chunk=int(chunk) if chunk else None)
+    budget = entry.get("max_batch_tokens", 2048)
+    gen = Generator(engine, max_batch_tokens=budget if budget == "auto" else int(budget), chunk=int(chunk) if chunk else None)
     params = SamplingParams(temperature=0.0, max_new_tokens=n_decode, ignore_eos=True)
     warm = gen.submit(rng.integers(0, engine.spec.vocab, size=min(n_prompt, 64)).tolist(),
                       SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True))

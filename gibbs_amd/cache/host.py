@@ -41,6 +41,7 @@ _SIGNATURES = {
                                   _lp, _ip], c_int),
     "gibbs_sched_create": ([c_void_p, c_long, c_long, c_long], c_void_p),
     "gibbs_sched_destroy": ([c_void_p], None),
+    "gibbs_sched_set_budget": ([c_void_p, c_long], c_int),
     "gibbs_sched_submit": ([c_void_p, c_long, c_long, c_int], c_int),
     "gibbs_sched_counts": ([c_void_p, _ip, _ip], c_int),
     "gibbs_sched_list": ([c_void_p, c_int, _ip, c_int], c_int),

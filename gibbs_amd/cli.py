@@ -40,7 +40,8 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "bf16", "float32", "fp32"])
     ap.add_argument("--random-weights", metavar="CONFIG_JSON",
                     help="write a model folder with random weights from this config.json into --model, then go on")
-    ap.add_argument("--max-batch-tokens", type=int, default=2048, help="prompt tokens per scheduler step")
+    ap.add_argument("--max-batch-tokens", type=lambda v: v if v == "auto" else int(v), default=2048,
+                    help="prompt tokens per scheduler step, or 'auto': sized by measured costs as the reference's scheduler does")
     ap.add_argument("--chunk", type=int, default=None, help="most prompt tokens of one request per step")
     ap.add_argument("--page-size", type=int, default=None, help="tokens per cache page")
     ap.add_argument("--cache-tokens", type=int, default=None, help="tokens the cache pool holds")

@@ -138,6 +138,13 @@ HOST_EXPORT void* gibbs_sched_create(void* cache_core, long context_len, long ma
   return s;
 }
 HOST_EXPORT void gibbs_sched_destroy(void* sched) { delete (Scheduler*)sched; }
+// The budget of prompt tokens of the steps planned from now on (a caller that sizes it by measured
+// costs sets it before every plan).
+HOST_EXPORT int gibbs_sched_set_budget(void* sched, long max_batch_tokens) {
+  if (max_batch_tokens < 1) return fail(ERR_ARGUMENT, "a budget of %ld prompt tokens", max_batch_tokens);
+  ((Scheduler*)sched)->budget = max_batch_tokens;
+  return 0;
+}
 
 // Queues a request of prompt_len tokens that may generate max_new more; returns its number.
 HOST_EXPORT int gibbs_sched_submit(void* sched, long prompt_len, long max_new, int ignore_eos) {

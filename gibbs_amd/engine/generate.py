@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import time
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Union
 
 import torch
 
@@ -52,10 +52,11 @@ MIN_STEPS_FOR_NEW_LOOP = 8
 
 
 class Generator:
-    def __init__(self, engine: Engine, *, max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
+    def __init__(self, engine: Engine, *, max_batch_tokens: Union[int, str] = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
                  eos_token_ids: Optional[Sequence[int]] = None, decode_burst: int = 16):
-        """`decode_burst`: while nothing waits and every running request decodes, up to this many
-        decode steps run back to back as captured graphs (0: every step goes through the host)."""
+        """`max_batch_tokens`: prompt tokens per step, or "auto" for the budget that the scheduler sizes
+        by measured costs.  `decode_burst`: while nothing waits and every running request decodes, up to
+        this many decode steps run back to back as captured graphs (0: every step goes through the host)."""
         self.engine = engine
         self.decode_burst = decode_burst
         self._loops: Dict[tuple, DecodeLoop] = {}
@@ -102,10 +103,14 @@ class Generator:
             else:
                 loop.params, loop.index = params, [i - loop.steps_done for i in index]
             self._stepped = False
+            started = self.scheduler.clock()
             loop.run(n)
+            tokens = loop.tokens(last=n)                    # (reading them back waits for the steps)
         except OutOfPages:
             return None                                     # let the scheduler make room
-        return self.scheduler.apply_burst(seqs, loop.tokens(last=n))
+        if self.scheduler.tuner is not None:
+            self.scheduler.tuner.record((self.scheduler.clock() - started) / n, 0, len(seqs))
+        return self.scheduler.apply_burst(seqs, tokens)
 
     def step(self) -> StepOutput:
         """One scheduler step (or one burst of decode steps), timed: a step that holds prompt tokens
@@ -140,7 +145,7 @@ class Generator:
 
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_tokens: int = 64,
              temperature: Optional[float] = None, top_p: Optional[float] = None, top_k: int = 50, seed: int = 0,
-             ignore_eos: bool = False, max_batch_tokens: int = MAX_PREFILL_CHUNK,
+             ignore_eos: bool = False, max_batch_tokens: Union[int, str] = MAX_PREFILL_CHUNK,
              chunk: Optional[int] = None, decode_burst: int = 16, repetition_penalty: float = 1.0) -> List[Generation]:
     """Generates a continuation of every prompt (lists of token ids), batched continuously."""
     gen = Generator(engine, max_batch_tokens=max_batch_tokens, chunk=chunk, decode_burst=decode_burst)

@@ -33,10 +33,12 @@ the sampled tokens back.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
+import time
 from collections import deque
 from dataclasses import dataclass, field
 from enum import Enum
-from typing import Callable, Deque, Dict, Hashable, List, Optional, Tuple
+from typing import Callable, Deque, Dict, Hashable, List, Optional, Tuple, Union
 from typing import Sequence as SeqOf
 
 from ..cache import host
@@ -45,6 +47,43 @@ from ..sampling.sampler import RECENT_TOKENS, Draw, SamplingParams
 from .batch import Entry
 
 MAX_PREFILL_CHUNK = 2048            # most prompt tokens one step prefills (scheduler/mod.rs:341)
+INITIAL_PREFILL_CHUNK = 64          # the budget before any prefill has been timed (scheduler/mod.rs:345)
+IDLE_STEP_SECONDS = 0.1             # with nothing decoding a step's prefill is sized to take this long (:348)
+
+
+class PrefillTuner:
+    """The reference's measured budget of prompt tokens per step (scheduler/mod.rs:359-403): while
+    requests decode, a step's prompt tokens are sized to cost about one decode round (at least one
+    token, and one token only until a decode round has been timed); with nothing decoding, about
+    100 ms; 64 before any prefill has been timed; never more than 2,048.  Costs are moving averages
+    (0.75 old + 0.25 new).  The reference times every sequence's pass by itself; here a step is one
+    batch, so a step of prompt tokens beside decoded ones counts as prefill for what it took beyond
+    a decode round (and as the decode round itself while none has been timed)."""
+
+    def __init__(self):
+        self.prefill_s_per_token = 0.0      # 0: not measured yet
+        self.decode_round_s = 0.0
+
+    def budget(self, decoding: bool) -> int:
+        if self.prefill_s_per_token == 0.0:
+            return INITIAL_PREFILL_CHUNK
+        if decoding and self.decode_round_s == 0.0:
+            return 1
+        target = self.decode_round_s if decoding else IDLE_STEP_SECONDS
+        return max(1, min(int(target / self.prefill_s_per_token), MAX_PREFILL_CHUNK))
+
+    def record(self, seconds: float, prefill_tokens: int, decode_tokens: int) -> None:
+        ewma = lambda old, new: new if old == 0.0 else 0.75 * old + 0.25 * new
+        if prefill_tokens > 0 and decode_tokens > 0:
+            if self.decode_round_s == 0.0:
+                self.decode_round_s = seconds
+                return
+            seconds = max(seconds - self.decode_round_s, 0.05 * seconds)
+            self.prefill_s_per_token = ewma(self.prefill_s_per_token, seconds / prefill_tokens)
+        elif prefill_tokens > 0:
+            self.prefill_s_per_token = ewma(self.prefill_s_per_token, seconds / prefill_tokens)
+        elif decode_tokens > 0:
+            self.decode_round_s = ewma(self.decode_round_s, seconds)
 
 
 class SequenceState(Enum):          # scheduler/mod.rs:327-332
@@ -113,13 +152,18 @@ EV_ADMITTED, EV_RELEASED, EV_PREEMPTED, EV_STOP, EV_LENGTH, EV_TOO_LARGE, EV_POO
 
 class ContinuousBatchScheduler:
     def __init__(self, cache: CacheManager, runner: Runner, *, context_len: int,
-                 max_batch_tokens: int = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
-                 eos_token_ids: SeqOf[int] = ()):
+                 max_batch_tokens: Union[int, str] = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
+                 eos_token_ids: SeqOf[int] = (), clock: Callable[[], float] = time.perf_counter):
         """`cache`: the engine's cache manager (pages and slots are taken here, before a step
-        runs).  `runner`: runs one batch and samples.  `max_batch_tokens`: prompt tokens per step.
+        runs).  `runner`: runs one batch and samples.  `max_batch_tokens`: prompt tokens per step,
+        or "auto" for the reference's measured budget (`PrefillTuner`; `clock` gives its seconds).
         `chunk`: most prompt tokens of one request per step (None: the budget)."""
-        if max_batch_tokens < 1 or (chunk is not None and chunk < 1):
-            raise ValueError("max_batch_tokens and chunk must be at least 1")
+        self.tuner: Optional[PrefillTuner] = None
+        self.clock = clock
+        if max_batch_tokens == "auto":
+            self.tuner, max_batch_tokens = PrefillTuner(), INITIAL_PREFILL_CHUNK
+        if not isinstance(max_batch_tokens, int) or max_batch_tokens < 1 or (chunk is not None and chunk < 1):
+            raise ValueError("max_batch_tokens (a number or 'auto') and chunk must be at least 1")
         self.cache = cache
         self.runner = runner
         self.context_len = context_len
@@ -160,8 +204,7 @@ class ContinuousBatchScheduler:
             raise ValueError(f"the prompt has {len(prompt)} tokens, the context holds {self.context_len}")
         room = self.context_len - len(prompt)
         if params.max_new_tokens > room:
-            params = SamplingParams(params.temperature, params.top_p, params.top_k, room, params.seed,
-                                    params.ignore_eos)
+            params = dataclasses.replace(params, max_new_tokens=room)
         number = self._lib.gibbs_sched_submit(self._core, len(prompt), params.max_new_tokens, int(params.ignore_eos))
         assert number == order
         self._seqs.append(Sequence(rid, prompt, params, order))
@@ -230,6 +273,10 @@ class ContinuousBatchScheduler:
     def step(self) -> StepOutput:
         self.steps += 1
         lib, n_ev = self._lib, ctypes.byref(self._n_events)
+        if self.tuner is not None:
+            decoding = any(s.state == SequenceState.DECODING for s in self.active)
+            self.max_batch_tokens = self.tuner.budget(decoding)
+            lib.gibbs_sched_set_budget(self._core, self.max_batch_tokens)
         n_plan = lib.gibbs_sched_plan(self._core, self._plan, len(self._plan) // 5, self._events, len(self._events), n_ev)
         if n_plan < 0:
             raise RuntimeError(host.last_error())
@@ -255,6 +302,7 @@ class ContinuousBatchScheduler:
                 prefill_tokens += n
         emitted: List[Tuple[Hashable, int]] = []
         if entries:
+            started = self.clock()
             try:
                 tokens = self.runner(entries, draws)
             except Exception as exc:                                # scheduler/mod.rs:1332-1340
@@ -263,6 +311,8 @@ class ContinuousBatchScheduler:
                 waiting, active = self._counts()
                 return StepOutput(entries, [], finished, preempted, prefill_tokens, decode_tokens, active, waiting)
             assert len(tokens) == len(sampled_for)
+            if self.tuner is not None:
+                self.tuner.record(self.clock() - started, prefill_tokens, decode_tokens)
             # emit and finish
             k = len(tokens)
             numbers = (ctypes.c_int * max(1, k))(*[s.submitted for s in sampled_for])

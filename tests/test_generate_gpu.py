@@ -181,6 +181,25 @@ def test_repetition_penalty_in_generation(dirs):
     assert res[rids[2]].tokens == plain_greedy(d, prompts[2], 24)
 
 
+def test_measured_budget_changes_no_token(dirs):
+    """`max_batch_tokens="auto"` (the budget sized by measured costs) cuts the prompts elsewhere and
+    gives the same tokens; bursts of decode steps feed the measurement too."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    d = dirs["B"]
+    prompts = [H.tokens(90 + i, n, 512) for i, n in enumerate([150, 9, 77])]
+    runs = []
+    for budget in (2048, "auto"):
+        eng = Engine(d, dtype="float32", max_tokens=2048, max_requests=4)
+        gen = Generator(eng, max_batch_tokens=budget)
+        rids = [gen.submit(p, SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True)) for p in prompts]
+        res = gen.run()
+        runs.append([res[r].tokens for r in rids])
+        if budget == "auto":
+            tuner = gen.scheduler.tuner
+            assert tuner.prefill_s_per_token > 0 and tuner.decode_round_s > 0
+    assert runs[0] == runs[1]
+
+
 def test_continuous_batching_under_page_pressure(dirs):
     """A pool so small that running requests collide: the youngest is preempted and recomputed, and
     every request still gets exactly the tokens it gets alone."""

@@ -262,3 +262,56 @@ def test_random_workloads_always_finish_with_the_tokens_of_a_run_alone():
             s2, _, _ = make(pages=64, ps=16)
             r2 = s2.submit(p, greedy(m))
             assert s2.run()[r2].output_tokens == got.output_tokens, f"case {case}: request {rid}"
+
+
+def test_prefill_tuner_budgets():
+    """The reference's numbers (/root/reference/src/scheduler/mod.rs:341-403): 64 before anything is
+    timed; one token while requests decode and no decode round has been timed; then the tokens that
+    cost one decode round, or 100 ms when nothing decodes; at most 2,048; averages move by a quarter."""
+    from gibbs_amd.engine.scheduler import PrefillTuner
+    t = PrefillTuner()
+    assert t.budget(False) == 64 and t.budget(True) == 64
+    t.record(0.064, 64, 0)                                   # 1 ms a prompt token
+    assert t.budget(False) == 100 and t.budget(True) == 1
+    t.record(0.005, 0, 8)                                    # a decode round of 5 ms
+    assert t.budget(True) == 5
+    t.record(0.009, 0, 8)                                    # 0.75 * 5 + 0.25 * 9 = 6 ms
+    assert abs(t.decode_round_s - 0.006) < 1e-12 and t.budget(True) == 6
+    t.record(0.012, 6, 8)                                    # beside a decode round: 6 ms for 6 tokens
+    assert abs(t.prefill_s_per_token - 0.001) < 1e-12
+    fast = PrefillTuner()
+    fast.record(1e-6, 1000, 0)
+    assert fast.budget(False) == 2048                        # the cap
+    slow = PrefillTuner()
+    slow.record(1.0, 1, 0); slow.record(0.01, 0, 1)
+    assert slow.budget(True) == 1 and slow.budget(False) == 1   # at least one token
+
+
+def test_measured_budget_through_the_scheduler():
+    """`max_batch_tokens="auto"` with a clock that the fake model moves: a prompt token costs 1 ms, a
+    step with decoded tokens 4 ms more.  The first step takes 64 prompt tokens; with nothing decoding
+    the next ones take 100 (100 ms); beside decoding requests a step takes the 4 tokens that cost
+    one decode round."""
+    now = [0.0]
+    cache = CacheManager([CacheNeed(1, 16), None], [(), (StateNeed("s", (2,)),)], 16, 256, 8)
+    model = FakeModel(cache)
+    def runner(entries, draws):
+        decoded = sum(1 for e in entries if len(e.tokens) == 1 and e.want)
+        now[0] += 0.001 * sum(len(e.tokens) for e in entries if not (len(e.tokens) == 1 and e.want)) + (0.004 if decoded else 0)
+        return model(entries, draws)
+    s = ContinuousBatchScheduler(cache, runner, context_len=4096, max_batch_tokens="auto", clock=lambda: now[0])
+    a = s.submit([1] * 300, greedy(40))
+    sizes = []
+    while len(sizes) < 4:
+        o = s.step()
+        sizes.append(sum(len(e.tokens) for e in o.entries))
+    assert sizes == [64, 100, 100, 36], sizes               # 64 untimed, then 100 ms worth, then the rest
+    s.step()                                                 # a decodes: the first decode round is timed
+    b = s.submit([2] * 50, greedy(2))
+    o = s.step()
+    took = {e.rid: len(e.tokens) for e in o.entries}
+    assert took[a] == 1 and took[b] == 4, took               # 4 ms a decode round / 1 ms a token
+    s.run()
+    assert len(s.finished[a].output_tokens) == 40 and len(s.finished[b].output_tokens) == 2
+    with pytest.raises(ValueError):
+        ContinuousBatchScheduler(cache, runner, context_len=4096, max_batch_tokens="many")
