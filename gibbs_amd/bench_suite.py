@@ -166,6 +166,14 @@ def serve(entry: Dict, base: str) -> Dict:
     done = [results[r] for r in rids if r in results and not results[r].error]
     generated = sum(len(r.tokens) for r in done)
     st = gen.stats
+    ttft = sorted(r.ttft_s for r in done if r.ttft_s is not None) or [0.0]
+    itl = [r.itl_s for r in done if r.itl_s is not None] or [0.0]
+    latency = {"ttft_ms_p50": round(1e3 * ttft[len(ttft) // 2], 2), "ttft_ms_max": round(1e3 * ttft[-1], 2),
+               "itl_ms_mean": round(1e3 * sum(itl) / len(itl), 3)}
+    return {**_serve_row(entry, n_req, live, n_prompt, n_decode, chunk, done, wall, generated, st), **latency}
+
+
+def _serve_row(entry, n_req, live, n_prompt, n_decode, chunk, done, wall, generated, st) -> dict:
     return {"model": entry["name"], "workload": "serve", "dtype": entry["dtype"], "requests": n_req, "live": live,
             "prompt_tokens": n_prompt, "decode_tokens": n_decode, "chunk": chunk,
             "finished": len(done), "wall_ms": round(1e3 * wall, 2),

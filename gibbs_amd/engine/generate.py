@@ -27,6 +27,8 @@ class Generation:
     finish_reason: str
     error: Optional[str] = None
     preemptions: int = 0
+    ttft_s: Optional[float] = None      # submission to first token (the reference's telemetry keeps the same two
+    itl_s: Optional[float] = None       # figures, src/telemetry/mod.rs:228-447); mean time between later tokens
 
 
 @dataclass
@@ -66,6 +68,7 @@ class Generator:
         self.scheduler = ContinuousBatchScheduler(engine.cache, self._run, context_len=engine.ctx_limit,
                                                   max_batch_tokens=max_batch_tokens, chunk=chunk, eos_token_ids=eos)
         self.stats = GenerationStats()
+        self._times: Dict[Hashable, List[float]] = {}       # request -> [submitted, first token, last token, tokens]
 
     def _run(self, entries: Sequence[Entry], draws: Sequence[Draw]) -> List[int]:
         logits = self.engine.step(entries)
@@ -75,7 +78,9 @@ class Generator:
 
     def submit(self, prompt_tokens: Sequence[int], params: Optional[SamplingParams] = None,
                rid: Optional[Hashable] = None) -> Hashable:
-        return self.scheduler.submit(prompt_tokens, params, rid)
+        rid = self.scheduler.submit(prompt_tokens, params, rid)
+        self._times[rid] = [time.perf_counter(), 0.0, 0.0, 0]
+        return rid
 
     def _burst(self) -> Optional[StepOutput]:
         plan = self.scheduler.burst_plan(self.decode_burst) if self.decode_burst > 0 else None
@@ -122,7 +127,14 @@ class Generator:
             out = self.scheduler.step()
             self._stepped = True
         torch.cuda.synchronize(self.engine.device)
-        dt = time.perf_counter() - t0
+        now = time.perf_counter()
+        dt = now - t0
+        for rid, _ in out.emitted:
+            t = self._times.get(rid)
+            if t is not None:
+                if t[3] == 0:
+                    t[1] = now
+                t[2], t[3] = now, t[3] + 1
         self.stats.steps += 1
         if out.prefill_tokens:
             self.stats.prefill_tokens += out.prefill_tokens
@@ -138,9 +150,14 @@ class Generator:
         return self.results()
 
     def results(self) -> Dict[Hashable, Generation]:
-        return {rid: Generation(rid, s.prompt_tokens, list(s.output_tokens),
-                                s.finish_reason.value if s.finish_reason else "stop", s.error, s.preemptions)
-                for rid, s in self.scheduler.finished.items()}
+        out = {}
+        for rid, s in self.scheduler.finished.items():
+            t = self._times.get(rid, [0.0, 0.0, 0.0, 0])
+            out[rid] = Generation(rid, s.prompt_tokens, list(s.output_tokens),
+                                  s.finish_reason.value if s.finish_reason else "stop", s.error, s.preemptions,
+                                  ttft_s=t[1] - t[0] if t[3] else None,
+                                  itl_s=(t[2] - t[1]) / (t[3] - 1) if t[3] > 1 else None)
+        return out
 
 
 def generate(engine: Engine, prompts: Sequence[Sequence[int]], max_tokens: int = 64,

@@ -55,6 +55,7 @@ def test_greedy_generation_matches_plain(dirs, dtype):
         outs = generate(eng, prompts, max_tokens=16, temperature=0.0, ignore_eos=True)
         for p, o in zip(prompts, outs):
             assert o.finish_reason == "length" and len(o.tokens) == 16
+            assert o.ttft_s > 0 and o.itl_s > 0
             if dtype == "float32":
                 assert o.tokens == plain_greedy(dirs[name], p, 16)
             acceptable(dirs[name], p, o.tokens, dtype)
@@ -397,6 +398,7 @@ def test_bench_suite_through_the_command_line(dirs, tmp_path):
     assert [r["model"] for r in rows] == ["Tiny A", "cfg", "served"] and rows[1]["batch"] == 3
     served = rows.pop()
     assert served["finished"] == 5 and served["live"] == 3 and served["decode_tok_s"] > 0 and served["prompt_tok_s"] > 0
+    assert 0 < served["ttft_ms_p50"] <= served["ttft_ms_max"] and served["itl_ms_mean"] > 0
     for r in rows:
         assert r["decode_tok_s"] > 0 and r["prefill_tok_s"] > 0 and 0 < r["roofline_pct"] < 100
         assert abs(r["roofline_tok_s"] * r["bytes_per_token"] - r["ceiling_gbps"] * 1e9) < 1e-3 * r["ceiling_gbps"] * 1e9
