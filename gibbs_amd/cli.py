@@ -52,11 +52,8 @@ def parser() -> argparse.ArgumentParser:
 
 
 def _tokenizer(model_dir: str):
-    path = os.path.join(model_dir, "tokenizer.json")
-    if not os.path.isfile(path):
-        return None
-    from tokenizers import Tokenizer
-    return Tokenizer.from_file(path)
+    from .text import open_text
+    return open_text(model_dir)
 
 
 def _parity(make_engine, prompt: List[int], steps: int = 8) -> int:
@@ -157,13 +154,15 @@ def main(argv: Optional[List[str]] = None) -> int:
         if tok is None:
             print("gibbs: --prompt needs tokenizer.json in the model folder; use --prompt-ids", file=sys.stderr)
             return 2
-        prompt = tok.encode(args.prompt).ids
+        prompt = tok.prompt_ids(args.prompt)      # through the folder's chat template when it declares one
     else:
         print("gibbs: give --prompt or --prompt-ids", file=sys.stderr)
         return 2
     print(f"💬 Generating from prompt: {args.prompt if args.prompt is not None else prompt!r}")
-    temperature = 0.7 if args.temperature is None else args.temperature       # main.rs:744-749
-    gen = Generator(engine, max_batch_tokens=args.max_batch_tokens, chunk=args.chunk)
+    declared_greedy = tok is not None and tok.sampling_defaults is not None and tok.sampling_defaults[0] <= 1e-4
+    temperature = (0.0 if declared_greedy else 0.7) if args.temperature is None else args.temperature   # main.rs:744-749
+    gen = Generator(engine, max_batch_tokens=args.max_batch_tokens, chunk=args.chunk,
+                    eos_token_ids=tuple(set(engine.spec.eos_token_ids) | set(tok.stop_ids)) if tok is not None else None)
     rid = gen.submit(prompt, SamplingParams(temperature, args.top_p, args.top_k, max_tokens, args.seed,
                                             args.ignore_eos or tok is None, args.repetition_penalty))
     result = gen.run()[rid]

@@ -353,6 +353,18 @@ def test_command_line(dirs, tmp_path):
     want = H.plain_logits(dirs["A"], [1, 2, 3])[-1]
     assert [t["id"] for t in top] == np.argsort(-want)[:5].tolist()
     assert run("--model", dirs["A"], "--prompt-ids", "1", "--backend", "cpu").returncode == 2
+    # a text prompt: through the folder's tokenizer and chat template, decoded on the way out
+    import pathlib
+    import shutil
+    from tests.test_text import TEMPLATE, write_folder
+    texted = pathlib.Path(shutil.copytree(dirs["A"], tmp_path / "texted"))
+    write_folder(texted, template=TEMPLATE, generation={"do_sample": False}, write_config=False)
+    p = run("--model", str(texted), "--prompt", "hello world", "--max-tokens", "5", "--ignore-eos", "--dtype", "float32")
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert "⚡ Prefill: 5 tokens" in p.stdout, "BOS, the user marker, two words and the assistant marker"
+    want = plain_greedy(dirs["A"], [1, 3, 5, 6, 4], 5)        # the folder declares greedy decoding
+    from gibbs_amd.text import open_text
+    assert p.stdout.split("✨ Output:\n")[1].splitlines()[0] == open_text(str(texted)).decode(want)
     cfgfile = tmp_path / "cfg.json"
     cfgfile.write_text(json.dumps(H.TINY["C"]))
     p = run("--model", str(tmp_path / "fresh"), "--random-weights", str(cfgfile), "--seed", "5", "--prompt-ids", "3,4",
