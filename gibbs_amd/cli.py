@@ -31,7 +31,7 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--replay", metavar="TRACE",
                     help="replay a trace (JSON lines as for bin/trace_run; '-' is standard input) and write logits to --out")
     ap.add_argument("--out", help="folder for the logits of --replay")
-    ap.add_argument("--probe-top5", help="print the top-5 next-token logits (JSON) for these comma-separated ids")
+    ap.add_argument("--probe-top5", help="print the top-5 next-token logits (JSON) for these comma-separated ids (or a text prompt)")
     ap.add_argument("--temperature", type=float, default=None, help="sampling temperature (one-shot default 0.7; <= 1e-4 is greedy)")
     ap.add_argument("--top-p", type=float, default=None, help="nucleus cut (default 0.9)")
     ap.add_argument("--top-k", type=int, default=50, help="candidates (default 50, at most 64)")
@@ -141,7 +141,14 @@ def main(argv: Optional[List[str]] = None) -> int:
         replay(engine, lines, args.out)
         return 0
     if args.probe_top5:
-        ids = _ids(args.probe_top5)
+        try:
+            ids = _ids(args.probe_top5)
+        except ValueError:                       # a text prompt, as the reference's probe takes (bench.rs:888-911)
+            tok = _tokenizer(args.model)
+            if tok is None:
+                print("gibbs: --probe-top5 takes token ids, or text when the model folder has tokenizer.json", file=sys.stderr)
+                return 2
+            ids = tok.prompt_ids(args.probe_top5)
         logits = engine.step([("probe", ids, [len(ids) - 1])])[0]
         top = logits.topk(5)
         print(json.dumps([{"id": int(i), "logit": float(v)} for v, i in zip(top.values.tolist(), top.indices.tolist())]))
