@@ -246,7 +246,13 @@ def test_random_workloads_always_finish_with_the_tokens_of_a_run_alone():
         reqs = rng.randint(1, 5)
         budget = rng.choice([1, 2, 3, 8, 64])
         chunk = rng.choice([None, 1, 5, 16])
-        s, model, cache = make(pages=pages, reqs=reqs, ps=ps, budget=budget, chunk=chunk)
+        if case % 2:
+            s, model, cache = make(pages=pages, reqs=reqs, ps=ps, budget=budget, chunk=chunk)
+        else:                                    # a second cache group that keeps a window of its keys
+            cache = CacheManager([CacheNeed(1, 16), CacheNeed(2, 16, window=rng.choice([1, 3, 8, 20, 50])), None],
+                                 [(), (), (StateNeed("s", (2,)),)], ps, pages, reqs)
+            model = FakeModel(cache)
+            s = ContinuousBatchScheduler(cache, model, context_len=4096, max_batch_tokens=budget, chunk=chunk)
         prompts = [[rng.randint(0, 99) for _ in range(a)] for a in lens]
         rids = [s.submit(p, greedy(m)) for p, m in zip(prompts, news)]
         steps, bound = 0, 50 * (sum(lens) + sum(news)) + 100
@@ -255,7 +261,7 @@ def test_random_workloads_always_finish_with_the_tokens_of_a_run_alone():
             steps += 1
             assert steps < bound, f"case {case}: no end after {steps} steps"
         cache.check()
-        assert cache.free_pages() == pages and cache.free_slots() == reqs, f"case {case}"
+        assert all(cache.free_pages(g) == pages for g in range(cache.n_groups)) and cache.free_slots() == reqs, f"case {case}"
         for rid, p, m in zip(rids, prompts, news):
             got = s.finished[rid]
             assert got.error is None and len(got.output_tokens) == m, f"case {case}: request {rid}: {got.error}"
