@@ -7,7 +7,7 @@
 // staged through LDS (rows padded by 16 bytes against bank conflicts), double-buffered so that
 // the next tile's global loads are in flight while the matrix cores work on the current one.
 // Rows beyond N or O and k beyond I are read as zero.  I and the row strides must be multiples
-// of 8 elements (16-byte loads).
+// of 8 elements (16-byte loads).  Large aligned shapes take a 256 x 256 kernel (below).
 #include "common.h"
 
 namespace {
@@ -99,6 +99,123 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__
 }
 #undef LOAD_GLOBAL
 #undef STORE_LDS
+
+// The same product for large aligned shapes (N and O multiples of 256, I of 64): a workgroup of 4 waves
+// computes 256 x 256, each wave 128 x 128 as 4 x 4 MFMA tiles (the accumulators fill the 256 AGPRs, so
+// one wave per SIMD), and asks LDS for half as many operand bytes per product as the 128 x 128 kernel.
+// Tiles of 64 k travel global -> LDS without passing through registers (global_load_lds, 16 bytes a
+// lane, a wave's instruction covers 8 whole rows of 128 bytes), two stages.  A tile in LDS is
+// [256 rows][64 k] with the 16-byte chunk c of row r at position c ^ ((r >> 1) & 7): the lane that
+// fills slot (r, p) loads chunk p ^ ((r >> 1) & 7) from memory, and the operand reads (ds_read_b128,
+// 32 rows x one chunk per instruction) are free of bank conflicts (measured: none).  The product is
+// computed transposed (features x tokens), so a lane's results are 4 consecutive features of one row.
+// Workgroups are numbered so that the 32 that an XCD runs at a time share 8 tiles of W and 4 of A.
+constexpr int TM = 256, TN = 256, TK = 64;
+__device__ __forceinline__ int swizzled(int row, int chunk) { return row * TK + ((chunk ^ ((row >> 1) & 7)) << 3); }
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_bf16_256_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                            OutT* __restrict__ C, int I, long lda, long ldw, long ldc,
+                                                            int tiles_n, int tiles_o) {
+  extern __shared__ __attribute__((aligned(16))) bf16 lds_tiles[];
+  bf16* sA = lds_tiles;                  // [2][TM * TK]
+  bf16* sB = lds_tiles + 2 * TM * TK;    // [2][TN * TK]
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int total = tiles_n * tiles_o;
+  int tn, to;
+  if (total % 8 == 0 && (total / 8) % tiles_n == 0) {
+    // workgroup b runs on XCD b % 8: each XCD takes a contiguous range of W tiles, W varying fastest
+    const int b = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
+    const int per = total / 8, i = b % per, x = b / per, wt = per / tiles_n;
+    to = x * wt + i % wt;
+    tn = i / wt;
+  } else {
+    tn = blockIdx.x % tiles_n;
+    to = blockIdx.x / tiles_n;
+  }
+  const int row0 = tn * TM, col0 = to * TN;
+  const int wm = wave / 2, wn = wave % 2;
+  const int lp = tid % 8, lr = tid / 8;
+  auto load_tile = [&](int k0, int buf) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int r = lr + 32 * i;
+      const int c = lp ^ ((r >> 1) & 7);
+      const bf16* ga = A + (size_t)(row0 + r) * lda + k0 + c * 8;
+      const bf16* gb = W + (size_t)(col0 + r) * ldw + k0 + c * 8;
+      bf16* la = sA + buf * TM * TK + (wave * 64 + i * 256) * 8;    // the same for the whole wave; lane l fills slot l after it
+      bf16* lb = sB + buf * TN * TK + (wave * 64 + i * 256) * 8;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ga,
+                                       (__attribute__((address_space(3))) void*)la, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gb,
+                                       (__attribute__((address_space(3))) void*)lb, 16, 0, 0);
+    }
+  };
+  floatx16 acc[4][4];   // [feature tile][token tile]
+#pragma unroll
+  for (int n = 0; n < 4; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[n][m][i] = 0.f;
+
+  const int nt = I / TK;
+  load_tile(0, 0);
+  __builtin_amdgcn_s_waitcnt(0);
+  __syncthreads();
+  const int r32 = lane % 32, h = lane / 32;
+  for (int t = 0; t < nt; ++t) {
+    const bf16* cA = sA + (t & 1) * TM * TK;
+    const bf16* cB = sB + (t & 1) * TN * TK;
+    if (t + 1 < nt) load_tile((t + 1) * TK, (t + 1) & 1);
+#pragma unroll
+    for (int kk = 0; kk < TK / 16; ++kk) {
+      bf16x8 fa[4], fb[4];
+      const int chunk = kk * 2 + h;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) fa[m] = *(const bf16x8*)(cA + swizzled(wm * 128 + m * 32 + r32, chunk));
+#pragma unroll
+      for (int n = 0; n < 4; ++n) fb[n] = *(const bf16x8*)(cB + swizzled(wn * 128 + n * 32 + r32, chunk));
+#pragma unroll
+      for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          acc[n][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[n], fa[m], acc[n][m], 0, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // the next tile has landed (this thread's part; the barrier covers the others')
+    __syncthreads();
+  }
+  // D[feature i][token j]: lane holds token j = lane % 32 and features (v / 4) * 8 + (lane / 32) * 4 + v % 4
+#pragma unroll
+  for (int n = 0; n < 4; ++n)
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      OutT* out = C + (size_t)(row0 + wm * 128 + m * 32 + r32) * ldc + col0 + wn * 128 + n * 32 + h * 4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[q * 8 + e] = from_float<OutT>(acc[n][m][q * 4 + e]);
+    }
+}
+
+template <typename OutT>
+int launch_256(const bf16* A, const bf16* W, OutT* C, int N, int O, int I, long lda, long ldw, long ldc, hipStream_t stream) {
+  constexpr int LDS_BYTES = 2 * (TM + TN) * TK * (int)sizeof(bf16);
+  static bool prepared = false;    // (per output type: the template makes one flag each)
+  if (!prepared) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_256_kernel<OutT>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (e != hipSuccess) return gibbs_fail("gemm_bf16: %s", hipGetErrorString(e));
+    prepared = true;
+  }
+  const int tiles_n = N / TM, tiles_o = O / TN;
+  gemm_bf16_256_kernel<OutT><<<tiles_n * tiles_o, 256, LDS_BYTES, stream>>>(A, W, C, I, lda, ldw, ldc, tiles_n, tiles_o);
+  GIBBS_LAUNCH_STATUS("gemm_bf16");
+}
+
+// Large aligned shapes that fill the chip with 256 x 256 tiles take the kernel above.
+bool takes_256(int N, int O, int I, long ldc) {
+  return N % TM == 0 && O % TN == 0 && I % TK == 0 && ldc % 4 == 0 && (long)(N / TM) * (O / TN) >= 192;
+}
 }  // namespace
 
 // A: [N, I] bfloat16, W: [O, I] bfloat16, C: [N, O] bfloat16 (out_dtype 1) or float32 (0).
@@ -109,6 +226,10 @@ GIBBS_EXPORT int gibbs_gemm_bf16(const void* A, const void* W, void* C, int out_
   GIBBS_REQUIRE(((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0, "gemm_bf16: operands must be 16-byte aligned");
   GIBBS_REQUIRE(lda >= I && ldw >= I && ldc >= O, "gemm_bf16: row strides shorter than rows");
   if (N == 0) return 0;
+  if (takes_256(N, O, I, ldc)) {
+    if (out_dtype == GIBBS_BF16) return launch_256((const bf16*)A, (const bf16*)W, (bf16*)C, N, O, I, lda, ldw, ldc, stream);
+    if (out_dtype == GIBBS_F32) return launch_256((const bf16*)A, (const bf16*)W, (float*)C, N, O, I, lda, ldw, ldc, stream);
+  }
   dim3 grid(ceil_div(O, BN), ceil_div(N, BM));
   GIBBS_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", N);
   if (out_dtype == GIBBS_BF16)

@@ -75,7 +75,8 @@ def test_gemm_f32(shape):
 
 
 @pytest.mark.parametrize("out_dtype", DT)
-@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 331, 112), (130, 200, 72), (257, 129, 1000), (300, 512, 2048)])
+@pytest.mark.parametrize("shape", [(1, 64, 32), (5, 331, 112), (130, 200, 72), (257, 129, 1000), (300, 512, 2048),
+                                   (2048, 6144, 192), (1024, 12288, 64), (768, 16384, 320)])   # the 256 x 256 kernel: both tile orders
 def test_gemm_bf16(shape, out_dtype):
     from gibbs_amd import ops
     n, o, i = shape
