@@ -100,26 +100,30 @@ __global__ __launch_bounds__(256) void gemm_bf16_kernel(const bf16* __restrict__
 #undef LOAD_GLOBAL
 #undef STORE_LDS
 
-// The same product for large aligned shapes (N and O multiples of 256, I of 64): a workgroup of 4 waves
-// computes 256 x 256, each wave 128 x 128 as 4 x 4 MFMA tiles (the accumulators fill the 256 AGPRs, so
-// one wave per SIMD), and asks LDS for half as many operand bytes per product as the 128 x 128 kernel.
-// Tiles of 64 k travel global -> LDS without passing through registers (global_load_lds, 16 bytes a
-// lane, a wave's instruction covers 8 whole rows of 128 bytes), two stages.  A tile in LDS is
-// [256 rows][64 k] with the 16-byte chunk c of row r at position c ^ ((r >> 1) & 7): the lane that
-// fills slot (r, p) loads chunk p ^ ((r >> 1) & 7) from memory, and the operand reads (ds_read_b128,
-// 32 rows x one chunk per instruction) are free of bank conflicts (measured: none).  The product is
-// computed transposed (features x tokens), so a lane's results are 4 consecutive features of one row.
-// Workgroups are numbered so that the 32 that an XCD runs at a time share 8 tiles of W and 4 of A.
-constexpr int TM = 256, TN = 256, TK = 64;
+// The same product for large aligned shapes (N and O multiples of 256, I of 64): a workgroup of 8 waves
+// computes 256 x 256, each wave 128 tokens x 64 features as 4 x 2 MFMA tiles (two waves per SIMD), and
+// asks LDS for fewer operand bytes per product than the 128 x 128 kernel.  Tiles of 64 k travel
+// global -> LDS without passing through registers (global_load_lds, 16 bytes a lane; a wave's
+// instruction covers 8 whole rows of 128 bytes).  LDS holds three tiles of A and two of W (160 KB): W
+// is asked for one tile ahead and A two, so that loads stay in flight across the tile's barrier.  The
+// loads are issued one after every four products: issued together they block the wave for as long as
+// the memory pipe takes to accept them (measured: 1,500 cycles a tile with idle matrix cores).  A tile
+// in LDS is [256 rows][64 k] with the 16-byte chunk c of row r at position c ^ ((r >> 1) & 7): the lane
+// that fills slot (r, p) loads chunk p ^ ((r >> 1) & 7) from memory, and the operand reads
+// (ds_read_b128, 32 rows x one chunk per instruction) are free of bank conflicts (measured: none).
+// The product is computed transposed (features x tokens), so a lane's results are 4 consecutive
+// features of one row.  Workgroups are numbered so that the 32 that an XCD runs at a time share 8
+// tiles of W and 4 of A.
+constexpr int TM = 256, TN = 256, TK = 64, TILE_ELEMS = 256 * TK;
 __device__ __forceinline__ int swizzled(int row, int chunk) { return row * TK + ((chunk ^ ((row >> 1) & 7)) << 3); }
 
 template <typename OutT>
-__global__ __launch_bounds__(256) void gemm_bf16_256_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+__global__ __launch_bounds__(512) void gemm_bf16_256_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                             OutT* __restrict__ C, int I, long lda, long ldw, long ldc,
                                                             int tiles_n, int tiles_o) {
   extern __shared__ __attribute__((aligned(16))) bf16 lds_tiles[];
-  bf16* sA = lds_tiles;                  // [2][TM * TK]
-  bf16* sB = lds_tiles + 2 * TM * TK;    // [2][TN * TK]
+  bf16* sA = lds_tiles;                     // [3][TILE_ELEMS]
+  bf16* sB = lds_tiles + 3 * TILE_ELEMS;    // [2][TILE_ELEMS]
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int total = tiles_n * tiles_o;
   int tn, to;
@@ -134,63 +138,71 @@ __global__ __launch_bounds__(256) void gemm_bf16_256_kernel(const bf16* __restri
     to = blockIdx.x / tiles_n;
   }
   const int row0 = tn * TM, col0 = to * TN;
-  const int wm = wave / 2, wn = wave % 2;
+  const int wm = wave / 4, wn = wave % 4;
   const int lp = tid % 8, lr = tid / 8;
-  auto load_tile = [&](int k0, int buf) {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = lr + 32 * i;
-      const int c = lp ^ ((r >> 1) & 7);
-      const bf16* ga = A + (size_t)(row0 + r) * lda + k0 + c * 8;
-      const bf16* gb = W + (size_t)(col0 + r) * ldw + k0 + c * 8;
-      bf16* la = sA + buf * TM * TK + (wave * 64 + i * 256) * 8;    // the same for the whole wave; lane l fills slot l after it
-      bf16* lb = sB + buf * TN * TK + (wave * 64 + i * 256) * 8;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)ga,
-                                       (__attribute__((address_space(3))) void*)la, 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)gb,
-                                       (__attribute__((address_space(3))) void*)lb, 16, 0, 0);
-    }
+  // instruction i (0..3) of a tile's loads: this thread fills slot (row lr + 64 i, position lp)
+  auto load_one = [&](const bf16* G, long ld, int g0, int k0, bf16* dst, int i) {
+    const int r = lr + 64 * i;
+    const int c = lp ^ ((r >> 1) & 7);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(G + (size_t)(g0 + r) * ld + k0 + c * 8),
+                                     (__attribute__((address_space(3))) void*)(dst + (wave * 64 + i * 512) * 8), 16, 0, 0);
   };
-  floatx16 acc[4][4];   // [feature tile][token tile]
+  floatx16 acc[2][4];   // [feature tile][token tile]
 #pragma unroll
-  for (int n = 0; n < 4; ++n)
+  for (int n = 0; n < 2; ++n)
 #pragma unroll
     for (int m = 0; m < 4; ++m)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[n][m][i] = 0.f;
 
   const int nt = I / TK;
-  load_tile(0, 0);
-  __builtin_amdgcn_s_waitcnt(0);
-  __syncthreads();
+  // A(0), W(0), A(1) before the loop (a tile beyond the last is the last once more: harmless, and the
+  // count of loads in flight stays the same in every iteration)
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_one(A, lda, row0, 0, sA, i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_one(W, ldw, col0, 0, sB, i);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) load_one(A, lda, row0, min(1, nt - 1) * TK, sA + TILE_ELEMS, i);
   const int r32 = lane % 32, h = lane / 32;
   for (int t = 0; t < nt; ++t) {
-    const bf16* cA = sA + (t & 1) * TM * TK;
-    const bf16* cB = sB + (t & 1) * TN * TK;
-    if (t + 1 < nt) load_tile((t + 1) * TK, (t + 1) & 1);
+    // A(t) and W(t) have landed (this thread's part; the barrier covers the others'); the four loads of
+    // A(t+1) may still be on their way
+    asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    __syncthreads();
+    const int kb = min(t + 1, nt - 1) * TK, ka = min(t + 2, nt - 1) * TK;
+    bf16* dB = sB + ((t + 1) & 1) * TILE_ELEMS;
+    bf16* dA = sA + ((t + 2) % 3) * TILE_ELEMS;
+    const bf16* cA = sA + (t % 3) * TILE_ELEMS;
+    const bf16* cB = sB + (t & 1) * TILE_ELEMS;
 #pragma unroll
     for (int kk = 0; kk < TK / 16; ++kk) {
-      bf16x8 fa[4], fb[4];
+      bf16x8 fa[4], fb[2];
       const int chunk = kk * 2 + h;
 #pragma unroll
       for (int m = 0; m < 4; ++m) fa[m] = *(const bf16x8*)(cA + swizzled(wm * 128 + m * 32 + r32, chunk));
 #pragma unroll
-      for (int n = 0; n < 4; ++n) fb[n] = *(const bf16x8*)(cB + swizzled(wn * 128 + n * 32 + r32, chunk));
+      for (int n = 0; n < 2; ++n) fb[n] = *(const bf16x8*)(cB + swizzled(wn * 64 + n * 32 + r32, chunk));
 #pragma unroll
-      for (int n = 0; n < 4; ++n)
+      for (int n = 0; n < 2; ++n) {
 #pragma unroll
         for (int m = 0; m < 4; ++m)
           acc[n][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[n], fa[m], acc[n][m], 0, 0, 0);
+        // one load of the tiles to come after every four products: W(t+1) first (it has to be through at
+        // the next barrier), then A(t+2)
+        const int j = kk * 2 + n;
+        if (j < 4) load_one(W, ldw, col0, kb, dB, j);
+        else load_one(A, lda, row0, ka, dA, j - 4);
+      }
     }
-    __builtin_amdgcn_s_waitcnt(0);   // the next tile has landed (this thread's part; the barrier covers the others')
-    __syncthreads();
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be writing LDS when the workgroup ends
   // D[feature i][token j]: lane holds token j = lane % 32 and features (v / 4) * 8 + (lane / 32) * 4 + v % 4
 #pragma unroll
-  for (int n = 0; n < 4; ++n)
+  for (int n = 0; n < 2; ++n)
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
-      OutT* out = C + (size_t)(row0 + wm * 128 + m * 32 + r32) * ldc + col0 + wn * 128 + n * 32 + h * 4;
+      OutT* out = C + (size_t)(row0 + wm * 128 + m * 32 + r32) * ldc + col0 + wn * 64 + n * 32 + h * 4;
 #pragma unroll
       for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -200,7 +212,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_256_kernel(const bf16* __restri
 
 template <typename OutT>
 int launch_256(const bf16* A, const bf16* W, OutT* C, int N, int O, int I, long lda, long ldw, long ldc, hipStream_t stream) {
-  constexpr int LDS_BYTES = 2 * (TM + TN) * TK * (int)sizeof(bf16);
+  constexpr int LDS_BYTES = 5 * TILE_ELEMS * (int)sizeof(bf16);   // three tiles of A, two of W
   static bool prepared = false;    // (per output type: the template makes one flag each)
   if (!prepared) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_bf16_256_kernel<OutT>, hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
@@ -208,7 +220,7 @@ int launch_256(const bf16* A, const bf16* W, OutT* C, int N, int O, int I, long 
     prepared = true;
   }
   const int tiles_n = N / TM, tiles_o = O / TN;
-  gemm_bf16_256_kernel<OutT><<<tiles_n * tiles_o, 256, LDS_BYTES, stream>>>(A, W, C, I, lda, ldw, ldc, tiles_n, tiles_o);
+  gemm_bf16_256_kernel<OutT><<<tiles_n * tiles_o, 512, LDS_BYTES, stream>>>(A, W, C, I, lda, ldw, ldc, tiles_n, tiles_o);
   GIBBS_LAUNCH_STATUS("gemm_bf16");
 }
 
