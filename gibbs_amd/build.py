@@ -121,8 +121,11 @@ def build(verbose: bool = True) -> str:
             if verbose:
                 _say(f"  [{done}/{len(srcs)}] {name} ({secs:.1f}s)")
     tmp_lib = os.path.join(lib_dir, f".{LIB_NAME}.{os.getpid()}")
-    proc = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp_lib],
-                          capture_output=True, text=True, env=env)
+    # the library product (hipBLASLt) comes from the ROCm installation that hipcc belongs to; a process
+    # that has loaded another copy of the same soname first (PyTorch brings one) keeps using that one
+    rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(cc))), "lib")
+    proc = subprocess.run([cc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, f"-L{rocm_lib}", "-lhipblaslt",
+                           f"-Wl,-rpath,{rocm_lib}", "-o", tmp_lib], capture_output=True, text=True, env=env)
     if proc.returncode != 0:
         raise BuildError(f"linking the HIP extension failed:\n{proc.stderr[-4000:]}")
     os.replace(tmp_lib, os.path.join(lib_dir, LIB_NAME))

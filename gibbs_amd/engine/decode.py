@@ -32,8 +32,8 @@ def capture(graph: "torch.cuda.CUDAGraph"):
     """Captures into `graph` with Python's cycle collector switched off.  The collector may run at
     any allocation; if it then destroys the graphs of a loop that was dropped earlier (a loop, its
     engine and its batch hold each other), a capturing stream refuses the call and the error, raised
-    from a destructor, ends the process.  What can be collected is collected before the capture."""
-    gc.collect()
+    from a destructor, ends the process.  Such garbage waits for the next collection outside a capture
+    (collecting it here first would cost tens of milliseconds per capture on a large heap)."""
     was_enabled = gc.isenabled()
     gc.disable()
     try:

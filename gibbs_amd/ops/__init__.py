@@ -135,6 +135,30 @@ def gemm_bf16(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.b
     return out
 
 
+_library_ready = False
+
+
+def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[n, o] = sum_k a[n, k] * w[o, k] by the library (hipBLASLt called directly, its choice of
+    algorithm kept per shape): bfloat16 operands and output, float32 accumulation."""
+    global _library_ready
+    require_cuda(a, w)
+    assert a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+    assert a.dim() == 2 and w.dim() == 2 and a.shape[1] == w.shape[1], (a.shape, w.shape)
+    assert a.stride(1) == 1 and w.stride(1) == 1
+    n, i = a.shape
+    o = w.shape[0]
+    if out is None:
+        out = torch.empty((n, o), dtype=torch.bfloat16, device=a.device)
+    assert out.shape == (n, o) and out.dtype == torch.bfloat16 and out.stride(1) == 1
+    if not _library_ready:
+        call("gibbs_gemm_library_init")
+        _library_ready = True
+    call("gibbs_gemm_library", ptr(a), ptr(w), ptr(out), n, o, i, a.stride(0) if n > 1 else i, w.stride(0),
+         out.stride(0) if n > 1 else o, stream())
+    return out
+
+
 class PackedWeight:
     """A matrix [groups * rows, inner] (bfloat16) in the order the few-row products read it:
     [group][ceil(rows/16)][ceil(inner/32)][64 lanes][8], lane (r, g) of a tile holding

@@ -60,6 +60,8 @@ _SIGNATURES = {
                                c_int, c_int, c_int, c_void_p],
     "gibbs_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_void_p],
+    "gibbs_gemm_library_init": [],
+    "gibbs_gemm_library": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
     "gibbs_repetition_penalty": [c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     "gibbs_sample": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],

@@ -3,8 +3,9 @@
 float32: the hand-written plain-FMA kernel (a true 32-bit product whose per-row result does not
 depend on the batch).  bfloat16, float32 accumulation throughout: up to 64 rows take the
 hand-written kernel that streams W once (decode); more rows take a matrix product on the matrix
-cores, by default the library's (hipBLASLt through `torch.matmul`, as the reference's engine
-uses a library product for its prefill), or the hand-written tiled kernel (`GIBBS_GEMM=own`),
+cores, by default the library's (hipBLASLt, called directly; `GIBBS_GEMM=torch`: through
+`torch.matmul`; the reference's engine uses a library product for its prefill as well), or the
+hand-written tiled kernel (`GIBBS_GEMM=own`),
 which also serves what the library does not give: float32 output (logits of many rows).
 """
 from __future__ import annotations
@@ -14,13 +15,16 @@ from typing import Optional
 
 import torch
 
-from . import PackedWeight, gemm_bf16, gemm_bf16_plain, gemm_f32, gemm_skinny, skinny_splits
+from . import PackedWeight, gemm_bf16, gemm_bf16_plain, gemm_f32, gemm_library, gemm_skinny, skinny_splits
 from .lib import KernelError, require_cuda
 
 # rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
 # output features, which stops paying beyond one or two MFMA tiles of rows)
 SKINNY_ROWS = int(os.environ.get("GIBBS_SKINNY_ROWS", "32"))
 USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
+# the library product is hipBLASLt called directly (its heuristic's choice kept per shape: a call costs
+# the host a fifth of what the same product costs through torch.matmul); "torch" goes through PyTorch
+LIBRARY_THROUGH_TORCH = os.environ.get("GIBBS_GEMM", "library") == "torch"
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = None,
@@ -45,6 +49,6 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
             splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
             return gemm_skinny(x, w if packed is None else packed, out_dtype, splits)
         if USE_LIBRARY_GEMM and out_dtype == torch.bfloat16:
-            return torch.matmul(x, w.t())
+            return torch.matmul(x, w.t()) if LIBRARY_THROUGH_TORCH else gemm_library(x, w)
         return gemm_bf16(x, w, out_dtype)
     raise KernelError(f"linear: unsupported dtype {x.dtype}")

@@ -91,6 +91,24 @@ def test_gemm_bf16(shape, out_dtype):
     close(ops.gemm_bf16(big[:, :i], w, out_dtype), big[:, :i].double() @ w.double().t(), out_dtype, "strided", f32=2e-5, bf16=4e-3)
 
 
+@pytest.mark.parametrize("shape", [(65, 64, 32), (130, 200, 72), (257, 129, 1000), (512, 6144, 2048), (2048, 2048, 512)])
+def test_gemm_library(shape):
+    """The library's product called directly (descriptors and algorithm kept per shape), also on a
+    view with a row stride and into a strided output, and twice (the second call takes the kept plan)."""
+    from gibbs_amd import ops
+    n, o, i = shape
+    a, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
+    want = a.double() @ w.double().t()
+    for _ in range(2):
+        close(ops.gemm_library(a, w), want, torch.bfloat16, f"gemm_library {shape}", bf16=4e-3)
+    big = rnd(n, i + 64, dtype=torch.bfloat16, seed=3)
+    close(ops.gemm_library(big[:, :i], w), big[:, :i].double() @ w.double().t(), torch.bfloat16, "strided input", bf16=4e-3)
+    wide = torch.zeros(n, o + 16, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_library(a, w, out=wide[:, :o])
+    close(wide[:, :o], want, torch.bfloat16, "strided output", bf16=4e-3)
+    assert float(wide[:, o:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("out_dtype", DT)
 @pytest.mark.parametrize("n,o,i,splits", [(1, 64, 128, 1), (8, 331, 1000, 1), (16, 2048, 2048, 2), (17, 200, 8192, 8),
                                           (33, 48, 72, 1), (64, 515, 1024, 1), (5, 2048, 8192, 4), (64, 96, 4096, 3),
