@@ -23,7 +23,7 @@ from .lib import KernelError, require_cuda
 SKINNY_ROWS = int(os.environ.get("GIBBS_SKINNY_ROWS", "32"))
 USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 # the library product is hipBLASLt called directly (its heuristic's choice kept per shape: a call costs
-# the host a fifth of what the same product costs through torch.matmul); "torch" goes through PyTorch
+# the host 12 us instead of the 20 us of torch.matmul); "torch" goes through PyTorch
 LIBRARY_THROUGH_TORCH = os.environ.get("GIBBS_GEMM", "library") == "torch"
 
 
