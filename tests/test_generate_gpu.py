@@ -303,6 +303,33 @@ def test_dropped_loops_are_collected_before_a_capture(dirs):
     assert new.tokens() == want and gc.isenabled()
 
 
+def test_decode_loop_of_more_requests_than_the_fused_path_takes(tmp_path_factory):
+    """72 requests decode together: more rows than the fused decode kernels take, so the captured step
+    holds the general path with the library's matrix products.  Replays (of one step and of eight),
+    with eager work and synchronisations between them, give what eager steps give."""
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.engine.decode import DecodeLoop
+    d = H.make_model_dir(str(tmp_path_factory.mktemp("medium")), "M", seed=5, std=0.05)
+    n = 72
+    prompts = [H.tokens(300 + i, 6 + i % 5, 4096) for i in range(n)]
+    def prefill(eng):
+        return [int(eng.step([Entry(i, p, [len(p) - 1])]).argmax(-1).item()) for i, p in enumerate(prompts)]
+    eng = Engine(d, dtype="bfloat16", max_tokens=(n + 1) * 64, max_requests=n + 1)
+    last, want = prefill(eng), [[] for _ in prompts]
+    for _ in range(20):
+        last = eng.step([Entry(i, [last[i]], [0]) for i in range(n)]).argmax(-1).tolist()
+        for i in range(n):
+            want[i].append(last[i])
+    eng = Engine(d, dtype="bfloat16", max_tokens=(n + 1) * 64, max_requests=n + 1)
+    loop = DecodeLoop(eng, list(range(n)), prefill(eng))
+    for k in (1, 3, 9, 7):
+        loop.run(k)
+        torch.cuda.synchronize()
+        eng.step([Entry("other", H.tokens(1, 11, 4096), [10])])
+        eng.release("other")
+    assert loop.tokens() == want
+
+
 def trace_lines(steps):
     return "".join(json.dumps({"step": i, "entries": [{"id": r, "tokens": t, "want": w} for r, t, w in e], "end": end}) + "\n"
                    for i, (e, end) in enumerate(steps))
