@@ -174,6 +174,100 @@ def test_glu_part(name, dtype):
         build_feed_forward(FeedForwardSpec("experts", {}, {}), 8)
 
 
+def run_block(block, xs, chunks, dtype, page_size=8):
+    """Feeds residual rows xs (one [T_r, hidden] array per request) through a bound block in the given
+    chunks per step; returns the stream after the block (x with whatever was left pending added)."""
+    from gibbs_amd.cache import CacheManager, DeviceCache
+    from gibbs_amd.engine.batch import BatchStager
+    from gibbs_amd.parts.base import Stream
+    cm = CacheManager([block.mixer.cache_need()], [tuple(block.mixer.state_needs())], page_size, 64, 4)
+    dc = DeviceCache(cm, dtype, torch.device(DEV))
+    view = dc.layer_view(0)
+    stager = BatchStager(torch.device(DEV))
+    outs = {r: [] for r in range(len(xs))}
+    fused_steps = 0
+    for step in chunks:
+        rids = [r for r, _, _ in step]
+        for r, a, b in step:
+            if r not in cm:
+                assert cm.admit(r)
+            assert cm.reserve(r, b - a)
+        dc.clear_fresh_slots()
+        q = np.array([b - a for _, a, b in step], dtype=np.int32)
+        cu = np.concatenate([[0], np.cumsum(q)]).astype(np.int32)
+        ctx = np.array([cm.tokens(r) for r in rids], dtype=np.int32)
+        row_req = np.repeat(np.arange(len(step), dtype=np.int32), q)
+        pos = (np.arange(cu[-1], dtype=np.int32) - cu[:-1][row_req] + ctx[row_req]).astype(np.int32)
+        batch = stager.stage(np.zeros(cu[-1], np.int32), pos, row_req, cu, ctx,
+                             np.array([cm.slot(r) for r in rids], np.int32), np.zeros(0, np.int32),
+                             [cm.block_table(rids, g) for g in range(cm.n_groups)])
+        x = torch.tensor(np.concatenate([xs[r][a:b] for r, a, b in step]), dtype=torch.float32, device=DEV).contiguous()
+        out = block.forward(Stream(x=x), batch, view)
+        fused_steps += out.pending is None
+        y = out.x.clone()
+        if out.pending is not None:
+            pend = out.pending.sum(0) if out.pending.dim() == 3 else out.pending
+            y += pend.float()
+        y = y.cpu().numpy()
+        for i, (r, a, b) in enumerate(step):
+            outs[r].append(y[cu[i]:cu[i + 1]])
+            cm.commit(r, b - a)
+    return {r: np.concatenate(v) for r, v in outs.items()}, fused_steps
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+@pytest.mark.parametrize("kind,hidden,inter", [("short_conv", 64, 128), ("attention", 64, 128), ("short_conv", 40, 72), ("short_conv", 36, 68)])
+def test_block_part(name, dtype, kind, hidden, inter):
+    """The arrangement alone: x + mixer(norm(x)), then + feed-forward(norm(.)), with norms whose gains
+    and eps differ, through ragged steps.  In bfloat16 the gains are folded into the matrices, and the
+    steps that hold single tokens only take the fused decode kernels where the sizes allow them (the
+    widths of 64 and 40 do, 36 is no multiple of 8 and does not): both ways give the plain block."""
+    from gibbs_amd.config import FeedForwardSpec, LayerSpec, MixerSpec, NormSpec, PositionSpec
+    from gibbs_amd.parts import Runtime, build_block
+    rng = np.random.default_rng(7)
+    heads, kv, hd = 4, 2, 16
+    if kind == "short_conv":
+        mixer = MixerSpec("short_conv", {"width": hidden, "kernel": 3, "bias": False}, {"in_proj": "in", "conv": "taps", "out_proj": "out"})
+        w = {"in": bf16_exact(rng.normal(size=(3 * hidden, hidden)) * 0.3), "taps": rng.normal(size=(hidden, 1, 3)),
+             "out": bf16_exact(rng.normal(size=(hidden, hidden)) * 0.3)}
+    else:
+        mixer = MixerSpec("attention", {"heads": heads, "kv_heads": kv, "head_dim": hd, "scale": hd ** -0.5, "qk_norm": "before",
+                                        "qk_norm_eps": 1e-6, "window": None},
+                          {k: k for k in ("q_proj", "k_proj", "v_proj", "out_proj", "q_norm", "k_norm")},
+                          PositionSpec("rope", {"theta": 1e4, "rotary_dim": hd, "precision": "f32"}))
+        w = {"q_proj": bf16_exact(rng.normal(size=(heads * hd, hidden)) * 0.3), "k_proj": bf16_exact(rng.normal(size=(kv * hd, hidden)) * 0.3),
+             "v_proj": bf16_exact(rng.normal(size=(kv * hd, hidden)) * 0.3), "out_proj": bf16_exact(rng.normal(size=(hidden, heads * hd)) * 0.2),
+             "q_norm": rng.normal(size=hd) * 0.1 + 1, "k_norm": rng.normal(size=hd) * 0.1 + 1}
+    w.update({"n1": rng.normal(size=hidden) * 0.2 + 1, "n2": rng.normal(size=hidden) * 0.2 + 1,
+              "w1": bf16_exact(rng.normal(size=(inter, hidden)) * 0.2), "w3": bf16_exact(rng.normal(size=(inter, hidden)) * 0.2),
+              "w2": bf16_exact(rng.normal(size=(hidden, inter)) * 0.2)})
+    spec = LayerSpec("l0", "pre_norm", NormSpec("rms", 1e-5, "n1"), mixer, NormSpec("rms", 1e-6, "n2"),
+                     FeedForwardSpec("glu", {"inter": inter, "activation": "silu"}, {"gate": "w1", "up": "w3", "down": "w2"}))
+    block = build_block(spec, hidden, 0)
+    block.bind(store(w, block.tensor_decls(), dtype), Runtime(torch.device(DEV), dtype))
+    xs = [rng.normal(size=(27, hidden)), rng.normal(size=(14, hidden))]
+    steps = STEPS + [[(0, 27, 28), (1, 14, 15)], [(1, 15, 16)]]
+    xs = [np.concatenate([x, rng.normal(size=(2, hidden))]) for x in xs]
+    got, fused = run_block(block, xs, steps, dtype)
+    n1, n2 = w["n1"].astype(np.float32).astype(np.float64), w["n2"].astype(np.float32).astype(np.float64)
+    for r, x in enumerate(xs):
+        x = x.astype(np.float32).astype(np.float64)[:len(got[r])]
+        h = P.rms_norm(x, n1, 1e-5)
+        if kind == "short_conv":
+            a = P.short_conv_mixer(h, w["in"], w["taps"].astype(np.float32).astype(np.float64), w["out"])
+        else:
+            a = P.attention_mixer(h, w["q_proj"], w["k_proj"], w["v_proj"], w["out_proj"], w["q_norm"].astype(np.float32), w["k_norm"].astype(np.float32),
+                                  heads=heads, kv_heads=kv, head_dim=hd, eps=1e-6, inv_freq=P.rope_inv_freq(hd, 1e4),
+                                  positions=list(range(len(x))), scale=hd ** -0.5)
+        y = x + a
+        want = y + P.swiglu_ffn(P.rms_norm(y, n2, 1e-6), w["w1"], w["w3"], w["w2"])
+        close(got[r], want, name, f"block {kind} request {r}")
+    if name == "bfloat16":
+        assert (fused >= 3) == (hidden % 8 == 0), f"{fused} steps took the fused decode kernels"
+    else:
+        assert fused == 0
+
+
 # --------------------------------------------------------------------------- whole specs built by hand
 def plain_spec_forward(spec, weights, ids):
     """Plain forward of a hand-built ModelSpec from the plain part functions: handles a run order
