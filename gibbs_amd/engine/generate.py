@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import time
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence, Union
+from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
 
 import torch
 
@@ -144,9 +144,13 @@ class Generator:
             self.stats.decode_seconds += dt
         return out
 
-    def run(self) -> Dict[Hashable, Generation]:
+    def run(self, on_step: Optional[Callable[[StepOutput], None]] = None) -> Dict[Hashable, Generation]:
+        """Steps until every submitted request has finished.  `on_step` sees every step's output as it
+        happens (`emitted`: the (request, token) pairs of the step or burst), for callers that stream."""
         while self.scheduler.has_work():
-            self.step()
+            out = self.step()
+            if on_step is not None:
+                on_step(out)
         return self.results()
 
     def results(self) -> Dict[Hashable, Generation]:

@@ -199,6 +199,13 @@ def test_measured_budget_changes_no_token(dirs):
             tuner = gen.scheduler.tuner
             assert tuner.prefill_s_per_token > 0 and tuner.decode_round_s > 0
     assert runs[0] == runs[1]
+    # a caller that streams sees every token once, in order, as the steps (or bursts) emit them
+    eng = Engine(d, dtype="float32", max_tokens=2048, max_requests=4)
+    gen = Generator(eng)
+    rids = [gen.submit(p, SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True)) for p in prompts]
+    seen = {r: [] for r in rids}
+    res = gen.run(on_step=lambda out: [seen[r].append(t) for r, t in out.emitted])
+    assert [seen[r] for r in rids] == [res[r].tokens for r in rids] == runs[0]
 
 
 def test_continuous_batching_under_page_pressure(dirs):
