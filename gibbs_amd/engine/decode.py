@@ -59,6 +59,7 @@ class DecodeLoop:
         self.capacity = max_steps
         self.graph: Optional[torch.cuda.CUDAGraph] = None          # one step
         self.graph_many: Optional[torch.cuda.CUDAGraph] = None     # UNROLL steps: fewer launches from the host
+        self._prepared = None                                      # (steps done, steps) that `prepare` last made ready
         self._allocate(params)
         self.rebind(rids, last_tokens, params, first_index)
 
@@ -129,6 +130,7 @@ class DecodeLoop:
         self.counter.zero_()
         self.steps_done = 0
         self.pending = 0
+        self._prepared = None
         if not self.greedy:
             dev = engine.device
             self.temperature.copy_(torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32))
@@ -175,18 +177,31 @@ class DecodeLoop:
             ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, self.u, self.u_all,
                         self.n)
 
-    def run(self, n_steps: int) -> None:
-        """Runs `n_steps` decode steps; tokens collect on the device (see `tokens`)."""
+    def prepare(self, n_steps: int) -> None:
+        """Everything a `run(n_steps)` needs before its first replay, so that a caller who times
+        the run times replays only: pages for the steps are reserved and the tables uploaded, and
+        the captured graphs the run will replay exist (capturing runs nothing)."""
+        if self._prepared == (self.steps_done, n_steps):
+            return
         if self.steps_done + n_steps > self.capacity:
             raise StepError(f"the decode loop was made for {self.capacity} steps")
         self._reserve(n_steps)
-        if not self.greedy:
-            rows = np.array([[uniform(p.seed, request_key(r), self.index[i] + self.steps_done + s)
-                              for i, (r, p) in enumerate(zip(self.rids, self.params))]
-                             for s in range(n_steps)], dtype=np.float32)
-            self.u_all[self.steps_done:self.steps_done + n_steps].copy_(torch.from_numpy(rows))
-            self.u.copy_(self.u_all[self.steps_done])
-        if self.use_graph and self.graph is None:
+        self._draws(n_steps)
+        if self.use_graph:
+            self._capture(many=n_steps >= UNROLL)
+        self._prepared = (self.steps_done, n_steps)
+
+    def _draws(self, n_steps: int) -> None:
+        if self.greedy:
+            return
+        rows = np.array([[uniform(p.seed, request_key(r), self.index[i] + self.steps_done + s)
+                          for i, (r, p) in enumerate(zip(self.rids, self.params))]
+                         for s in range(n_steps)], dtype=np.float32)
+        self.u_all[self.steps_done:self.steps_done + n_steps].copy_(torch.from_numpy(rows))
+        self.u.copy_(self.u_all[self.steps_done])
+
+    def _capture(self, many: bool) -> None:
+        if self.graph is None:
             # warm up outside capture (lazy initialisation inside libraries), then capture one step
             # (the warm-up step is undone: metadata and per-request state are put back; its key and
             # value writes are rewritten with the same values by the first replay)
@@ -202,15 +217,19 @@ class DecodeLoop:
             with capture(g):
                 self._step()
             self.graph = g                                  # the capture itself ran nothing
+        if many and self.graph_many is None:
+            g = torch.cuda.CUDAGraph()
+            torch.cuda.synchronize()
+            with capture(g):
+                for _ in range(UNROLL):
+                    self._step()
+            self.graph_many = g
+
+    def run(self, n_steps: int) -> None:
+        """Runs `n_steps` decode steps; tokens collect on the device (see `tokens`)."""
+        self.prepare(n_steps)
         left = n_steps
-        if self.graph is not None and left >= UNROLL:
-            if self.graph_many is None:
-                g = torch.cuda.CUDAGraph()
-                torch.cuda.synchronize()
-                with capture(g):
-                    for _ in range(UNROLL):
-                        self._step()
-                self.graph_many = g
+        if self.graph_many is not None:
             while left >= UNROLL:
                 self.graph_many.replay()
                 left -= UNROLL
@@ -221,6 +240,7 @@ class DecodeLoop:
                 self._step()
         self.pending += n_steps
         self.steps_done += n_steps
+        self._prepared = None
         self.sync_cache()
 
     def sync_cache(self) -> None:
