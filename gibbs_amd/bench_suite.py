@@ -1,6 +1,6 @@
 """`gibbs --bench SUITE.json`: the reference's suite protocol on this engine.
 
-A suite is `{"defaults": {...}, "models": [{...}, ...]}` (/root/reference/bench/loop.json).  Every
+A suite is `{"defaults": {...}, "models": [{...}, ...]}` (bench/loop.json).  Every
 model entry inherits the defaults; the keys that mean something here:
 
     id              a model folder (config.json + model.safetensors), or "random:CONFIG.json" for
@@ -17,9 +17,13 @@ model entry inherits the defaults; the keys that mean something here:
                     scheduler and generate `decode_tokens` tokens each (greedy, no EOS), with
                     `max_requests` live at a time (default: all), prompts cut into portions of at
                     most `chunk` tokens (default: none) under `max_batch_tokens` (default 2048) per
-                    step; the row reports generated and prompt tokens a second over the whole run
+                    step; the row reports generated and prompt tokens a second over the whole run;
+                    or "products": every distinct matrix of the model's layers against `rows`
+                    (default 2048) rows of activations, the library's product and the hand-written
+                    tiled kernel side by side (`only`: "library" or "own" keeps one of them, for a
+                    trace under rocprofv3), each reading its matrix cold as a model step does
 
-Protocol (/root/reference/src/bench.rs:241-322): prompts are seeded synthetic ids (the reference
+Protocol (src/bench.rs:241-322): prompts are seeded synthetic ids (the reference
 cycles an encoded sentence to length, :255-259; without tokenizers on this path the ids are drawn
 instead); one warm-up prefill, then the median of `runs`; 16 warm-up decode steps, then `runs`
 runs of `decode_tokens` steps with sampling on the device, median tokens a second.
@@ -175,6 +179,60 @@ def serve(entry: Dict, base: str) -> Dict:
     return {**_serve_row(entry, n_req, live, n_prompt, n_decode, chunk, done, wall, generated, st), **latency}
 
 
+def products(entry: Dict, base: str) -> Dict:
+    """The matrix products of a prompt step one by one: microseconds and PFLOP/s of the library's
+    product and of the hand-written tiled kernel for every distinct [out, in] among the model's
+    matrices.  Six copies of a matrix take turns, so that every product reads its weights cold."""
+    import torch
+
+    from . import ops
+    from .config import config_from_dict
+    from .parts import DecoderModel
+    ident = entry["id"]
+    if not ident.startswith("random:"):
+        raise ValueError("the products workload takes a configuration (random:CONFIG.json): only shapes matter")
+    with open(os.path.join(base, ident[len("random:"):])) as f:
+        cfg = config_from_dict(json.load(f))
+    model = DecoderModel(cfg.model_spec())
+    rows, iters, only = int(entry.get("rows", 2048)), int(entry.get("iters", 24)), entry.get("only")
+    shapes: List[tuple] = []
+    for block in model.blocks:
+        for part in (block.mixer, block.ffn):
+            for shape in part.product_shapes():
+                if shape not in shapes:
+                    shapes.append(shape)
+
+    def timed(fn) -> float:
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters * 1e6
+
+    cells = []
+    for o, i in shapes:
+        x = torch.randn(rows, i, device="cuda:0", dtype=torch.bfloat16)
+        ws = [torch.randn(o, i, device="cuda:0", dtype=torch.bfloat16) for _ in range(6)]
+        turn = [0]
+
+        def weight():
+            turn[0] = (turn[0] + 1) % len(ws)
+            return ws[turn[0]]
+        flops = 2.0 * rows * o * i
+        cell = {"out": o, "in": i}
+        if only != "own":
+            us = timed(lambda: ops.gemm_library(x, weight()))
+            cell.update(library_us=round(us, 1), library_pflops=round(flops / us / 1e9, 3))
+        if only != "library":
+            us = timed(lambda: ops.gemm_bf16(x, weight(), torch.bfloat16))
+            cell.update(own_us=round(us, 1), own_pflops=round(flops / us / 1e9, 3))
+        cells.append(cell)
+    return {"model": entry["name"], "workload": "products", "dtype": "bfloat16", "rows": rows, "products": cells}
+
+
 def _serve_row(entry, n_req, live, n_prompt, n_decode, chunk, done, wall, generated, st) -> dict:
     return {"model": entry["name"], "workload": "serve", "dtype": entry["dtype"], "requests": n_req, "live": live,
             "prompt_tokens": n_prompt, "decode_tokens": n_decode, "chunk": chunk,
@@ -208,7 +266,8 @@ def run_suite(path: str) -> int:
         ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
         entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
         try:
-            row = serve(entry, base) if entry.get("workload", "decode") == "serve" else measure(entry, base)
+            workload = entry.get("workload", "decode")
+            row = {"serve": serve, "products": products}.get(workload, measure)(entry, base)
         except Exception as e:     # one model's failure is reported; the others still run (bench.rs:751)
             print(f"gibbs --bench: {entry['name']}: {type(e).__name__}: {e}", file=sys.stderr)
             failed = True
@@ -216,11 +275,12 @@ def run_suite(path: str) -> int:
         rows.append(row)
         print(json.dumps(row), flush=True)
         floor = entry.get("min_tok_s")
-        if floor is not None and row["decode_tok_s"] < float(floor):
+        if floor is not None and row.get("decode_tok_s", float("inf")) < float(floor):
             missed.append(f"{row['model']}: {row['decode_tok_s']} tok/s is below min_tok_s {floor}")
     for row in rows:
-        print(f"METRIC {_slug(row['model'])}_tok_s={row['decode_tok_s']}")
-        print(f"METRIC {_slug(row['model'])}_prefill_tok_s={row['prefill_tok_s']}")
+        if "decode_tok_s" in row:
+            print(f"METRIC {_slug(row['model'])}_tok_s={row['decode_tok_s']}")
+            print(f"METRIC {_slug(row['model'])}_prefill_tok_s={row['prefill_tok_s']}")
     pcts = [r["roofline_pct"] for r in rows if "roofline_pct" in r]
     if pcts:
         geo = math.exp(sum(math.log(max(p, 1e-9)) for p in pcts) / len(pcts))

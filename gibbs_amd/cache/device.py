@@ -15,29 +15,31 @@ class LayerCache:
     """What one layer's mixer sees of the cache during a step."""
     group: Optional[int]                        # cache group of the pages (None: no pages)
     kpages: Optional[torch.Tensor]              # [num_pages, kv_heads, page_size, head_dim]
-    vpages: Optional[torch.Tensor]
+    vpages: Optional[torch.Tensor]              # [num_pages, kv_heads, page_size, value head_dim]
     owns_pages: bool                            # False: reads another layer's pages, writes none
     states: Dict[str, torch.Tensor]             # name -> [slots, *shape] float32 (slot stride = arena row)
 
 
 class DeviceCache:
-    """Pages are laid out [layer of group, k|v, page, kv head, slot in page, head_dim] in the
-    cache dtype (the activation dtype of the run); states are float32."""
+    """Keys and values of a group are laid out [layer of group, page, kv head, slot in page, head_dim]
+    (values with their own head size) in the cache dtype (the activation dtype of the run); every
+    group has as many pages as its pool; states are float32."""
 
     def __init__(self, manager: CacheManager, cache_dtype: torch.dtype, device: torch.device):
         self.manager = manager
         self.device = device
-        self.pages: List[torch.Tensor] = []
+        self.cache_dtype = cache_dtype
+        self.kpages: List[torch.Tensor] = []
+        self.vpages: List[torch.Tensor] = []
         for g, need in enumerate(manager.group_needs):
-            n_layers = len(manager.group_layers[g])
-            self.pages.append(torch.zeros(
-                (n_layers, 2, manager.pools[g].num_pages, need.kv_heads, manager.page_size, need.head_dim),
-                dtype=cache_dtype, device=device))
+            lead = (len(manager.group_layers[g]), manager.pools[g].num_pages, need.kv_heads, manager.page_size)
+            self.kpages.append(torch.zeros(lead + (need.head_dim,), dtype=cache_dtype, device=device))
+            self.vpages.append(torch.zeros(lead + (need.value_dim,), dtype=cache_dtype, device=device))
         self.arena = torch.zeros((manager.max_requests, max(1, manager.slot_floats)),
                                  dtype=torch.float32, device=device)
 
     def nbytes(self) -> int:
-        return sum(p.numel() * p.element_size() for p in self.pages) + self.arena.numel() * 4
+        return sum(p.numel() * p.element_size() for p in self.kpages + self.vpages) + self.arena.numel() * 4
 
     def layer_view(self, layer: int, kv_source: Optional[int] = None) -> LayerCache:
         m = self.manager
@@ -46,7 +48,7 @@ class DeviceCache:
         k = v = None
         if group is not None:
             idx = m.group_layers[group].index(src)
-            k, v = self.pages[group][idx, 0], self.pages[group][idx, 1]
+            k, v = self.kpages[group][idx], self.vpages[group][idx]
         states = {}
         for (li, name), (off, shape) in m.state_layout.items():
             if li == layer:

@@ -22,7 +22,7 @@ _SIGNATURES = {
     "gibbs_pool_is_held": ([c_void_p, c_int], c_int),
     "gibbs_pool_allocate": ([c_void_p, c_int, _ip], c_int),
     "gibbs_pool_release": ([c_void_p, _ip, c_int], c_int),
-    "gibbs_cache_create": ([c_int, _ip, c_int, c_int, c_int], c_void_p),
+    "gibbs_cache_create": ([c_int, _ip, c_int, _ip, c_int], c_void_p),
     "gibbs_cache_destroy": ([c_void_p], None),
     "gibbs_cache_free_pages": ([c_void_p, c_int], c_int),
     "gibbs_cache_free_slots": ([c_void_p], c_int),

@@ -14,19 +14,22 @@ What is given back and when.  `release` returns every page and the slot (a reque
 failed or was preempted); `commit` returns a window group's passed pages.  Pages are used
 again without being cleared: kernels see a key only through its position, never through what
 a page holds.  The reference returns blocks on the same events
-(/root/reference/src/scheduler/mod.rs:1215-1217, :1561-1563).
+(src/scheduler/mod.rs:1215-1217, :1561-1563).
 """
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple, Union
 
 import numpy as np
 
 from . import host
 from .needs import CacheNeed, StateNeed
-from .pages import PageError
 
 NO_PAGE = -1
+
+
+class PageError(RuntimeError):
+    """A page was freed twice, freed without being held, or is not of its pool."""
 
 
 class _PoolView:
@@ -50,9 +53,10 @@ class CacheManager:
     hang on `DeviceCache`, which reads this."""
 
     def __init__(self, needs: Sequence[Optional[CacheNeed]], states: Sequence[Sequence[StateNeed]],
-                 page_size: int, num_pages: int, max_requests: int):
+                 page_size: int, num_pages: Union[int, Sequence[int]], max_requests: int):
         """`needs[i]` / `states[i]`: what the mixer of run i of the layer order asks for (None / ()
-        for nothing).  `num_pages`: pages of every group's pool."""
+        for nothing).  `num_pages`: pages of every group's pool, or one count per group in the
+        order the groups first appear (a group with a window can do with fewer)."""
         if page_size <= 0 or max_requests <= 0:
             raise ValueError("page_size and max_requests must be positive")
         self.page_size = page_size
@@ -69,8 +73,12 @@ class CacheManager:
             g = self.group_needs.index(need)
             self.group_layers[g].append(i)
             self.layer_group[i] = g
-        if self.group_needs and num_pages <= 0:
-            raise ValueError(f"a page pool needs at least one page, not {num_pages}")
+        n_groups = len(self.group_needs)
+        per_group = [int(num_pages)] * n_groups if isinstance(num_pages, int) else [int(n) for n in num_pages]
+        if len(per_group) != n_groups:
+            raise ValueError(f"{len(per_group)} page counts for {n_groups} cache groups")
+        if any(n <= 0 for n in per_group):
+            raise ValueError(f"a page pool needs at least one page, not {min(per_group)}")
         # state layout of a slot: (layer, name) -> (offset, shape), in float32 elements
         self.state_layout: Dict[Tuple[int, str], Tuple[int, Tuple[int, ...]]] = {}
         off = 0
@@ -83,11 +91,10 @@ class CacheManager:
         self.slot_floats = off
         self._lib = host.library()
         windows = host.ints([int(n.window or 0) for n in self.group_needs])
-        self._core = self._lib.gibbs_cache_create(len(self.group_needs), windows, page_size, max(1, num_pages),
-                                                  max_requests)
+        self._core = self._lib.gibbs_cache_create(n_groups, windows, page_size, host.ints(per_group), max_requests)
         if not self._core:
             raise ValueError("the cache core refused its sizes")
-        self.pools = [_PoolView(self, g, num_pages) for g in range(len(self.group_needs))]
+        self.pools = [_PoolView(self, g, per_group[g]) for g in range(n_groups)]
         self._slots: Dict[Hashable, int] = {}
         self._needed = host.ints([0] * len(self.group_needs))
 
@@ -204,9 +211,13 @@ class CacheManager:
         return out
 
     def take_fresh_slots(self) -> List[int]:
-        out = host.ints([0] * self.max_requests)
-        n = self._lib.gibbs_cache_take_fresh_slots(self._core, out, self.max_requests)
-        return list(out[:n])
+        """Slots that requests have taken since the last call (every one of them, once)."""
+        out, fresh = host.ints([0] * self.max_requests), []
+        while True:
+            n = self._lib.gibbs_cache_take_fresh_slots(self._core, out, self.max_requests)
+            fresh += list(out[:n])
+            if n < self.max_requests:
+                return fresh
 
     # ------------------------------------------------------------------ invariants (tests)
     def check(self) -> None:

@@ -9,10 +9,16 @@ from typing import Optional, Tuple
 class CacheNeed:
     """Keys and values of every cached position (`window` None), or of the last `window`
     positions only.  Layers with equal needs form one group: one page pool and one block
-    table per request serve all of them."""
+    table per request serve all of them.  Values may have a head size of their own
+    (`v_head_dim`, default: the keys')."""
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)

@@ -1,4 +1,4 @@
-"""Command line in the manner of the reference's `gibbs` binary (/root/reference/src/main.rs:27-189):
+"""Command line in the manner of the reference's `gibbs` binary (src/main.rs:27-189):
 the same option names and meanings where it has them (`--model`, `--prompt`, `--max-tokens`, `--ctx`,
 `--backend`, `--seed`, `--arch`, `--arch-dump`, `--bench`, `--bench-parity`, `--probe-top5`), and this
 engine's own beside them (`--replay`, `--random-weights`, sampling and cache options).  One-shot generation prints the reference's lines (main.rs:741-772,
@@ -57,7 +57,7 @@ def _tokenizer(model_dir: str):
 
 
 def _parity(make_engine, prompt: List[int], steps: int = 8) -> int:
-    """The reference's device-parity gate (/root/reference/src/bench.rs:761-883: 8 greedy steps on
+    """The reference's device-parity gate (src/bench.rs:761-883: 8 greedy steps on
     Metal and on the CPU, same argmax, cosine >= 0.999), here between the bfloat16 path and the
     true 32-bit path.  The float32 run's tokens are forced on the bfloat16 run so that every step
     compares logits of the same sequence."""

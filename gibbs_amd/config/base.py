@@ -15,7 +15,7 @@ class ConfigError(ValueError):
 def first(cfg: Mapping[str, Any], *keys: str, default: Any = None) -> Any:
     """The value of the first of `keys` that config.json holds (dotted keys descend into
     objects), else `default`: the precedence rule of the reference's config expressions
-    (`first(cfg.a, cfg.b, ...)`, /root/reference/src/arch/expr.rs:723)."""
+    (`first(cfg.a, cfg.b, ...)`, src/arch/expr.rs:723)."""
     for key in keys:
         node: Any = cfg
         for part in key.split("."):

@@ -1,7 +1,7 @@
 """Typed configuration of LFM2 (`Lfm2ForCausalLM`, model_type `lfm2`).
 
 Keys, their precedence and defaults follow the reference's family spec
-(/root/reference/arch/families/lfm2.json5:27-57).  Where the reference decides by
+(arch/families/lfm2.json5:27-57).  Where the reference decides by
 which tensors a checkpoint holds (layer kind :78-80, tied head :91, vocabulary :35),
 the same rule is used when the tensor table of the checkpoint is at hand, and
 config.json's own keys (`layer_types`, `full_attn_idxs`, `tie_embedding`) otherwise.
@@ -23,7 +23,7 @@ ATTENTION = "full_attention"
 def feed_forward_width(ff_raw: int, auto_adjust: bool, multiplier: float, multiple_of: int) -> int:
     """The SwiGLU width (lfm2.json5:38-41): with `block_auto_adjust_ff_dim`, two thirds of
     the raw width, rounded up to `block_multiple_of` only when a multiplier is given
-    (`int()` truncates, /root/reference/src/arch/expr.rs:820); else the raw width."""
+    (`int()` truncates, src/arch/expr.rs:820); else the raw width."""
     if not auto_adjust:
         return ff_raw
     ff_23 = ff_raw * 2 // 3
@@ -138,6 +138,13 @@ class Lfm2Config(ArchConfig):
                               for i in range(layers))
             if kinds is None:
                 kinds = by_tensor
+            elif kinds != by_tensor:
+                # (a layer without the convolution's in-projection counts as attention, as the reference's
+                # spec decides it, arch/families/lfm2.json5:78-80)
+                wrong = [i for i in range(layers) if kinds[i] != by_tensor[i]]
+                raise ConfigError(
+                    "config.json and the checkpoint's tensors disagree about the kind of layers "
+                    f"{wrong}: config.json says {[kinds[i] for i in wrong]}, the tensors say {[by_tensor[i] for i in wrong]}")
         if kinds is None:
             raise ConfigError("config.json lacks layer_types / full_attn_idxs")
         return kinds

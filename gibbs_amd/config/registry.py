@@ -1,9 +1,9 @@
 """One registry from an architecture's name to its configuration class.
 
-Detection follows the reference (/root/reference/src/arch/mod.rs:723-759): the first
+Detection follows the reference (src/arch/mod.rs:723-759): the first
 registered architecture whose names match config.json's `architectures` entries or its
 `model_type`; `arch=` forces one (the CLI's `--arch`,
-/root/reference/src/main.rs:180-183).
+src/main.rs:180-183).
 """
 from __future__ import annotations
 

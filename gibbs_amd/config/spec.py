@@ -24,9 +24,11 @@ class NormSpec:
 @dataclass(frozen=True)
 class PositionSpec:
     """A position encoding applied inside a mixer (`"rope"`, `"none"`, or one that a
-    test or another architecture registers)."""
+    test or another architecture registers).  `tensors` names the checkpoint tensors of an
+    encoding that has any (a learned table)."""
     kind: str
     params: Mapping[str, Any] = field(default_factory=dict)
+    tensors: Mapping[str, str] = field(default_factory=dict)
 
 
 @dataclass(frozen=True)

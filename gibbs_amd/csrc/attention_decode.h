@@ -528,8 +528,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   const long longest = (bound + a.n_splits - 1) / a.n_splits + 8 * TILE;
   const bool mm_can = a.hd % 16 == 0 && a.hd <= 128 && longest / a.page_size + 2 <= SEG_PAGES;
   GIBBS_REQUIRE(kind != 2 || mm_can, "attention_decode: the matrix-core kernel takes head sizes in steps of 16 up to 128 and key slices of at most %d pages (head size %d, %ld keys a slice)", SEG_PAGES - 2, a.hd, longest);
-  static const char* env = getenv("GIBBS_DECODE_ATTENTION");   // "valu" or "mfma": for measurements
-  const bool mm = kind == 2 || (kind == 0 && mm_can && !(env && env[0] == 'v'));
+  const bool mm = kind == 2 || (kind == 0 && mm_can);
   if (lanes <= 2) launch_waves<2, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);
   else if (lanes <= 4) launch_waves<4, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);
   else if (lanes <= 8) launch_waves<8, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);

@@ -4,7 +4,8 @@
 //
 //   row n, head h (kv head g = h / (nh / nkv)), position p = pos[n], request r = row_req[n]:
 //   visible keys are lo .. p with lo = max(0, p - window + 1) (window 0: all keys);
-//   s_k = (q . K[k]) * scale;  out = sum_k softmax(s)_k V[k], maxima and sums in float32.
+//   s_k = (q . K[k]) * scale (+ slopes[h] * (k - p) when the position encoding is a linear bias over
+//   the distance);  out = sum_k softmax(s)_k V[k], maxima and sums in float32.
 // Key k of request r lives in page table[r][k / ps] at slot k % ps; pages are
 // [page, kv head, slot in page, hd].  Visibility is by position only; what else a page holds is
 // never read.  One wave per (row, head).  Keys are taken in blocks of 64 aligned to absolute key
@@ -25,6 +26,7 @@ struct AttnArgs {
   long ldo;  // row stride of out
   float scale;
   int window;
+  const float* slopes;  // [nh] or null: s_k += slopes[h] * (k - p)
 };
 
 template <typename T>
@@ -66,6 +68,7 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
       float dot = 0.f;
       for (int e = 0; e < hd; ++e) dot = fmaf(sq[wave][e], to_float(kr[e]), dot);
       s = dot * a.scale;
+      if (a.slopes) s += a.slopes[h] * (float)(key - p);
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float w = valid ? expf(s - m_new) : 0.f;
@@ -98,14 +101,14 @@ __global__ __launch_bounds__(256) void attention_plain_kernel(const T* __restric
 GIBBS_EXPORT int gibbs_attention_plain(const void* q, const void* kpages, const void* vpages, void* out, int dtype,
                                        const int* pos, const int* row_req, const int* table, int max_pages,
                                        int page_size, int num_pages, int n_rows, int nh, int nkv, int hd, long ldq,
-                                       long ldo, float scale, int window, hipStream_t stream) {
+                                       long ldo, float scale, int window, const float* slopes, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && nh > 0 && nkv > 0 && hd > 0, "attention: bad sizes rows=%d heads=%d kv=%d hd=%d", n_rows, nh, nkv, hd);
   GIBBS_REQUIRE(nh % nkv == 0, "attention: %d heads are not a multiple of %d kv heads", nh, nkv);
   GIBBS_REQUIRE(hd <= MAX_HD, "attention: head size %d above %d", hd, MAX_HD);
   GIBBS_REQUIRE(ldq >= (long)nh * hd && ldo >= (long)nh * hd, "attention: row strides shorter than heads * hd");
   GIBBS_REQUIRE(page_size > 0 && max_pages > 0 && num_pages > 0 && window >= 0, "attention: bad cache geometry");
   if (n_rows == 0) return 0;
-  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window};
+  AttnArgs a{pos, row_req, table, max_pages, page_size, num_pages, nh, nkv, hd, ldq, ldo, scale, window, slopes};
   dim3 grid(n_rows, ceil_div(nh, 4));
   GIBBS_REQUIRE(grid.y <= 65535, "attention: too many heads (%d)", nh);
   if (dtype == GIBBS_F32)

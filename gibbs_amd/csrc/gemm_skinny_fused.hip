@@ -19,10 +19,10 @@
 //   epilogues      STORE     y = acc (bfloat16)
 //                  RESIDUAL  x += acc (float32 stream, each element owned by one workgroup);
 //                            xb = bfloat16(x), the mirror the next product reads
-//                  GLU       out = silu(gate) * up
+//                  GLU       out = act(gate) * up (activation.h)
 //                  CONV      bx = B * x;  cv = bias + taps . [state, bx];  y = C * cv;  state shifts
 //                            (every row is one decoded token of a different request)
-#include "common.h"
+#include "activation.h"
 #include <stdlib.h>
 
 namespace {
@@ -58,6 +58,7 @@ struct FusedArgs {
   const int* slot;  // [N]
   const int* ctx;   // [N] cached length of each row's request (history rows before position 0 are zero)
   int K;
+  int act;  // GLU: the activation's code
 };
 
 // KC: the convolution's kernel length when it is 2..4 (its operands are then asked for before the
@@ -320,7 +321,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
         const float gt = sum[0][t][i] * scale, up = sum[RG > 1 ? 1 : 0][t][i] * scale;
-        y[i] = (bf16)(gt * (1.0f / (1.0f + expf(-gt))) * up);
+        y[i] = (bf16)(activate(gt, a.act) * up);
       }
     } else if (KC > 1) {  // EPI_CONV, operands at hand
       float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
@@ -375,8 +376,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 
 template <int NT, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
-  static const int rows8_below = getenv("GIBBS_SKINNY_ROWS8_BELOW") ? atoi(getenv("GIBBS_SKINNY_ROWS8_BELOW")) : 256;
-  static const int tiles2_from = getenv("GIBBS_SKINNY_TILES2_FROM") ? atoi(getenv("GIBBS_SKINNY_TILES2_FROM")) : 192;
+  constexpr int rows8_below = 256;   // tiles of 16 features below which a workgroup takes 8 (one per compute unit)
+  constexpr int tiles2_from = 192;   // pairs of tiles from which a workgroup takes two (measured at 33 to 64 rows)
   if constexpr (NT >= 3 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
     // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
     if (a.O / 32 >= tiles2_from) {
@@ -421,8 +422,7 @@ int check_common(const char* what, const void* X, const void* W, int N, int O, i
 
 // A row stride of 0 says that W is in tile order (pack_weight).
 void note_layout(FusedArgs& a) {
-  static const int rotate = getenv("GIBBS_SKINNY_ROTATE") ? atoi(getenv("GIBBS_SKINNY_ROTATE")) : 1;   // for measurements
-  a.rotate = rotate;
+  a.rotate = 1;
   if (a.ldw != 0) return;
   a.packed = 1;
   a.ktiles = ceil_div(a.I, 32);
@@ -459,12 +459,13 @@ GIBBS_EXPORT int gibbs_skinny_residual(const void* X, const void* W, float* x, v
 
 // out[n, f] = silu(s_n gate_f . X_n) * (s_n up_f . X_n); W = [gate rows (F); up rows (F)], rms prologue.
 GIBBS_EXPORT int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, int F, int I, long ldx, long ldw,
-                                  long ldy, int rms, float eps, hipStream_t stream) {
+                                  long ldy, int rms, float eps, int act, hipStream_t stream) {
   if (check_common("skinny_glu", X, W, N, F, I, ldx, ldw)) return 1;
   GIBBS_REQUIRE(ldy >= F, "skinny_glu: output rows shorter than %d", F);
+  GIBBS_REQUIRE(act >= 0 && act < ACT_COUNT, "skinny_glu: unknown activation %d", act);
   FusedArgs a{};
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
-  a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy;
+  a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy; a.act = act;
   if (rms) launch_nt<2, true, EPI_GLU>(a, stream);
   else launch_nt<2, false, EPI_GLU>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_glu");

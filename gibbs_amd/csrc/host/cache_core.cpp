@@ -2,10 +2,10 @@
 // cache group, slots for per-request state, and the packing of one step's integer metadata into
 // the staging buffer that travels to the device in one copy.  Plain C++ (no GPU calls), C interface.
 //
-// The accounting follows the reference's block pool (/root/reference/src/kv/mod.rs:337-430: a free
+// The accounting follows the reference's block pool (src/kv/mod.rs:337-430: a free
 // list that allocation pops and release pushes) without its reference counts and prefix tree: a
 // page belongs to at most one request.  Blocks are given back on the events the reference gives
-// them back on (/root/reference/src/scheduler/mod.rs:1215-1217, :1561-1563), and, for a group with
+// them back on (src/scheduler/mod.rs:1215-1217, :1561-1563), and, for a group with
 // a window, as soon as no later query can see them.
 //
 // A live request is named by its slot index.  Every function returns 0 (or a count) on success
@@ -48,15 +48,18 @@ HOST_EXPORT int gibbs_pool_release(void* pool, const int* pages, int n) {
 }
 
 // ------------------------------------------------------------------------------------------- cache core
-// windows[g]: the window of group g, 0 for none.  Every group's pool has num_pages pages.
-HOST_EXPORT void* gibbs_cache_create(int n_groups, const int* windows, int page_size, int num_pages, int max_requests) {
-  if (n_groups < 0 || page_size <= 0 || max_requests <= 0 || (n_groups > 0 && num_pages <= 0)) return nullptr;
+// windows[g]: the window of group g, 0 for none; num_pages[g]: the pages of its pool (a group with a
+// window needs fewer than one that keeps every key).
+HOST_EXPORT void* gibbs_cache_create(int n_groups, const int* windows, int page_size, const int* num_pages, int max_requests) {
+  if (n_groups < 0 || page_size <= 0 || max_requests <= 0) return nullptr;
+  for (int g = 0; g < n_groups; ++g)
+    if (num_pages[g] <= 0) return nullptr;
   CacheCore* c = new CacheCore();
   c->page_size = page_size;
   c->max_requests = max_requests;
   for (int g = 0; g < n_groups; ++g) {
     c->window.push_back(windows[g]);
-    c->pools.emplace_back(num_pages);
+    c->pools.emplace_back(num_pages[g]);
   }
   c->requests.resize(max_requests);
   for (int s = max_requests - 1; s >= 0; --s) c->free_slots.push_back(s);
@@ -155,6 +158,9 @@ HOST_EXPORT int gibbs_cache_release(void* core, int slot) {
   r.live = false;
   r.pages.clear();
   c->free_slots.push_back(slot);
+  // a slot that was taken and given back before any step ran is not fresh any more (its next taker
+  // lists it again)
+  c->fresh_slots.erase(std::remove(c->fresh_slots.begin(), c->fresh_slots.end(), slot), c->fresh_slots.end());
   return status;
 }
 

@@ -4,7 +4,7 @@
 // the sampling parameters and the results stay with the caller) and takes slots and pages from the
 // cache core directly.
 //
-// Policy of the reference's scheduler (/root/reference/src/scheduler/mod.rs:1128-1580): first-in
+// Policy of the reference's scheduler (src/scheduler/mod.rs:1128-1580): first-in
 // first-out admission that stops at the first request that does not fit (:1155-1221); decoders first,
 // then the shortest remaining prompt, while the oldest prefilling request keeps up to half the budget
 // (:1235-1246, :1271-1283); one token per decoding request per step (:1376-1487); a request ends on an
@@ -214,15 +214,21 @@ HOST_EXPORT int gibbs_sched_plan(void* sched, long* plan, int plan_cap, long* ev
     Seq& q = s->seqs[id];
     if (q.max_new == 0 && q.output_len == 0) {
       s->waiting.pop_front();
-      s->finish(id, EV_FINISHED_LENGTH);                  // /root/reference/src/scheduler/mod.rs:1357-1359
+      s->finish(id, EV_FINISHED_LENGTH);                  // src/scheduler/mod.rs:1357-1359
       continue;
     }
     const long total = q.total();
-    long pool = 1L << 60;
-    for (const PagePool& p : c->pools) pool = std::min<long>(pool, p.num_pages);
-    if (c->pages_for(total + 1) > pool) {
+    // a request that no pool can ever hold: every key in a group without a window; in a group with one,
+    // the window and the portion that is reserved before the window moves on
+    long short_by = 0;
+    for (int g = 0; g < c->n_groups(); ++g) {
+      long need = c->pages_for(total + 1);
+      if (c->window[g] > 0) need = std::min(need, c->pages_for(c->window[g] + std::min(total, cap)) + 2);
+      if (need > c->pools[g].num_pages) short_by = std::max(short_by, need);
+    }
+    if (short_by > 0) {
       s->waiting.pop_front();
-      s->finish(id, EV_ERROR_TOO_LARGE, c->pages_for(total + 1));
+      s->finish(id, EV_ERROR_TOO_LARGE, short_by);
       continue;
     }
     const int slot = gibbs_cache_admit(c);

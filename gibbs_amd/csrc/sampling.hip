@@ -247,7 +247,7 @@ __global__ __launch_bounds__(THREADS) void sample_kernel(const float* __restrict
 
 // Repetition penalty of the reference's sampler, applied to the logits in place before a row is
 // sampled.  A token that occurs c times among the row's recent tokens (the reference passes the last
-// 64 of prompt and output): greedy rows (/root/reference/src/runtime/lm.rs:1089-1105): c times
+// 64 of prompt and output): greedy rows (src/runtime/lm.rs:1089-1105): c times
 // v = v > 0 ? v / penalty : v * penalty, then v -= 1.5 c; sampled rows (:1176-1189): c times
 // v = (v > 0 ? v / penalty : v * penalty) - 1.5.  Rows whose penalty is <= 1 are left alone (:1072,
 // :1163).  One workgroup of R threads per row; the first thread that holds a token does its update.

@@ -3,7 +3,7 @@
 `step(entries)` runs exactly the tokens it is given, as one batch, from the cache that earlier
 steps left, and returns the logits at the wanted places.  The reference's counterpart is
 `NativeLm::forward(tokens, start_pos, state)` for one sequence
-(/root/reference/src/model/native.rs:78-83, /root/reference/src/runtime/lm.rs:513-583); here a
+(src/model/native.rs:78-83, src/runtime/lm.rs:513-583); here a
 step takes any mix of prompt portions and decoded tokens of several requests.  Its guards are
 the reference's (lm.rs:528-544): no empty token list, no position beyond the context limit.
 """
@@ -25,7 +25,7 @@ from ..parts import DecoderModel, Runtime
 from ..weights import WeightStore, load_weights, table_of
 from .batch import BatchStager, Entry, StepBatch
 
-DEFAULT_PAGE_SIZE = 16      # tokens per cache page, the reference's block size (/root/reference/src/kv/mod.rs:6)
+DEFAULT_PAGE_SIZE = 16      # tokens per cache page, the reference's block size (src/kv/mod.rs:6)
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
 
@@ -41,11 +41,17 @@ class Engine:
     def __init__(self, model_dir: Optional[str] = None, *, dtype: str = "bfloat16", max_tokens: int = 8192,
                  max_requests: int = 8, page_size: int = DEFAULT_PAGE_SIZE, device: str = "cuda:0", arch: Optional[str] = None,
                  ctx: Optional[int] = None, config: Optional[ArchConfig] = None,
-                 weights: Optional[WeightStore] = None):
+                 weights: Optional[WeightStore] = None, fold_gains: bool = True, fused_decode_rows: int = 64,
+                 group_pages: Optional[Sequence[int]] = None):
         """`model_dir`: a folder with config.json and model.safetensors (the model class is chosen
         by config.json).  `max_tokens`: tokens the cache pool holds (each request's count rounded
         up to whole pages).  `ctx`: context limit, default config.json's max_position_embeddings.
-        `config` + `weights` may stand in for a folder (weights already on the device)."""
+        `config` + `weights` may stand in for a folder (weights already on the device).
+        `fold_gains=False` keeps the norms' gains out of the bfloat16 matrices and `fused_decode_rows=0`
+        keeps steps of decoded tokens off the fused decode kernels: the same model on the general path,
+        for comparisons.  `group_pages`: pages of every cache group's pool, one count per group in
+        the order the groups first appear in the layer order (default: `max_tokens` worth for each; a
+        group with a window can do with about max_requests x (window + longest portion) tokens)."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU: this engine has no CPU path")
         if dtype not in DTYPES:
@@ -65,13 +71,14 @@ class Engine:
         self.page_size = page_size
         self.ctx_limit = int(ctx) if ctx else self.spec.max_position
         num_pages = max(1, -(-max_tokens // page_size))
-        self.rt = Runtime(self.device, self.dtype, max_positions=min(self.ctx_limit, num_pages * page_size))
+        self.rt = Runtime(self.device, self.dtype, max_positions=min(self.ctx_limit, num_pages * page_size),
+                          fold_gains=fold_gains, fused_decode_rows=fused_decode_rows)
         self.model.bind(weights, self.rt)
         self.weight_bytes = weights.nbytes()
         del weights
 
-        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), page_size, num_pages,
-                                  max_requests)
+        self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), page_size,
+                                  num_pages if group_pages is None else list(group_pages), max_requests)
         self.device_cache = DeviceCache(self.cache, self.dtype, self.device)
         self._views = [self.device_cache.layer_view(run, src)
                        for run, src in enumerate(self.model.kv_source_runs())]

@@ -1,8 +1,8 @@
 """Generation through the scheduler: the Python entry point and what the command line prints.
 
 `Generator` ties an `Engine` to a `ContinuousBatchScheduler` and a `Sampler`, in the manner of the
-reference's one-shot path (/root/reference/src/scheduler/mod.rs:1080-1120,
-/root/reference/src/main.rs:741-772): submit, step until done, report prefill and decode speed.
+reference's one-shot path (src/scheduler/mod.rs:1080-1120,
+src/main.rs:741-772): submit, step until done, report prefill and decode speed.
 """
 from __future__ import annotations
 

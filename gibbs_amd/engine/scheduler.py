@@ -1,6 +1,6 @@
 """Continuous batching above the step function.
 
-Policy follows the reference's scheduler (/root/reference/src/scheduler/mod.rs:1128-1580):
+Policy follows the reference's scheduler (src/scheduler/mod.rs:1128-1580):
   * waiting requests are admitted first-in first-out while a slot and the pages of their first
     portion are free; the first that does not fit goes back to the front and admission stops for
     this step (:1155-1221);

@@ -9,7 +9,7 @@ import torch
 from .lib import KernelError, call, dtype_code, library, ptr, require_cuda, stream
 
 ROPE_VARIANTS = {"half_split": 0, "interleaved": 1}
-ACTIVATIONS = {"silu": 0}
+ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "gelu": 2, "relu": 3}     # csrc/activation.h
 
 
 def _i32(t: torch.Tensor, n: int, what: str) -> None:
@@ -282,16 +282,18 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
 
 
 def skinny_glu(x: torch.Tensor, w_gate_up: torch.Tensor, rms_eps: Optional[float] = None,
-               out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """out = silu(s x @ gate^T) * (s x @ up^T) with w_gate_up = [gate rows; up rows]."""
+               out: Optional[torch.Tensor] = None, activation: str = "silu") -> torch.Tensor:
+    """out = act(s x @ gate^T) * (s x @ up^T) with w_gate_up = [gate rows; up rows]."""
     n, i, ldx = _skinny_check(x, w_gate_up, "skinny_glu", groups=2)
+    if activation not in ACTIVATIONS:
+        raise KernelError(f"skinny_glu: activation {activation!r} is not implemented; known: {sorted(ACTIVATIONS)}")
     assert w_gate_up.shape[0] % 2 == 0
     f = w_gate_up.shape[0] // 2
     if out is None:
         out = torch.empty((n, f), dtype=torch.bfloat16, device=x.device)
     assert out.shape == (n, f) and out.dtype == torch.bfloat16 and out.is_contiguous()
     call("gibbs_skinny_glu", ptr(x), ptr(_w(w_gate_up)), ptr(out), n, f, i, ldx, w_gate_up.stride(0), f,
-         int(rms_eps is not None), float(rms_eps or 0.0), stream())
+         int(rms_eps is not None), float(rms_eps or 0.0), ACTIVATIONS[activation], stream())
     return out
 
 
@@ -459,10 +461,13 @@ def rope_table(inv_freq: torch.Tensor, n_pos: int) -> torch.Tensor:
 
 def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
-                    scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
+                    slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal grouped-query attention of every row over its request's cache pages.
-    q: [N, >= nh*hd] (row stride free); pages: [num_pages, nkv, page_size, hd]; table: [R, max_pages]."""
-    require_cuda(q, kpages, vpages, table, pos, row_req)
+    q: [N, >= nh*hd] (row stride free); pages: [num_pages, nkv, page_size, hd]; table: [R, max_pages].
+    `slopes` (float32 [nh]): the score of key k for a query at position p gets slopes[h] * (k - p) added."""
+    require_cuda(q, kpages, vpages, table, pos, row_req, slopes)
+    assert slopes is None or (slopes.dtype == torch.float32 and slopes.shape == (nh,) and slopes.is_contiguous())
     assert q.dim() == 2 and q.shape[0] == n_rows and q.stride(1) == 1 and q.shape[1] >= nh * hd
     num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
     assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
@@ -473,7 +478,7 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
     call("gibbs_attention_plain", ptr(q), ptr(kpages), ptr(vpages), ptr(out), dtype_code(q.dtype), ptr(pos),
          ptr(row_req), ptr(table), table.shape[1], page_size, num_pages, n_rows, nh, nkv, hd,
-         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), stream())
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), ptr(slopes), stream())
     return out
 
 

@@ -39,7 +39,7 @@ _SIGNATURES = {
                            c_void_p],
     "gibbs_skinny_residual": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_void_p],
     "gibbs_skinny_glu": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_int, c_float,
-                         c_void_p],
+                         c_int, c_void_p],
     "gibbs_skinny_conv": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_int, c_float, c_void_p,
                           c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_void_p],
     "gibbs_attention_decode_fused": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -53,7 +53,7 @@ _SIGNATURES = {
                          c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long,
                          c_void_p],
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
-                              c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p],
+                              c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p, c_void_p],
     "gibbs_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,

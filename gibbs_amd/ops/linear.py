@@ -20,7 +20,7 @@ from .lib import KernelError, require_cuda
 
 # rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
 # output features, which stops paying beyond one or two MFMA tiles of rows)
-SKINNY_ROWS = int(os.environ.get("GIBBS_SKINNY_ROWS", "32"))
+SKINNY_ROWS = 32
 USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 # the library product is hipBLASLt called directly (its heuristic's choice kept per shape: a call costs
 # the host 12 us instead of the 20 us of torch.matmul); "torch" goes through PyTorch

@@ -1,12 +1,17 @@
 """Grouped-query attention mixer over the paged cache.
 
-In the reference's order (/root/reference/arch/lib/transformer.json5:46-87): q, k, v
+In the reference's order (arch/lib/transformer.json5:46-87): q, k, v
 projections; optional RMSNorm of every head of q and k with one [head_dim] gain (`qk_norm:
-"before"` the rotation, as LFM2 has it, /root/reference/arch/families/lfm2.json5:80-83);
+"before"` the rotation, as LFM2 has it, arch/families/lfm2.json5:80-83);
 position encoding of q and k; k, v written to the cache at their positions; causal attention of
 each row over the keys up to its own position (within `window`, if given), query head h reading
 kv head h // (heads / kv_heads) with scale `scale`; output projection.  A mixer whose params
 name `kv_source` projects no k, v and reads that layer's pages (the reference's `write: false`).
+
+The position encoding is asked how it works (`PositionEncoding`): a rotation goes to the kernels
+as tables and every fast path stays open; an encoding that changes q and k itself (`apply`) or
+biases the scores by distance (`score_slopes`) sends the mixer down its general path (norm, the
+hook, cache write; the plain attention kernel takes the slopes).
 """
 from __future__ import annotations
 
@@ -49,6 +54,10 @@ class AttentionMixer(Mixer):
             return None
         return CacheNeed(self.kv_heads, self.head_dim, None if self.window is None else int(self.window))
 
+    def attention_flops(self, keys: float) -> float:
+        """Multiply-adds x 2 of scores and weighted values when the step's rows see `keys` keys in all."""
+        return 2.0 * 2.0 * keys * self.heads * self.head_dim
+
     def kv_source(self) -> Optional[int]:
         return self.source
 
@@ -62,6 +71,8 @@ class AttentionMixer(Mixer):
             decls.append(TensorDecl(t["q_norm"], (hd,), FLOAT32, init="gain"))
             if self.source is None:
                 decls.append(TensorDecl(t["k_norm"], (hd,), FLOAT32, init="gain"))
+        if self.position is not None:
+            decls += self.position.tensor_decls()
         return decls
 
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
@@ -76,15 +87,27 @@ class AttentionMixer(Mixer):
         self.p_qkv = self.p_out = None
         self.q_gain = weights[t["q_norm"]] if self.qk_norm else None
         self.k_gain = weights[t["k_norm"]] if self.qk_norm and self.source is None else None
+        self.rot, self.slopes, self.pos_hook = None, None, False
         if self.position is not None:
             self.position.bind(weights, rt)
+            self.rot = self.position.rotation()
+            self.slopes = self.position.score_slopes(self.heads)
+            self.pos_hook = self.rot is None and self.position.transforms_rows()
+        if self.slopes is not None and (self.slopes.dtype != torch.float32 or tuple(self.slopes.shape) != (self.heads,)):
+            raise ValueError(f"score slopes must be float32 [{self.heads}]")
+        # the fast kernels know rotations only (or no encoding at all)
+        self.fast_ok = self.slopes is None and not self.pos_hook
 
     def matrices(self):
         return [self.w_qkv, self.w_out]
 
+    def product_shapes(self):
+        kv = 2 * self.kv_heads if self.source is None else 0
+        return [((self.heads + kv) * self.head_dim, self.hidden), (self.hidden, self.heads * self.head_dim)]
+
     def small_tensors(self):
-        return [t for t in (self.q_gain, self.k_gain, None if self.position is None else self.position.inv_freq)
-                if t is not None]   # of the cos/sin table a step reads one row per token: not counted
+        own = [t for t in (self.q_gain, self.k_gain, self.slopes) if t is not None]
+        return own + ([] if self.position is None else list(self.position.small_tensors()))
 
     def fold_input_gain(self, gain: torch.Tensor) -> None:
         """The preceding norm's gain, multiplied into the columns of the q, k, v projections."""
@@ -94,8 +117,15 @@ class AttentionMixer(Mixer):
         self.p_qkv = ops.PackedWeight(self.w_qkv)
         self.p_out = ops.PackedWeight(self.w_out)
 
+    def _rotation_args(self) -> dict:
+        """The rotation as the kernels take it (no rotation: nulls)."""
+        r = self.rot
+        if r is None:
+            return dict(inv_freq=None, rotary_dim=0, variant="half_split", cos_sin=None)
+        return dict(inv_freq=r.inv_freq, rotary_dim=r.rotary_dim, variant=r.variant, cos_sin=r.cos_sin)
+
     def can_decode_fused(self, batch) -> bool:
-        rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
+        rot_ok = self.fast_ok and (self.rot is None or self.rot.rotary_dim % 16 == 0)
         return (self.source is None and self.hidden % 8 == 0 and self.head_dim % 16 == 0 and self.head_dim <= 256
                 and rot_ok and (self.heads * self.head_dim) % 8 == 0)
 
@@ -109,13 +139,11 @@ class AttentionMixer(Mixer):
     def _attend_decoded(self, qkv, batch, cache) -> torch.Tensor:
         """A step of single decoded tokens, from the raw projection: one kernel norms and rotates q and
         the new key, writes key and value to their pages and attends."""
-        pos = self.position
         return ops.attention_decode_fused(
             qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages, cache.vpages,
             batch.tables[cache.group], batch.n_req, batch.pos, batch.row_req, self.scale, q_gain=self.q_gain,
-            k_gain=self.k_gain, eps=self.qk_norm_eps, inv_freq=None if pos is None else pos.inv_freq,
-            rotary_dim=0 if pos is None else pos.rotary_dim, variant="half_split" if pos is None else pos.variant,
-            window=self.window, max_seq=batch.max_seq, cos_sin=None if pos is None else pos.cos_sin)
+            k_gain=self.k_gain, eps=self.qk_norm_eps, window=self.window, max_seq=batch.max_seq,
+            **self._rotation_args())
 
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
@@ -123,19 +151,29 @@ class AttentionMixer(Mixer):
         qkv = linear(h, self.w_qkv)
         table = batch.tables[cache.group]
         owns = self.source is None
-        rot_ok = self.position is None or self.position.rotary_dim % 16 == 0
+        rot_ok = self.fast_ok and (self.rot is None or self.rot.rotary_dim % 16 == 0)
         if (owns and self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and self.head_dim % 16 == 0
                 and self.head_dim <= 256 and rot_ok):
             return linear(self._attend_decoded(qkv, batch, cache), self.w_out, partial_ok=True, packed=self.p_out)
-        pos = self.position
-        ops.qk_rope_kv(qkv, n, self.heads, self.kv_heads if owns else 0, self.head_dim,
-                       q_gain=self.q_gain, k_gain=self.k_gain, eps=self.qk_norm_eps,
-                       inv_freq=None if pos is None else pos.inv_freq,
-                       rotary_dim=0 if pos is None else pos.rotary_dim,
-                       variant="half_split" if pos is None else pos.variant,
-                       pos=batch.pos, row_req=batch.row_req,
-                       kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None,
-                       table=table, n_req=batch.n_req, cos_sin=None if pos is None else pos.cos_sin)
+        nkv = self.kv_heads if owns else 0
+        where = dict(pos=batch.pos, row_req=batch.row_req, table=table, n_req=batch.n_req)
+        pages = dict(kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None)
+        if self.pos_hook:
+            # q/k norm, then the encoding's own doing on the rows, then k and v into their pages
+            hd = self.head_dim
+            plain = dict(k_gain=None, eps=self.qk_norm_eps, **self._rotation_args(), **where)
+            k_rows = qkv[:, self.heads * hd:(self.heads + nkv) * hd]
+            if self.q_gain is not None:          # the kernel norms heads in place when it is given no pages
+                ops.qk_rope_kv(qkv, n, self.heads, 0, hd, q_gain=self.q_gain, kpages=None, vpages=None, **plain)
+            if owns and self.k_gain is not None:
+                ops.qk_rope_kv(k_rows, n, nkv, 0, hd, q_gain=self.k_gain, kpages=None, vpages=None, **plain)
+            self.position.apply(qkv[:, :self.heads * hd].unflatten(1, (self.heads, hd)),
+                                k_rows.unflatten(1, (nkv, hd)) if owns else None, batch)
+            if owns:
+                ops.qk_rope_kv(qkv, n, self.heads, nkv, hd, q_gain=None, **pages, **plain)
+        else:
+            ops.qk_rope_kv(qkv, n, self.heads, nkv, self.head_dim, q_gain=self.q_gain, k_gain=self.k_gain,
+                           eps=self.qk_norm_eps, **self._rotation_args(), **pages, **where)
         a = self.attend(qkv, batch, cache, table)
         return linear(a, self.w_out, partial_ok=True, packed=self.p_out)
 
@@ -144,7 +182,7 @@ class AttentionMixer(Mixer):
         tokens take the kernel that splits the keys, steps with prompt portions the matrix-core
         kernel (head sizes up to 128).  float32, and whatever the fast kernels do not take: the
         plain kernel."""
-        bf16 = self.rt.act_dtype == torch.bfloat16
+        bf16 = self.rt.act_dtype == torch.bfloat16 and self.slopes is None   # (the fast kernels take no score bias)
         if bf16 and batch.max_q > 1 and self.head_dim % 16 == 0 and self.head_dim <= 128:
             # decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that
             # splits their keys; a row of its own in the matrix-core kernel would walk its cache alone
@@ -163,4 +201,4 @@ class AttentionMixer(Mixer):
                                         self.window, max_seq=batch.max_seq)
         return ops.attention_plain(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
                                    cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
-                                   self.window)
+                                   self.window, slopes=self.slopes)

@@ -38,6 +38,10 @@ class Runtime:
     act_dtype: torch.dtype          # activations and cache pages: bfloat16, or float32 for the 32-bit path
     max_positions: int = 0          # positions a request can reach (tables over positions are sized by it); 0: unknown
     shared: Dict = field(default_factory=dict)   # what parts of one model derive once and share (tables)
+    # bfloat16 only: norm gains are multiplied into the matrices that read the normed rows, and steps of
+    # up to `fused_decode_rows` single decoded tokens take the parts' fused decode kernels (0: never)
+    fold_gains: bool = True
+    fused_decode_rows: int = 64
 
 
 @dataclass
@@ -63,6 +67,11 @@ class Part:
         has to stream, and 2 * numel flops per row)."""
         return []
 
+    def product_shapes(self) -> List[tuple]:
+        """(out, in) of the matrix products that every row of a step goes through, known from the
+        sizes alone (before any weights are bound)."""
+        return []
+
     def small_tensors(self) -> List[torch.Tensor]:
         """Gains, biases, taps and tables that a step also reads."""
         return []
@@ -85,9 +94,44 @@ class Norm(Part):
         raise NotImplementedError
 
 
+@dataclass
+class Rotation:
+    """A rotation of q and k by position that the attention kernels apply themselves."""
+    inv_freq: torch.Tensor                 # float32 [rotary_dim / 2]
+    rotary_dim: int
+    variant: str                           # "half_split": pairs (j, j + rotary_dim/2); "interleaved": pairs (2j, 2j+1)
+    cos_sin: Optional[torch.Tensor] = None  # [positions, rotary_dim / 2, 2] of the first positions, or None
+
+
 class PositionEncoding(Part):
+    """How positions enter an attention mixer.  An encoding answers in one (or more) of three ways,
+    and the mixer asks in this order:
+
+      rotation()        a `Rotation`: the kernels rotate q and k themselves (all fast paths stay open);
+      apply(q, k, batch)  anything else done to q and k in place before k is cached (the mixer then
+                        takes its general path: norm, this hook, cache write, attention);
+      score_slopes(heads)  float32 [heads]: slope[h] * (key position - query position) is added to the
+                        scores (a linear bias over the distance; the plain attention kernel takes it).
+
+    An encoding that answers none of them leaves q, k and the scores alone."""
+
     def __init__(self, spec: PositionSpec, head_dim: int):
         self.spec, self.head_dim = spec, head_dim
+
+    def rotation(self) -> Optional[Rotation]:
+        return None
+
+    def apply(self, q: torch.Tensor, k: Optional[torch.Tensor], batch) -> None:
+        """q: [N, heads, head_dim], k: [N, kv_heads, head_dim] (None for a mixer that reads another
+        layer's cache): views of the step's rows, after the q/k norm, changed in place.  `batch.pos`
+        holds every row's position."""
+
+    def score_slopes(self, heads: int) -> Optional[torch.Tensor]:
+        return None
+
+    def transforms_rows(self) -> bool:
+        """Whether `apply` does anything (the mixer skips the hook's extra passes otherwise)."""
+        return type(self).apply is not PositionEncoding.apply
 
 
 class Mixer(Part):
@@ -104,6 +148,11 @@ class Mixer(Part):
 
     def state_needs(self) -> Sequence[StateNeed]:
         return ()
+
+    def attention_flops(self, keys: float) -> float:
+        """Flops that grow with the keys the step's rows see (`keys`: their sum over the rows), beside
+        the matrix products: scores and weighted values of an attention; 0 for a mixer without."""
+        return 0.0
 
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         raise NotImplementedError

@@ -1,27 +1,31 @@
 """Arrangements of a layer's parts.
 
-`pre_norm` is LFM2's (/root/reference/arch/families/lfm2.json5:77-88):
+`pre_norm` is LFM2's (arch/families/lfm2.json5:77-88):
     x = x + mixer(norm(x));   x = x + ffn(norm(x))
 The residual stream x is float32.  On the general path each residual add is fused into the norm
 that follows it, so a block hands its last delta on instead of adding it.
 
 In bfloat16 the block folds each norm's gain into the matrices that read the normed rows (the
-reference's graph passes fold norm gains into weights too, /root/reference/src/graph/passes/mod.rs).
-A step of single decoded tokens (up to `FUSED_DECODE_ROWS` rows) then takes the parts' fused decode kernels: the
+reference's graph passes fold norm gains into weights too, src/graph/passes/mod.rs).
+A step of single decoded tokens (up to `Runtime.fused_decode_rows` rows, at most 64) then takes the parts' fused decode kernels: the
 product itself computes 1/rms of its input rows, and the last product of each half adds its result
 into the stream, so a half of a layer is two or three kernels.
 """
 from __future__ import annotations
-
-import os
 
 import torch
 
 from .. import ops
 from .base import Block, Runtime, Stream, register_arrangement
 
-# rows (decoded tokens) up to which a step takes the fused decode kernels; they take at most 64
-FUSED_DECODE_ROWS = min(64, int(os.environ.get("GIBBS_FUSED_DECODE_ROWS", "64")))
+# rows (decoded tokens) that the fused decode kernels take at most
+MAX_FUSED_DECODE_ROWS = 64
+
+
+def fused_decode_step(rt: Runtime, batch) -> bool:
+    """Whether this step (every row one decoded token, few enough of them) may take the fused decode kernels."""
+    return (rt.act_dtype == torch.bfloat16 and batch is not None and batch.max_q == 1
+            and batch.n_rows <= min(rt.fused_decode_rows, MAX_FUSED_DECODE_ROWS))
 
 
 @register_arrangement("pre_norm")
@@ -35,7 +39,7 @@ class PreNormBlock(Block):
             self.ffn.pack_matrices()
 
     def _fold(self, norm, part) -> bool:
-        if self.rt.act_dtype != torch.bfloat16 or os.environ.get("GIBBS_FOLD_GAINS", "1") == "0":
+        if self.rt.act_dtype != torch.bfloat16 or not self.rt.fold_gains:
             return False
         if not (hasattr(norm, "fold_gain") and hasattr(part, "fold_input_gain")):
             return False
@@ -52,8 +56,7 @@ class PreNormBlock(Block):
         return stream
 
     def _fused(self, part, folded: bool, batch, cache=None) -> bool:
-        return (folded and self.rt.act_dtype == torch.bfloat16 and batch is not None and batch.max_q == 1
-                and batch.n_rows <= FUSED_DECODE_ROWS and hasattr(part, "decode_fused")
+        return (folded and fused_decode_step(self.rt, batch) and hasattr(part, "decode_fused")
                 and part.can_decode_fused(batch))
 
     def forward(self, stream: Stream, batch, cache) -> Stream:

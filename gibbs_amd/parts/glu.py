@@ -1,5 +1,5 @@
-"""Dense gated feed-forward: down(act(gate(h)) * up(h)); with `activation: "silu"` this is
-SwiGLU (/root/reference/arch/lib/transformer.json5:117-130, /root/reference/src/graph/cpu.rs:378-390).
+"""Dense gated feed-forward: down(act(gate(h)) * up(h)), `activation` one of `ops.ACTIVATIONS`; with "silu" this is
+SwiGLU (arch/lib/transformer.json5:117-130, src/graph/cpu.rs:378-390).
 Gate and up are one product against [W_gate; W_up]."""
 from __future__ import annotations
 
@@ -37,6 +37,9 @@ class GluFeedForward(FeedForward):
     def matrices(self):
         return [self.w_gate_up, self.w_down]
 
+    def product_shapes(self):
+        return [(2 * self.inter, self.hidden), (self.hidden, self.inter)]
+
     def fold_input_gain(self, gain: torch.Tensor) -> None:
         """The preceding norm's gain, multiplied into the columns of the gate and up matrices."""
         self.w_gate_up = (self.w_gate_up.float() * gain[None, :]).to(self.w_gate_up.dtype)
@@ -50,7 +53,7 @@ class GluFeedForward(FeedForward):
 
     def decode_fused(self, stream, norm_eps: float, batch) -> None:
         """norm -> gate/up -> activation in one kernel, down + residual add in another."""
-        act = ops.skinny_glu(stream.mirror, self.p_gate_up or self.w_gate_up, rms_eps=norm_eps)
+        act = ops.skinny_glu(stream.mirror, self.p_gate_up or self.w_gate_up, rms_eps=norm_eps, activation=self.activation)
         ops.skinny_residual(act, self.p_down or self.w_down, stream.x, stream.mirror)
 
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:

@@ -1,6 +1,6 @@
 """A decoder put together from a `ModelSpec`: token table, blocks in the spec's run order, final
-norm and head (/root/reference/arch/families/lfm2.json5:66-95,
-/root/reference/arch/lib/transformer.json5:170-198).
+norm and head (arch/families/lfm2.json5:66-95,
+arch/lib/transformer.json5:170-198).
 
 Only the rows whose logits are wanted go through the final norm and the head: the gather comes
 before the norm, as in the reference's `last_row` (transformer.json5:177-192).
@@ -17,7 +17,7 @@ from ..config.spec import ModelSpec
 from ..ops.linear import linear
 from ..weights.loader import TensorDecl, WeightStore
 from .base import Block, Part, Runtime, Stream, build_block, build_norm
-from .block import FUSED_DECODE_ROWS
+from .block import fused_decode_step
 
 
 class DecoderModel(Part):
@@ -81,7 +81,7 @@ class DecoderModel(Part):
         run number `run` of the layer order); returns float32 logits [len(logit_rows), vocab]
         (None if no logits are wanted)."""
         mirror = None
-        if self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and batch.n_rows <= FUSED_DECODE_ROWS:
+        if fused_decode_step(self.rt, batch):
             # a step of decoded tokens: the fused kernels read the stream's bfloat16 mirror
             mirror = torch.empty((batch.n_rows, self.spec.hidden), dtype=torch.bfloat16, device=self.rt.device)
         stream = Stream(ops.embed(self.table, batch.ids, batch.n_rows, mirror=mirror), None, mirror)

@@ -1,6 +1,6 @@
 """RMSNorm: out = x * 1/sqrt(mean(x^2) + eps) * gain, eps inside the root, the gain multiplied
-last, no (1 + gain) offset (/root/reference/src/model/simd.rs:75-110,
-/root/reference/arch/lib/transformer.json5:9-11)."""
+last, no (1 + gain) offset (src/model/simd.rs:75-110,
+arch/lib/transformer.json5:9-11)."""
 from __future__ import annotations
 
 from typing import List, Optional

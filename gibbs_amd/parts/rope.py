@@ -2,9 +2,9 @@
 attention mixer hands to its kernel.
 
 inv_freq[j] = 1 / theta^(2j / rotary_dim); with `precision: "f32"` every step of that is a
-float32 operation, as LFM2's spec asks (/root/reference/src/arch/gen.rs:154-164,
-/root/reference/arch/families/lfm2.json5:64).  The angle of position p is float32(p) * inv_freq[j]
-(/root/reference/src/graph/cpu.rs:673); variant `half_split` turns the pair (j, j + rot/2),
+float32 operation, as LFM2's spec asks (src/arch/gen.rs:154-164,
+arch/families/lfm2.json5:64).  The angle of position p is float32(p) * inv_freq[j]
+(src/graph/cpu.rs:673); variant `half_split` turns the pair (j, j + rot/2),
 `interleaved` the pair (2j, 2j + 1) (:676-695).
 
 Cosine and sine of every angle up to the run's longest position are computed once, when the part is
@@ -18,7 +18,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import WeightStore
-from .base import PositionEncoding, Runtime, register_position
+from .base import PositionEncoding, Rotation, Runtime, register_position
 
 
 MAX_TABLE_POSITIONS = 1 << 20   # 8 bytes * rotary_dim / 2 each
@@ -57,3 +57,9 @@ class RotaryPosition(PositionEncoding):
             inv_freq = torch.from_numpy(rope_inv_freq(self.rotary_dim, self.theta, self.precision)).to(rt.device)
             rt.shared[key] = (inv_freq, ops.rope_table(inv_freq, n_pos) if n_pos > 0 else None)
         self.inv_freq, self.cos_sin = rt.shared[key]
+
+    def rotation(self) -> Rotation:
+        return Rotation(self.inv_freq, self.rotary_dim, self.variant, self.cos_sin)
+
+    def small_tensors(self):
+        return [self.inv_freq]      # of the cos/sin table a step reads one row per token: not counted

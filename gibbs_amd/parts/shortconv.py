@@ -1,9 +1,9 @@
-"""LFM2's gated short-convolution mixer (/root/reference/arch/lib/transformer.json5:138-151).
+"""Gated short-convolution mixer (the reference's `shortconv` block, arch/lib/transformer.json5:138-151).
 
 [B | C | x] = thirds of in_proj(h), in that order; bx = B * x; a depthwise causal convolution of
 length K over bx whose history is the request's state (the last K-1 rows of bx, oldest first,
-zeros at a sequence start; /root/reference/src/graph/cpu.rs:952-994); y = C * conv; out_proj(y).
-The reference refuses a convolution bias (/root/reference/arch/families/lfm2.json5:53); here
+zeros at a sequence start; src/graph/cpu.rs:952-994); y = C * conv; out_proj(y).
+The reference refuses a convolution bias (arch/families/lfm2.json5:53); here
 `bias: true` adds it after the tap sum.
 """
 from __future__ import annotations
@@ -28,7 +28,7 @@ class ShortConvMixer(Mixer):
         p = spec.params
         self.width, self.kernel, self.bias = int(p["width"]), int(p["kernel"]), bool(p.get("bias", False))
         if self.kernel < 2:
-            raise ValueError(f"LFM2 short-conv kernel (conv_L_cache) {self.kernel} must be >= 2")
+            raise ValueError(f"a short convolution needs a kernel of at least 2 taps, not {self.kernel}")
 
     def state_needs(self) -> Sequence[StateNeed]:
         return (StateNeed(STATE, (self.kernel - 1, self.width)),)
@@ -54,6 +54,9 @@ class ShortConvMixer(Mixer):
 
     def matrices(self):
         return [self.w_in, self.w_out]
+
+    def product_shapes(self):
+        return [(3 * self.width, self.hidden), (self.hidden, self.width)]
 
     def small_tensors(self):
         return [self.taps] + ([self.conv_bias] if self.bias else [])

@@ -1,6 +1,6 @@
 """What a step must at least move and compute, for the roofline figures of the bench and the
 command line (the reference reports decode speed against bytes-per-token at a bandwidth ceiling,
-/root/reference/src/bench.rs:298-308)."""
+src/bench.rs:298-308)."""
 from __future__ import annotations
 
 from typing import Sequence
@@ -8,6 +8,11 @@ from typing import Sequence
 # MI355X's published peaks.
 HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float16": 2.5e15, "float8": 5.0e15, "float32": 157.3e12}
+
+
+def torch_element_size(dtype) -> int:
+    import torch
+    return torch.empty((), dtype=dtype).element_size()
 
 
 def _nbytes(t) -> int:
@@ -31,10 +36,10 @@ def weight_bytes_per_step(engine) -> int:
 def cache_bytes(engine, seq_lens: Sequence[int]) -> int:
     """Keys and values that the live requests' next tokens attend over, and their state slots."""
     cm = engine.cache
-    elem = engine.device_cache.pages[0].element_size() if engine.device_cache.pages else 0
+    elem = torch_element_size(engine.device_cache.cache_dtype)
     total = 0
     for g, need in enumerate(cm.group_needs):
-        per_token = 2 * need.kv_heads * need.head_dim * elem * len(cm.group_layers[g])
+        per_token = need.kv_heads * (need.head_dim + need.value_dim) * elem * len(cm.group_layers[g])
         for n in seq_lens:
             total += per_token * (n if need.window is None else min(n, need.window))
     total += len(seq_lens) * cm.slot_floats * 4
@@ -55,9 +60,6 @@ def prefill_flops(engine, n_tokens: int, n_logit_rows: int = 1, start: int = 0) 
     for i in m.spec.order:
         b = m.blocks[i]
         flops += 2.0 * n_tokens * sum(t.numel() for t in b.matrices())
-        need = b.mixer.cache_need()
-        if need is not None or b.mixer.kv_source() is not None:
-            heads, hd = b.mixer.heads, b.mixer.head_dim
-            flops += 2.0 * 2.0 * keys * heads * hd
+        flops += b.mixer.attention_flops(keys)
     flops += 2.0 * n_logit_rows * m.head.numel()
     return flops

@@ -3,9 +3,9 @@ pure function of (seed, request key, index), so a fixed seed reproduces the toke
 runs beside the request and however often it was preempted and recomputed.
 
 The reference derives its draw from a hash of the recent tokens and the candidate set, without a
-seed (/root/reference/src/runtime/lm.rs:1126-1137); a seeded stream replaces that here.  The
+seed (src/runtime/lm.rs:1126-1137); a seeded stream replaces that here.  The
 mixer is SplitMix64, which the reference's device sampler also uses
-(/root/reference/src/graph/metal_kernels.metal:2369-2460).
+(src/graph/metal_kernels.metal:2369-2460).
 """
 from __future__ import annotations
 

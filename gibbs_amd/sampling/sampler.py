@@ -1,7 +1,7 @@
 """Greedy and temperature sampling on the device, with the reference's pipeline and defaults:
 temperature <= 1e-4 is the first maximum; else top-k (50, at most 64) by (logit descending, id
 ascending), softmax at the temperature, the shortest prefix reaching top_p, and a draw
-(/root/reference/src/runtime/lm.rs:1043-1240, /root/reference/src/scheduler/mod.rs:171-178,
+(src/runtime/lm.rs:1043-1240, src/scheduler/mod.rs:171-178,
 :335-339).  The reference's sampler also takes a repetition penalty over the last 64 tokens
 (lm.rs:1084-1105, :1163-1189), which its scheduler leaves at 1.0 (scheduler/mod.rs:178); here it is
 a per-request parameter with the same default."""

@@ -1,11 +1,11 @@
 """Text in and out of a model folder: tokenizer.json through the `tokenizers` package, the model's own
 chat template, the ids that end generation and the folder's sampling defaults.
 
-What the reference's tokenizer does on the request path (/root/reference/src/model/tokenizer/mod.rs):
+What the reference's tokenizer does on the request path (src/model/tokenizer/mod.rs):
 `encode` runs tokenizer.json's pipeline without adding special tokens and then prepends the
 model-declared BOS unless the text already starts with it (:719-737), so a prompt rendered by a chat
 template that writes `bos_token` gets exactly one; a one-shot prompt is rendered as a single user
-message when the folder declares a template (/root/reference/src/scheduler/mod.rs:1094-1097);
+message when the folder declares a template (src/scheduler/mod.rs:1094-1097);
 generation ends at the `eos_token_id`(s) of generation_config.json and at special tokens
 (tokenizer/mod.rs:710-717); generation_config.json's temperature and top_p stand in for values a
 request leaves unset, with `do_sample: false` meaning greedy (:25-27).

@@ -3,12 +3,12 @@
 Every part of a model declares the tensors it reads (`TensorDecl`).  Loading compares the
 declarations with the checkpoint's table and fails once, listing every missing tensor,
 every tensor nobody reads, and every wrong shape: the reference refuses unread checkpoint
-tensors (/root/reference/src/runtime/lm.rs:357-367) and missing ones
-(/root/reference/src/arch/build.rs:454-457) separately.
+tensors (src/runtime/lm.rs:357-367) and missing ones
+(src/arch/build.rs:454-457) separately.
 
 Precision policy: floating matrices are kept in the compute dtype of the run (bfloat16, or
 float32 for the true 32-bit path); tensors of rank <= 1 (gains, biases) are float32, as in
-the reference (/root/reference/src/arch/load.rs:902-917); a declaration can pin float32 for
+the reference (src/arch/load.rs:902-917); a declaration can pin float32 for
 a tensor whatever its rank; integer tables become int32.
 """
 from __future__ import annotations

@@ -3,7 +3,7 @@ configuration and a seed.
 
 Every tensor has its own stream seeded by hash(name) ^ seed, so values do not depend on the
 order tensors are written in: the idea of the reference's synthetic checkpoints
-(/root/reference/src/arch/load.rs:2355-2420, per-name seed :1410), with a normal
+(src/arch/load.rs:2355-2420, per-name seed :1410), with a normal
 distribution of standard deviation 0.02 instead of its uniform +-0.02.
 """
 from __future__ import annotations

@@ -1,9 +1,9 @@
 """Reading and writing safetensors files without touching tensor data until it is asked for.
 
-Layout (/root/reference/src/model/loaders/safetensors.rs:15-64): an unsigned 64-bit
+Layout (src/model/loaders/safetensors.rs:15-64): an unsigned 64-bit
 little-endian header length, a JSON header {name: {dtype, shape, data_offsets}}, then the
 data.  Sharded checkpoints name their files in `model.safetensors.index.json`
-(/root/reference/src/arch/load.rs:365).
+(src/arch/load.rs:365).
 """
 from __future__ import annotations
 

@@ -15,7 +15,10 @@ import os
 import numpy as np
 
 MASK = (1 << 64) - 1
-GOLDEN_JSON = "/root/reference/tests/golden/lm_graphlm_lfm2.json"
+# the reference's checkout, if there is one here: $GIBBS_REFERENCE, else a `reference` folder beside the repository
+REFERENCE = os.environ.get("GIBBS_REFERENCE") or os.path.join(
+    os.path.dirname(os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))), "reference")
+GOLDEN_JSON = os.path.join(REFERENCE, "tests", "golden", "lm_graphlm_lfm2.json")
 GOLDEN_NPZ = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden_lfm2_expected.npz")
 
 PROMPT = [5, 17, 42, 99, 133, 200]            # tests/golden/lm.rs:13

@@ -5,7 +5,7 @@ import random
 import numpy as np
 import pytest
 
-from gibbs_amd.cache import NO_PAGE, CacheManager, CacheNeed, PageError, PagePool, StateNeed
+from gibbs_amd.cache import NO_PAGE, CacheManager, CacheNeed, PageError, StateNeed, host
 
 FULL = CacheNeed(2, 16)
 WIN = CacheNeed(2, 16, window=40)
@@ -14,6 +14,30 @@ WIN = CacheNeed(2, 16, window=40)
 def manager(needs=(None, FULL, None, FULL), pages=12, reqs=3, ps=16):
     states = [(StateNeed("conv", (2, 8)),) if n is None else () for n in needs]
     return CacheManager(list(needs), states, ps, pages, reqs)
+
+
+class PagePool:
+    """A handle on one pool of the native core (the cache manager holds one per group)."""
+
+    def __init__(self, num_pages: int):
+        self.lib, self.num_pages = host.library(), num_pages
+        self.pool = self.lib.gibbs_pool_create(num_pages)
+
+    def __del__(self):
+        self.lib.gibbs_pool_destroy(self.pool)
+
+    @property
+    def n_free(self) -> int:
+        return self.lib.gibbs_pool_free(self.pool)
+
+    def allocate(self, n: int):
+        out = host.ints([0] * n)
+        return None if self.lib.gibbs_pool_allocate(self.pool, n, out) < 0 else list(out[:n])
+
+    def release(self, pages) -> None:
+        pages = list(pages)
+        if self.lib.gibbs_pool_release(self.pool, host.ints(pages), len(pages)) < 0:
+            raise PageError(host.last_error())
 
 
 def test_pool_basics():
@@ -89,6 +113,41 @@ def test_window_group_returns_passed_pages():
     assert 20 - m.free_pages(1) == m.pages_for(103), "the full group keeps every page"
     m.release("a")
     assert m.free_pages(0) == m.free_pages(1) == 20
+
+
+def test_groups_with_pools_of_their_own_size():
+    """A group with a window does with a pool much smaller than the group that keeps every key; keys and
+    values with different head sizes are a need of their own."""
+    m = CacheManager([FULL, WIN, FULL], [(), (), ()], 16, [40, 6], 2)
+    assert [p.num_pages for p in m.pools] == [40, 6] and m.group_layers == [[0, 2], [1]]
+    m.admit("a")
+    for n in [30, 20, 1, 40, 40, 1, 33]:          # 165 tokens: 11 pages of the full group, never more than 6 of the window's
+        assert m.reserve("a", n), f"the window group ran out at {m.tokens('a')} + {n} tokens"
+        assert m.free_pages(1) >= 0
+        m.commit("a", n)
+        m.check()
+    assert 40 - m.free_pages(0) == m.pages_for(165) and 6 - m.free_pages(1) <= 40 // 16 + 2
+    assert not m.reserve("a", 16 * 5), "a portion that the small pool cannot hold beside the window is refused"
+    assert m.free_pages(1) == 6 - (m.pages_for(165) - (165 - 40 + 1) // 16) and m.tokens("a") == 165
+    m.release("a")
+    assert (m.free_pages(0), m.free_pages(1)) == (40, 6)
+    with pytest.raises(ValueError, match="page counts"):
+        CacheManager([FULL, WIN], [(), ()], 16, [40], 2)
+    wide_values = CacheNeed(2, 16, v_head_dim=24)
+    assert wide_values != FULL and wide_values.value_dim == 24 and FULL.value_dim == 16
+    m = CacheManager([FULL, wide_values, FULL], [(), (), ()], 16, 8, 2)
+    assert m.group_needs == [FULL, wide_values] and m.group_layers == [[0, 2], [1]]
+
+
+def test_a_slot_given_back_before_any_step_is_listed_once():
+    """Admission that is undone (the scheduler tries the head of its queue and finds no room) must not
+    pile the slot up among the fresh ones: every fresh slot is reported, each once."""
+    m = manager(reqs=3)
+    for i in range(10):
+        assert m.admit(("try", i))
+        m.release(("try", i))
+    assert m.admit("a") and m.admit("b") and m.admit("c")
+    assert sorted(m.take_fresh_slots()) == [0, 1, 2] and m.take_fresh_slots() == []
 
 
 @pytest.mark.parametrize("seed", range(8))

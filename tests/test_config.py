@@ -50,6 +50,10 @@ def test_layer_kinds():
                "lm_head.weight": (77, 64)}
     c = Lfm2Config.from_dict({**BASE, "layer_types": None}, tensors)
     assert c.layer_types == ("full_attention", "conv") and c.vocab_size == 77 and not c.tie_embedding
+    # config.json names the kinds and the checkpoint holds other layers: one error that names them
+    with pytest.raises(ConfigError, match=r"disagree about the kind of layers \[0, 1\].*'conv', 'full_attention'.*'full_attention', 'conv'"):
+        Lfm2Config.from_dict(BASE, tensors)
+    assert Lfm2Config.from_dict({**BASE, "layer_types": ["full_attention", "conv"]}, tensors).layer_types == c.layer_types
 
 
 def test_refusals():

@@ -109,17 +109,20 @@ def test_reference_golden_vector_through_the_engine(dirs, dtype):
     from gibbs_amd import Engine, Entry, generate
     exp = G.golden_expected()
     eng = Engine(dirs["golden"], dtype=dtype, max_tokens=256, max_requests=2)
-    rel, cos = (1e-3, 0.9999) if dtype == "float32" else (1.0, 0.999)
+    # (bfloat16: 1.5 x the measured relative L2 error of this small model, 3.2 %)
+    rel, cos = (1e-3, 0.9999) if dtype == "float32" else (4.8e-2, 0.999)
     def last(rid, ids):
         out = eng.step([Entry(rid, ids, [len(ids) - 1])]).cpu().numpy()[0]
         return out
     for name, ids in (("prefill6", G.PROMPT), ("prefill20", G.LONG_PROMPT)):
         got = last(name, ids)
+        H._record(f"golden {name}", "golden", dtype, float(G.rel_l2(got, exp["f32"][name])), float(G.cosine(got, exp["f32"][name])), 0.0)
         assert G.rel_l2(got, exp["f32"][name]) < rel and G.cosine(got, exp["f32"][name]) > cos, name
         eng.release(name)
     last("d", G.PROMPT)
     for i, t in enumerate(G.DECODE):                                    # cached decode of forced tokens
         got = last("d", [t])
+        H._record(f"golden decode{i}", "golden", dtype, float(G.rel_l2(got, exp["f32"][f"decode{i}"])), float(G.cosine(got, exp["f32"][f"decode{i}"])), 0.0)
         assert G.rel_l2(got, exp["f32"][f"decode{i}"]) < rel and G.cosine(got, exp["f32"][f"decode{i}"]) > cos
     eng.release("d")
     if dtype == "float32":

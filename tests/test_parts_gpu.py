@@ -169,7 +169,7 @@ def test_glu_part(name, dtype):
     y = y.sum(0) if y.dim() == 3 else y
     close(y.float().cpu().numpy(), P.swiglu_ffn(h, w["w1"], w["w3"], w["w2"]), name, "glu part")
     with pytest.raises(ValueError, match="activation"):
-        build_feed_forward(FeedForwardSpec("glu", {"inter": 8, "activation": "relu"}, {}), 8)
+        build_feed_forward(FeedForwardSpec("glu", {"inter": 8, "activation": "softsign"}, {}), 8)
     with pytest.raises(KeyError, match="no feed-forward of kind"):
         build_feed_forward(FeedForwardSpec("experts", {}, {}), 8)
 
@@ -377,9 +377,10 @@ def window_spec(hidden=40, vocab=83, window=20):
 @pytest.mark.parametrize("name,dtype", DTYPES)
 def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
     """A model whose layers need different caches: all keys in one group, a window of 20 in another.
-    Three requests through the engine, portions beside decoded tokens, in a pool of 24 pages of 8
-    tokens per group: the window group hands out 29 pages over the run, so pages that a window has
-    passed are in use again while their first owner still runs; the logits equal the plain model's."""
+    Three requests through the engine, portions beside decoded tokens, in pools of 8-token pages of
+    different sizes: 24 pages for the group that keeps every key, 12 for the window's group, which hands
+    out 29 pages over the run, so pages that a window has passed are in use again while their first
+    owner still runs; the logits equal the plain model's."""
     from gibbs_amd import Engine, Entry
     from gibbs_amd.config.base import ArchConfig
     from gibbs_amd.parts import DecoderModel
@@ -392,9 +393,11 @@ def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
         def model_spec(self):
             return spec
     ws = store({k: v.float().numpy() for k, v in tensors.items()}, decls, dtype)
-    eng = Engine(config=Windowed(), weights=ws, dtype=name, max_tokens=24 * 8, max_requests=2, page_size=8)
+    eng = Engine(config=Windowed(), weights=ws, dtype=name, max_tokens=24 * 8, max_requests=2, page_size=8,
+                 group_pages=[24, 12])
     cm = eng.cache
     assert cm.n_groups == 2 and cm.group_layers == [[0], [1]]
+    assert [t.shape[1] for t in eng.device_cache.kpages] == [24, 12], "every group has the pages of its own pool"
     win = 1                                                     # the window's group
     seqs = {"a": H.tokens(1, 150, spec.vocab), "b": H.tokens(2, 40, spec.vocab), "c": H.tokens(3, 40, spec.vocab)}
     plain = {r: plain_spec_forward(spec, {k: v.double().numpy() for k, v in tensors.items()}, ids) for r, ids in seqs.items()}
@@ -427,7 +430,7 @@ def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
     for _ in range(7):
         step([("a", 1), ("c", 1)])                              # c ends
     step([("a", 150 - at["a"])])
-    assert not any(r in cm for r in seqs) and all(cm.free_pages(g) == 24 for g in range(2))
+    assert not any(r in cm for r in seqs) and [cm.free_pages(g) for g in range(2)] == [24, 12]
     assert used_again >= 5, "the pool was meant to be so small that pages a window has passed are used again"
     for r in seqs:
         H.assert_close(np.concatenate(got[r]), plain[r], name, f"windowed model request {r}")
@@ -576,7 +579,7 @@ def register_toy_routed():
     tensor code and are registered from here."""
     from gibbs_amd import ops
     from gibbs_amd.ops.linear import linear
-    from gibbs_amd.parts import FeedForward, PositionEncoding, register_feed_forward, register_position
+    from gibbs_amd.parts import FeedForward, PositionEncoding, Rotation, register_feed_forward, register_position
     from gibbs_amd.weights import TensorDecl
 
     @register_feed_forward("toy_routed")
@@ -610,14 +613,17 @@ def register_toy_routed():
 
     @register_position("toy_stretched_rope")
     class StretchedRope(PositionEncoding):
-        """Pairs (2j, 2j + 1) turned by pos / stretch * theta^(-2j/dim): the attention mixer's kernels
-        take the table of inverse frequencies, the pairing and the cos/sin table from this object."""
+        """Pairs (2j, 2j + 1) turned by pos / stretch * theta^(-2j/dim): a rotation, which the attention
+        mixer's kernels apply themselves from the tables that `rotation()` hands over."""
         def bind(self, weights, rt):
             p = self.spec.params
-            self.rt, self.rotary_dim, self.variant = rt, self.head_dim, "interleaved"
+            self.rt = rt
             inv = np.array([p["theta"] ** (-2.0 * j / self.head_dim) / p["stretch"] for j in range(self.head_dim // 2)])
             self.inv_freq = torch.tensor(inv, dtype=torch.float32, device=rt.device)
             self.cos_sin = ops.rope_table(self.inv_freq, rt.max_positions) if rt.max_positions > 0 else None
+
+        def rotation(self):
+            return Rotation(self.inv_freq, self.head_dim, "interleaved", self.cos_sin)
 
 
 def routed_config_class():
@@ -731,3 +737,197 @@ def test_toy_routed_feed_forward_and_position_encoding(name, dtype, tmp_path):
     for a, b in [(0, 11), (11, 13), (13, 14), (14, 15), (15, 37), (37, 38), (38, 39), (39, 40)]:
         got.append(eng.step([Entry("r", ids[a:b], list(range(b - a)))]).cpu().numpy())
     H.assert_close(np.concatenate(got), want, name, "toy routed feed-forward, stretched positions")
+
+
+# --------------------------------------------------------------------------- positions that are no rotation, values wider than keys, other activations
+def register_toy_positions_and_wide_values():
+    """Two position encodings that are no rotation (a linear bias on the scores by distance; a learned
+    vector per position added to q and k), and an attention mixer of the test's own whose values have
+    another head size than its keys and whose pages it reads and writes with plain tensor code.  All
+    registered from here; the framework's attention mixer, cache manager and kernels take them as they are."""
+    from gibbs_amd.cache import CacheNeed
+    from gibbs_amd.ops.linear import linear
+    from gibbs_amd.parts import Mixer, PositionEncoding, register_mixer, register_position
+    from gibbs_amd.weights import TensorDecl
+    from gibbs_amd.weights.loader import FLOAT32
+
+    @register_position("toy_distance_bias")
+    class DistanceBias(PositionEncoding):
+        """score(q at p, key at k) += slope_h * (k - p), slope_h = base^-(h + 1)."""
+        def score_slopes(self, heads):
+            base = float(self.spec.params["base"])
+            return torch.tensor([base ** -(h + 1) for h in range(heads)], dtype=torch.float32, device=self.rt.device)
+
+    @register_position("toy_learned_offsets")
+    class LearnedOffsets(PositionEncoding):
+        """q and k of position p get row p of a learned table [positions, head_dim] added (every head the same)."""
+        def tensor_decls(self):
+            return [TensorDecl(self.spec.tensors["table"], (self.spec.params["positions"], self.head_dim), FLOAT32)]
+
+        def bind(self, weights, rt):
+            self.rt, self.table = rt, weights[self.spec.tensors["table"]]
+
+        def apply(self, q, k, batch):
+            rows = self.table[batch.pos[:q.shape[0]].long()].to(q.dtype)[:, None, :]
+            q += rows
+            if k is not None:
+                k += rows
+
+    @register_mixer("toy_wide_values")
+    class WideValues(Mixer):
+        """Causal attention without position encoding, keys of `head_dim`, values of `v_head_dim`."""
+        def __init__(self, spec, hidden, layer_index):
+            super().__init__(spec, hidden, layer_index)
+            p = spec.params
+            self.heads, self.hd, self.vd = p["heads"], p["head_dim"], p["v_head_dim"]
+
+        def cache_need(self):
+            return CacheNeed(self.heads, self.hd, v_head_dim=self.vd)
+
+        def tensor_decls(self):
+            t, n = self.spec.tensors, self.heads
+            return [TensorDecl(t["q"], (n * self.hd, self.hidden)), TensorDecl(t["k"], (n * self.hd, self.hidden)),
+                    TensorDecl(t["v"], (n * self.vd, self.hidden)), TensorDecl(t["o"], (self.hidden, n * self.vd))]
+
+        def bind(self, weights, rt):
+            self.rt = rt
+            self.w = {r: weights[self.spec.tensors[r]] for r in "qkvo"}
+
+        def forward(self, h, batch, cache):
+            n, ps = self.heads, cache.kpages.shape[2]
+            assert cache.kpages.shape[3] == self.hd and cache.vpages.shape[3] == self.vd
+            q = linear(h, self.w["q"]).unflatten(1, (n, self.hd))
+            k = linear(h, self.w["k"]).unflatten(1, (n, self.hd))
+            v = linear(h, self.w["v"]).unflatten(1, (n, self.vd))
+            table = batch.tables[cache.group]
+            out = torch.empty((h.shape[0], n, self.vd), dtype=torch.float32, device=h.device)
+            row = 0
+            for r, (q_len, ctx) in enumerate(zip(batch.q_lens, batch.ctx_lens)):
+                pos = torch.arange(ctx, ctx + q_len, device=h.device)
+                pages = table[r, pos // ps].long()
+                cache.kpages[pages, :, pos % ps] = k[row:row + q_len]
+                cache.vpages[pages, :, pos % ps] = v[row:row + q_len]
+                held = table[r, :-(-(ctx + q_len) // ps)].long()
+                keys = cache.kpages[held].transpose(1, 2).reshape(-1, n, self.hd)[:ctx + q_len].float()
+                vals = cache.vpages[held].transpose(1, 2).reshape(-1, n, self.vd)[:ctx + q_len].float()
+                s = torch.einsum("thd,lhd->htl", q[row:row + q_len].float(), keys) * self.hd ** -0.5
+                s = s.masked_fill(torch.arange(ctx + q_len, device=h.device)[None, None, :] > pos[None, :, None], -torch.inf)
+                out[row:row + q_len] = torch.einsum("htl,lhd->thd", s.softmax(-1), vals)
+                row += q_len
+            return linear(out.flatten(1).to(self.rt.act_dtype).contiguous(), self.w["o"])
+
+
+def wide_config_class():
+    from gibbs_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                  register_architecture)
+    from gibbs_amd.config.base import ArchConfig
+
+    class WideConfig(ArchConfig):
+        architecture = "ToyWideForCausalLM"
+
+        def __init__(self, cfg):
+            self.cfg = dict(cfg)
+
+        @classmethod
+        def from_dict(cls, cfg, tensors=None):
+            return cls(cfg)
+
+        def to_dict(self):
+            return dict(self.cfg)
+
+        def model_spec(self):
+            c, layers = self.cfg, []
+            H_, hd = c["width"], c["head_size"]
+            attn = {"heads": c["heads"], "kv_heads": c["kv_heads"], "head_dim": hd, "scale": hd ** -0.5,
+                    "qk_norm": "before", "qk_norm_eps": c["eps"], "window": None}
+            for i, kind in enumerate(c["mixers"]):
+                p = f"l.{i}"
+                names = {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o",
+                         "q_norm": f"{p}.qn", "k_norm": f"{p}.kn"}
+                if kind == "bias":
+                    mixer = MixerSpec("attention", attn, names, PositionSpec("toy_distance_bias", {"base": c["slope_base"]}))
+                elif kind == "learned":
+                    mixer = MixerSpec("attention", attn, names,
+                                      PositionSpec("toy_learned_offsets", {"positions": c["max_len"]}, {"table": f"{p}.pos"}))
+                else:
+                    mixer = MixerSpec("toy_wide_values", {"heads": c["heads"], "head_dim": hd, "v_head_dim": c["v_head_size"]},
+                                      {"q": f"{p}.q", "k": f"{p}.k", "v": f"{p}.v", "o": f"{p}.o"})
+                ffn = FeedForwardSpec("glu", {"inter": c["ff"], "activation": c["activations"][i]},
+                                      {"gate": f"{p}.g", "up": f"{p}.u", "down": f"{p}.d"})
+                layers.append(LayerSpec(p, "pre_norm", NormSpec("rms", c["eps"], f"{p}.n1"), mixer,
+                                        NormSpec("rms", c["eps"], f"{p}.n2"), ffn))
+            return ModelSpec(self.architecture, H_, c["vocab"], tuple(layers), tuple(range(len(layers))), "tok",
+                             NormSpec("rms", c["eps"], "out_norm"), None, c["max_len"])
+    register_architecture("ToyWideForCausalLM", WideConfig, aliases=("toy_wide",))
+    return WideConfig
+
+
+def wide_plain(cfg, w, ids):
+    T, hd, vd, nh, nkv = len(ids), cfg["head_size"], cfg["v_head_size"], cfg["heads"], cfg["kv_heads"]
+    acts = {"silu": lambda g: g / (1 + np.exp(-g)), "relu": lambda g: np.maximum(g, 0.0),
+            "gelu_tanh": lambda g: 0.5 * g * (1 + np.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3))),
+            "gelu": lambda g: 0.5 * g * (1 + np.vectorize(math.erf)(g / math.sqrt(2)))}
+    x = P.embedding(w["tok"], ids)
+    for i, kind in enumerate(cfg["mixers"]):
+        p = f"l.{i}"
+        h = P.rms_norm(x, w[f"{p}.n1"], cfg["eps"])
+        if kind == "wide":
+            q, k = (P.linear(h, w[f"{p}.{r}"]).reshape(T, nh, hd) for r in "qk")
+            v = P.linear(h, w[f"{p}.v"]).reshape(T, nh, vd)
+            a = P.causal_attention(q, k, v, hd ** -0.5).reshape(T, nh * vd)
+        else:
+            q = P.rms_norm(P.linear(h, w[f"{p}.q"]).reshape(T, nh, hd), w[f"{p}.qn"], cfg["eps"])
+            k = P.rms_norm(P.linear(h, w[f"{p}.k"]).reshape(T, nkv, hd), w[f"{p}.kn"], cfg["eps"])
+            v = P.linear(h, w[f"{p}.v"]).reshape(T, nkv, hd)
+            if kind == "learned":
+                q, k = q + w[f"{p}.pos"][:T, None, :], k + w[f"{p}.pos"][:T, None, :]
+                a = P.causal_attention(q, k, v, hd ** -0.5)
+            else:   # scores biased by the distance
+                a = np.zeros((T, nh, hd))
+                for t in range(T):
+                    for hh in range(nh):
+                        g = hh // (nh // nkv)
+                        s = (k[:t + 1, g] @ q[t, hh]) * hd ** -0.5 + cfg["slope_base"] ** -(hh + 1) * (np.arange(t + 1) - t)
+                        e = np.exp(s - s.max())
+                        a[t, hh] = (e / e.sum()) @ v[:t + 1, g]
+            a = a.reshape(T, nh * hd)
+        x = x + P.linear(a, w[f"{p}.o"])
+        h = P.rms_norm(x, w[f"{p}.n2"], cfg["eps"])
+        x = x + P.linear(acts[cfg["activations"][i]](P.linear(h, w[f"{p}.g"])) * P.linear(h, w[f"{p}.u"]), w[f"{p}.d"])
+    return P.linear(P.rms_norm(x, w["out_norm"], cfg["eps"]), w["tok"])
+
+
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_positions_that_are_no_rotation_and_values_wider_than_keys(name, dtype, tmp_path):
+    """The attention mixer with a position encoding that biases the scores by distance and with one that
+    changes q and k itself (a learned table of its own in the checkpoint), a mixer from outside whose
+    cache group has values of another head size than keys, and feed-forwards with three other
+    activations (general path and the fused decode epilogue): registered, built from config.json and
+    stepped in portions and single tokens of two requests, against a plain implementation."""
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import write_random_model
+    register_toy_positions_and_wide_values()
+    Wide = wide_config_class()
+    cfg = {"architectures": ["ToyWideForCausalLM"], "width": 64, "heads": 4, "kv_heads": 2, "head_size": 16,
+           "v_head_size": 24, "ff": 96, "vocab": 77, "mixers": ["bias", "wide", "learned", "bias"],
+           "activations": ["gelu_tanh", "relu", "gelu", "silu"], "slope_base": 1.6, "eps": 1e-5, "max_len": 96}
+    folder = str(tmp_path / "wide")
+    config = Wide.from_dict(cfg)
+    write_random_model(folder, config, DecoderModel(config.model_spec()).tensor_decls(), seed=4, std=0.2, gain_std=0.2)
+    eng = Engine(folder, dtype=name, max_tokens=160, max_requests=2, page_size=8)
+    needs = eng.cache.group_needs
+    assert len(needs) == 2 and {n.value_dim for n in needs} == {16, 24}, "values of another head size are a group of their own"
+    assert [tuple(t.shape[-2:]) for t in eng.device_cache.vpages] == [(8, n.value_dim) for n in needs]
+    weights, _ = P.load_model_dir(folder)
+    seqs = {"a": H.tokens(5, 41, 77), "b": H.tokens(6, 23, 77)}
+    plan = [[("a", 0, 9)], [("a", 9, 10), ("b", 0, 13)], [("a", 10, 11), ("b", 13, 14)], [("a", 11, 12), ("b", 14, 15)],
+            [("a", 12, 35), ("b", 15, 16)], [("a", 35, 36), ("b", 16, 23)]] + [[("a", t, t + 1)] for t in range(36, 41)]
+    got = {}
+    for step in plan:
+        out = eng.step([Entry(r, seqs[r][a:b], list(range(b - a))) for r, a, b in step]).cpu().numpy()
+        at = 0
+        for r, a, b in step:
+            got.setdefault(r, []).append(out[at:at + b - a]); at += b - a
+    for r, ids in seqs.items():
+        H.assert_close(np.concatenate(got[r]), wide_plain(cfg, weights, ids), name, f"toy positions / wide values request {r}")

@@ -1,5 +1,5 @@
 """The scheduler's decisions, with a fake step function (no GPU).  The policy tests follow the
-reference's (/root/reference/src/scheduler/mod.rs:1635-1737, :1873-1931); what happens when pages
+reference's (src/scheduler/mod.rs:1635-1737, :1873-1931); what happens when pages
 run out is this engine's own decision."""
 import pytest
 
@@ -271,7 +271,7 @@ def test_random_workloads_always_finish_with_the_tokens_of_a_run_alone():
 
 
 def test_prefill_tuner_budgets():
-    """The reference's numbers (/root/reference/src/scheduler/mod.rs:341-403): 64 before anything is
+    """The reference's numbers (src/scheduler/mod.rs:341-403): 64 before anything is
     timed; one token while requests decode and no decode round has been timed; then the tokens that
     cost one decode round, or 100 ms when nothing decodes; at most 2,048; averages move by a quarter."""
     from gibbs_amd.engine.scheduler import PrefillTuner
