@@ -19,7 +19,7 @@ def parser() -> argparse.ArgumentParser:
     ap.add_argument("--prompt", help="text prompt (needs tokenizer.json in the model folder)")
     ap.add_argument("--prompt-ids", help="prompt as comma-separated token ids")
     ap.add_argument("--max-tokens", type=int, default=None, help="most new tokens (default 64)")
-    ap.add_argument("--ctx", type=int, default=None, help="context limit (default: max_position_embeddings)")
+    ap.add_argument("--ctx", type=int, default=None, help="context limit (default: max_position_embeddings, at most 4096)")
     ap.add_argument("--backend", default="auto", help="auto | rocm | hip (cpu is refused: there is no CPU path)")
     ap.add_argument("--seed", type=int, default=0, help="sampling seed (and the seed of --random-weights)")
     ap.add_argument("--arch", help="load --model as this architecture, skipping detection")

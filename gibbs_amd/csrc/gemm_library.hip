@@ -25,10 +25,25 @@ struct Plan {
   hipblasLtMatrixLayout_t w = nullptr, a = nullptr, c = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
+  bool timed = false;          // the algorithm was chosen by timing: such plans are kept
+  unsigned long last_use = 0;
+
+  void destroy() {
+    if (desc) hipblasLtMatmulDescDestroy(desc);
+    for (hipblasLtMatrixLayout_t l : {w, a, c})
+      if (l) hipblasLtMatrixLayoutDestroy(l);
+    desc = nullptr;
+    w = a = c = nullptr;
+  }
 };
 constexpr size_t WORKSPACE_BYTES = 64u << 20;   // what the heuristic may count on (stream-K kernels use some)
 constexpr size_t FLUSH_BYTES = 320u << 20;      // copies of a weight matrix: more than L2 and the memory-side cache hold
 constexpr int CANDIDATES = 24;
+// Plans are kept per exact shape, and a scheduler that cuts prompts under a measured budget brings steps of
+// any number of rows: beyond this many, the plan that was used longest ago goes (its descriptors are freed).
+constexpr size_t MAX_PLANS = 192;
+unsigned long use_clock = 0;
+long timings_done = 0;
 hipblasLtHandle_t handle = nullptr;
 void* workspace = nullptr;
 void* flush = nullptr;                          // allocated when the first shape is timed, kept
@@ -115,6 +130,8 @@ int make_plan(Plan& p, int N, int O, int I, long lda, long ldw, long ldc, const 
   if (timed && n_found > 1) {
     const int best = fastest(p, found, n_found, A, W, C, (size_t)O * ldw * sizeof(bf16), stream);
     if (best >= 0) pick = best;
+    p.timed = true;
+    ++timings_done;
   }
   p.algo = found[pick].algo;
   p.workspace = found[pick].workspaceSize;
@@ -137,6 +154,11 @@ GIBBS_EXPORT int gibbs_gemm_library_init() {
   return 0;
 }
 
+// How many shapes have had their algorithm chosen by timing so far (a step during which this number
+// grows took longer than its like will: whoever times steps leaves it out), and how many plans are kept.
+GIBBS_EXPORT long gibbs_gemm_library_timings() { return timings_done; }
+GIBBS_EXPORT long gibbs_gemm_library_plans() { return (long)plans.size(); }
+
 // A: [N, I] bfloat16 (row stride lda), W: [O, I] bfloat16 (row stride ldw), C: [N, O] bfloat16 (row stride ldc).
 GIBBS_EXPORT int gibbs_gemm_library(const void* A, const void* W, void* C, int N, int O, int I, long lda, long ldw,
                                     long ldc, hipStream_t stream) {
@@ -149,11 +171,24 @@ GIBBS_EXPORT int gibbs_gemm_library(const void* A, const void* W, void* C, int N
     const auto key = std::make_tuple(N, O, I, lda, ldw, ldc);
     auto it = plans.find(key);
     if (it == plans.end()) {
+      if (plans.size() >= MAX_PLANS) {
+        auto oldest = plans.end();
+        for (auto j = plans.begin(); j != plans.end(); ++j)
+          if (!j->second.timed && (oldest == plans.end() || j->second.last_use < oldest->second.last_use)) oldest = j;
+        if (oldest != plans.end()) {
+          oldest->second.destroy();
+          plans.erase(oldest);
+        }
+      }
       Plan p;
-      if (make_plan(p, N, O, I, lda, ldw, ldc, A, W, C, stream)) return 1;
+      if (make_plan(p, N, O, I, lda, ldw, ldc, A, W, C, stream)) {
+        p.destroy();
+        return 1;
+      }
       it = plans.emplace(key, p).first;
     }
     plan = &it->second;
+    plan->last_use = ++use_clock;
   }
   const float one = 1.f, zero = 0.f;
   LT(hipblasLtMatmul(handle, plan->desc, &one, W, plan->w, A, plan->a, &zero, C, plan->c, C, plan->c, &plan->algo,

@@ -60,6 +60,7 @@ class DecodeLoop:
         self.graph: Optional[torch.cuda.CUDAGraph] = None          # one step
         self.graph_many: Optional[torch.cuda.CUDAGraph] = None     # UNROLL steps: fewer launches from the host
         self._prepared = None                                      # (steps done, steps) that `prepare` last made ready
+        self._workspace: Optional[torch.Tensor] = None             # activations of the native step under the captured graphs
         self._allocate(params)
         self.rebind(rids, last_tokens, params, first_index)
 
@@ -68,7 +69,8 @@ class DecodeLoop:
         engine, b = self.engine, self.n
         cm, dev = engine.cache, engine.device
         self.greedy = params is None or all(p.greedy for p in params)
-        self.width = [cm.pages_for(engine.ctx_limit) for _ in range(cm.n_groups)]
+        # a request holds at most the pages of the context limit, and never more than its group's pool has
+        self.width = [min(cm.pages_for(engine.ctx_limit), cm.pools[g].num_pages) for g in range(cm.n_groups)]
         # static metadata: ids pos row_req cu ctx slot logit_rows tables...
         sizes = [b, b, b, b + 1, b, b, b] + [b * w for w in self.width]
         offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])
@@ -168,7 +170,7 @@ class DecodeLoop:
 
     # ------------------------------------------------------------------ one step on the device
     def _step(self) -> None:
-        logits = self.engine.model.forward(self.batch, self.engine._views)
+        logits = self.engine.forward(self.batch, self._workspace)
         if self.greedy:
             ops.argmax(logits, out=self.batch.ids)
             ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, None, None, self.n)
@@ -201,6 +203,12 @@ class DecodeLoop:
         self.u.copy_(self.u_all[self.steps_done])
 
     def _capture(self, many: bool) -> None:
+        if self.graph is None and self.engine.plan is not None:
+            # the native step's activations: a buffer of the loop's own, which the captured graphs replay
+            # over (the engine's own may be replaced by a larger one when another step needs more)
+            need = self.engine.plan.workspace_bytes(self.batch)
+            if self._workspace is None or self._workspace.numel() < need:
+                self._workspace = torch.empty(need, dtype=torch.uint8, device=self.engine.device)
         if self.graph is None:
             # warm up outside capture (lazy initialisation inside libraries), then capture one step
             # (the warm-up step is undone: metadata and per-request state are put back; its key and

@@ -22,10 +22,12 @@ from ..config import config_from_dict, read_config_json
 from ..config.base import ArchConfig
 from ..ops.lib import KernelError, library
 from ..parts import DecoderModel, Runtime
+from ..parts.native import MAX_GROUPS, NativePlan
 from ..weights import WeightStore, load_weights, table_of
 from .batch import BatchStager, Entry, StepBatch
 
 DEFAULT_PAGE_SIZE = 16      # tokens per cache page, the reference's block size (src/kv/mod.rs:6)
+DEFAULT_MAX_CONTEXT = 4096  # the context limit when none is asked for, if the model allows as much
 DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
 
 
@@ -42,16 +44,19 @@ class Engine:
                  max_requests: int = 8, page_size: int = DEFAULT_PAGE_SIZE, device: str = "cuda:0", arch: Optional[str] = None,
                  ctx: Optional[int] = None, config: Optional[ArchConfig] = None,
                  weights: Optional[WeightStore] = None, fold_gains: bool = True, fused_decode_rows: int = 64,
-                 group_pages: Optional[Sequence[int]] = None):
+                 group_pages: Optional[Sequence[int]] = None, native_step: bool = True):
         """`model_dir`: a folder with config.json and model.safetensors (the model class is chosen
         by config.json).  `max_tokens`: tokens the cache pool holds (each request's count rounded
-        up to whole pages).  `ctx`: context limit, default config.json's max_position_embeddings.
+        up to whole pages).  `ctx`: context limit, default config.json's max_position_embeddings or 4,096,
+        whichever is smaller.
         `config` + `weights` may stand in for a folder (weights already on the device).
         `fold_gains=False` keeps the norms' gains out of the bfloat16 matrices and `fused_decode_rows=0`
         keeps steps of decoded tokens off the fused decode kernels: the same model on the general path,
         for comparisons.  `group_pages`: pages of every cache group's pool, one count per group in
         the order the groups first appear in the layer order (default: `max_tokens` worth for each; a
-        group with a window can do with about max_requests x (window + longest portion) tokens)."""
+        group with a window can do with about max_requests x (window + longest portion) tokens).
+        `native_step=False` steps through the parts in Python instead of the one native call (the
+        same kernels; a model with a part from outside the package always does)."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU: this engine has no CPU path")
         if dtype not in DTYPES:
@@ -69,7 +74,8 @@ class Engine:
         if weights is None:
             weights = load_weights(model_dir, self.model.tensor_decls(), self.dtype, self.device)
         self.page_size = page_size
-        self.ctx_limit = int(ctx) if ctx else self.spec.max_position
+        # the reference's default: first(runtime.ctx, min(max_position_embeddings or 2048, 4096)) (arch/families/lfm2.json5:50)
+        self.ctx_limit = int(ctx) if ctx else min(self.spec.max_position or 2048, DEFAULT_MAX_CONTEXT)
         num_pages = max(1, -(-max_tokens // page_size))
         self.rt = Runtime(self.device, self.dtype, max_positions=min(self.ctx_limit, num_pages * page_size),
                           fold_gains=fold_gains, fused_decode_rows=fused_decode_rows)
@@ -83,6 +89,7 @@ class Engine:
         self._views = [self.device_cache.layer_view(run, src)
                        for run, src in enumerate(self.model.kv_source_runs())]
         self._stager = BatchStager(self.device)
+        self.plan = NativePlan.build(self.model, self._views, self.rt) if native_step and self.cache.n_groups <= MAX_GROUPS else None
 
     # ------------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> bool:
@@ -143,12 +150,19 @@ class Engine:
         widths = [int(info[1 + g]) for g in range(cache.n_groups)]
         return self._stager.stage_native(lib, cache.core, operands, info, widths, int(want_cu[-1]))
 
+    def forward(self, batch: StepBatch, workspace: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """The model's forward pass over a staged batch: one native call when the model has a plan
+        (`workspace`: see `NativePlan.step`), else through the parts."""
+        if self.plan is not None:
+            return self.plan.step(batch, workspace)
+        return self.model.forward(batch, self._views)
+
     def step(self, entries: Sequence[Entry]) -> Optional[torch.Tensor]:
         """Runs one batch; returns float32 logits [wanted places, vocab] in the order of the
         entries and of their `want` (None if nothing is wanted)."""
         entries = [e if isinstance(e, Entry) else Entry(*e) for e in entries]
         batch = self.prepare(entries)
-        logits = self.model.forward(batch, self._views)
+        logits = self.forward(batch)
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))
         return logits

@@ -12,6 +12,7 @@ from typing import Callable, Dict, Hashable, List, Optional, Sequence, Union
 
 import torch
 
+from .. import ops
 from ..sampling.sampler import Draw, Sampler, SamplingParams
 from .batch import Entry
 from .decode import DecodeLoop
@@ -66,7 +67,8 @@ class Generator:
         self.sampler = Sampler(engine.device)
         eos = engine.spec.eos_token_ids if eos_token_ids is None else eos_token_ids
         self.scheduler = ContinuousBatchScheduler(engine.cache, self._run, context_len=engine.ctx_limit,
-                                                  max_batch_tokens=max_batch_tokens, chunk=chunk, eos_token_ids=eos)
+                                                  max_batch_tokens=max_batch_tokens, chunk=chunk, eos_token_ids=eos,
+                                                  one_off_work=ops.one_off_work)
         self.stats = GenerationStats()
         self._times: Dict[Hashable, List[float]] = {}       # request -> [submitted, first token, last token, tokens]
 

@@ -153,11 +153,15 @@ EV_ADMITTED, EV_RELEASED, EV_PREEMPTED, EV_STOP, EV_LENGTH, EV_TOO_LARGE, EV_POO
 class ContinuousBatchScheduler:
     def __init__(self, cache: CacheManager, runner: Runner, *, context_len: int,
                  max_batch_tokens: Union[int, str] = MAX_PREFILL_CHUNK, chunk: Optional[int] = None,
-                 eos_token_ids: SeqOf[int] = (), clock: Callable[[], float] = time.perf_counter):
+                 eos_token_ids: SeqOf[int] = (), clock: Callable[[], float] = time.perf_counter,
+                 one_off_work: Callable[[], int] = lambda: 0):
         """`cache`: the engine's cache manager (pages and slots are taken here, before a step
         runs).  `runner`: runs one batch and samples.  `max_batch_tokens`: prompt tokens per step,
         or "auto" for the reference's measured budget (`PrefillTuner`; `clock` gives its seconds).
-        `chunk`: most prompt tokens of one request per step (None: the budget)."""
+        `chunk`: most prompt tokens of one request per step (None: the budget).  `one_off_work`: a
+        count that grows when a step did set-up work that its like will not do again (the engine's
+        `ops.one_off_work`); such a step's time is kept from the measured budget."""
+        self.one_off_work = one_off_work
         self.tuner: Optional[PrefillTuner] = None
         self.clock = clock
         if max_batch_tokens == "auto":
@@ -302,7 +306,7 @@ class ContinuousBatchScheduler:
                 prefill_tokens += n
         emitted: List[Tuple[Hashable, int]] = []
         if entries:
-            started = self.clock()
+            started, setup = self.clock(), self.one_off_work()
             try:
                 tokens = self.runner(entries, draws)
             except Exception as exc:                                # scheduler/mod.rs:1332-1340
@@ -311,7 +315,7 @@ class ContinuousBatchScheduler:
                 waiting, active = self._counts()
                 return StepOutput(entries, [], finished, preempted, prefill_tokens, decode_tokens, active, waiting)
             assert len(tokens) == len(sampled_for)
-            if self.tuner is not None:
+            if self.tuner is not None and self.one_off_work() == setup:      # (a step that did set-up work is no measure)
                 self.tuner.record(self.clock() - started, prefill_tokens, decode_tokens)
             # emit and finish
             k = len(tokens)

@@ -159,6 +159,13 @@ def gemm_library(a: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] =
     return out
 
 
+def one_off_work() -> int:
+    """A count that grows whenever a call did set-up work that its like will not do again (the timed
+    choice of a library algorithm for a new shape): a step during which it grew is no measure of
+    what such steps cost."""
+    return int(library().gibbs_gemm_library_timings())
+
+
 class PackedWeight:
     """A matrix [groups * rows, inner] (bfloat16) in the order the few-row products read it:
     [group][ceil(rows/16)][ceil(inner/32)][64 lanes][8], lane (r, g) of a tile holding

@@ -68,6 +68,23 @@ _SIGNATURES = {
 }
 
 
+_PLAN_SIGNATURES = {
+    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int], c_void_p),
+    "gibbs_plan_destroy": ([c_void_p], None),
+    "gibbs_plan_add_block": ([c_void_p, c_void_p, c_float, c_void_p, c_float], c_int),
+    "gibbs_plan_set_conv": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                             c_long, c_int], c_int),
+    "gibbs_plan_set_attention": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
+                                  c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
+                                  c_int, c_int, c_int, c_int, c_int], c_int),
+    "gibbs_plan_set_glu": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
+    "gibbs_plan_workspace": ([c_void_p, c_void_p], c_long),
+    "gibbs_plan_step": ([c_void_p, c_void_p], c_int),
+    "gibbs_plan_decode_tail": ([c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p], c_int),
+}
+
+
 def library() -> ctypes.CDLL:
     """The loaded kernel library (built at the first call if it is not there yet)."""
     global _lib
@@ -84,6 +101,10 @@ def library() -> ctypes.CDLL:
                     fn = getattr(lib, name)
                     fn.argtypes = argtypes
                     fn.restype = c_int
+                for name, (argtypes, restype) in _PLAN_SIGNATURES.items():
+                    getattr(lib, name).argtypes, getattr(lib, name).restype = argtypes, restype
+                for name in ("gibbs_gemm_library_timings", "gibbs_gemm_library_plans"):
+                    getattr(lib, name).argtypes, getattr(lib, name).restype = [], c_long
                 lib.gibbs_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]
                 lib.gibbs_attention_decode_workspace.restype = c_long
                 _lib = lib

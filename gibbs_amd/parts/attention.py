@@ -145,6 +145,16 @@ class AttentionMixer(Mixer):
             k_gain=self.k_gain, eps=self.qk_norm_eps, window=self.window, max_seq=batch.max_seq,
             **self._rotation_args())
 
+    def emit_native(self, builder, cache, folded: bool) -> bool:
+        if not self.fast_ok or cache.kpages is None or cache.kpages.shape != cache.vpages.shape:
+            return False                # (an encoding with a hook or score slopes steps through `forward`)
+        builder.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
+                          kv_heads=self.kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+                          q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
+                          kpages=cache.kpages, vpages=cache.vpages, group=cache.group, owns=self.source is None,
+                          fusable=folded and self.can_decode_fused(None))
+        return True
+
     # ------------------------------------------------------------------ one step
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         n = batch.n_rows

@@ -59,6 +59,16 @@ class PreNormBlock(Block):
         return (folded and fused_decode_step(self.rt, batch) and hasattr(part, "decode_fused")
                 and part.can_decode_fused(batch))
 
+    def emit_native(self, builder, cache) -> bool:
+        """Lays the block down in the native step's plan; False if one of its parts cannot."""
+        parts = (self.mixer_norm, self.ffn_norm, self.mixer, self.ffn)
+        if not all(hasattr(p, "native_norm") for p in parts[:2]) or not all(hasattr(p, "emit_native") for p in parts[2:]):
+            return False
+        (g1, e1), (g2, e2) = self.mixer_norm.native_norm(), self.ffn_norm.native_norm()
+        builder.block(g1, e1, g2, e2)
+        return (self.mixer.emit_native(builder, cache, self.mixer_folded)
+                and self.ffn.emit_native(builder, self.ffn_folded))
+
     def forward(self, stream: Stream, batch, cache) -> Stream:
         if self._fused(self.mixer, self.mixer_folded, batch):
             self.mixer.decode_fused(self._with_mirror(stream), self.mixer_norm.spec.eps, batch, cache)

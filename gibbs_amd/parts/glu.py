@@ -56,6 +56,12 @@ class GluFeedForward(FeedForward):
         act = ops.skinny_glu(stream.mirror, self.p_gate_up or self.w_gate_up, rms_eps=norm_eps, activation=self.activation)
         ops.skinny_residual(act, self.p_down or self.w_down, stream.x, stream.mirror)
 
+    def emit_native(self, builder, folded: bool) -> bool:
+        builder.glu(w_gate_up=self.w_gate_up, p_gate_up=self.p_gate_up, w_down=self.w_down, p_down=self.p_down,
+                    inter=self.inter, activation=ops.ACTIVATIONS[self.activation],
+                    fusable=folded and self.can_decode_fused(None))
+        return True
+
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
         gu = linear(h, self.w_gate_up)
         return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True, packed=self.p_down)

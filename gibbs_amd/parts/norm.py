@@ -32,3 +32,7 @@ class RMSNorm(Norm):
 
     def small_tensors(self):
         return [] if self.gain is None else [self.gain]
+
+    def native_norm(self):
+        """(gain or None, eps) for the native step."""
+        return self.gain, self.spec.eps

@@ -79,6 +79,12 @@ class ShortConvMixer(Mixer):
                             batch.ctx, rms_eps=norm_eps)
         ops.skinny_residual(y, self.p_out or self.w_out, stream.x, stream.mirror)
 
+    def emit_native(self, builder, cache, folded: bool) -> bool:
+        builder.short_conv(w_in=self.w_in, p_in=self.p_in, w_out=self.w_out, p_out=self.p_out, taps=self.taps,
+                           bias=self.conv_bias, width=self.width, kernel=self.kernel, state=cache.states[STATE],
+                           fusable=folded and self.can_decode_fused(None))
+        return True
+
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
         bcx = linear(h, self.w_in)
         y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,

@@ -254,7 +254,7 @@ def test_sequence_past_one_segment_of_page_ids(tmp_path_factory, dtype):
             entries.insert(0 if m == 1 else 1, ("other", seqs["other"][at["other"]:at["other"] + m], [m - 1]))
             at["other"] += m
         steps.append((entries, []))
-    eng = make_engine(d, dtype, max_tokens=4608, max_requests=2, page_size=8)
+    eng = make_engine(d, dtype, max_tokens=4608, max_requests=2, page_size=8, ctx=8192)
     got = run_steps(eng, steps)
     assert ("long", 4399) in got and sum(1 for r, p in got if r == "long" and p > 4096) >= 50
     check(d, seqs, got, dtype, f"past one segment {dtype}", against_whole=False)
@@ -392,3 +392,28 @@ def test_benchmark_layer_sizes(tmp_path_factory, dtype):
     got = run_steps(eng, steps)
     assert ("a", 149) in got and ("b", 39) in got
     check(d, seqs, got, dtype, f"1.2B layer sizes, portions and decoding {dtype}", against_whole=False)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "M"])
+def test_native_step_equals_stepping_through_the_parts(model_dirs, tmp_path_factory, name, dtype):
+    """The step as one native call queues the kernels that the parts' `forward` would queue, with the
+    same choices: the logits of a mixed schedule (portions, decoded tokens alone and at the head of a
+    step, many rows) are the same bit for bit."""
+    d = model_dirs[name] if name in model_dirs else H.make_model_dir(str(tmp_path_factory.mktemp("native")), name, seed=8, std=0.05)
+    vocab = H.TINY[name]["vocab_size"]
+    rng = np.random.default_rng(11)
+    seqs = {f"q{i}": H.tokens(700 + i, int(n), vocab) for i, n in enumerate([70, 45, 131, 33, 64])}
+    steps = mixed_schedule(seqs, rng)
+    long = H.tokens(710, 300, vocab)
+    steps.append(([("long", long[:200], [0, 199])], []))
+    steps.append(([("long", long[200:203], [2]), ("q0", [1, 2], [1])], ["q0"]))
+    steps += [([("long", [t], [0])], []) for t in long[203:240]]
+    got = {}
+    for native in (True, False):
+        eng = make_engine(d, dtype, max_tokens=1024, max_requests=5, native_step=native)
+        assert (eng.plan is not None) == native
+        got[native] = run_steps(eng, steps)
+    assert got[True].keys() == got[False].keys()
+    for key in got[True]:
+        assert np.array_equal(got[True][key], got[False][key]), f"{name} {dtype}: place {key} differs between the two ways"
