@@ -12,6 +12,7 @@ model entry inherits the defaults; the keys that mean something here:
     batch           requests decoded side by side (default 1)
     dtype           "bfloat16" (default) or "float32"
     min_tok_s       the run fails (exit status 3) if decode is slower
+    native_step     false: step through the parts in Python instead of the one native call
     workload        "decode" (default: the protocol below) or "serve": `requests` prompts of
                     `prefill_tokens` seeded ids each are submitted at once to the continuous-batching
                     scheduler and generate `decode_tokens` tokens each (greedy, no EOS), with
@@ -72,9 +73,11 @@ def _load(entry: Dict, base: str, batch: int = 0, ctx: int = 0):
         decls = DecoderModel(cfg.model_spec()).tensor_decls()
         compute = torch.bfloat16 if entry["dtype"] == "bfloat16" else torch.float32
         weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0")
-        return Engine(config=cfg, weights=weights, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
+        return Engine(config=cfg, weights=weights, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx,
+                      native_step=bool(entry.get("native_step", True)))
     path = ident if os.path.isabs(ident) else os.path.join(base, ident)
-    return Engine(path, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
+    return Engine(path, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx,
+                      native_step=bool(entry.get("native_step", True)))
 
 
 def measure(entry: Dict, base: str) -> Dict:
@@ -158,10 +161,16 @@ def serve(entry: Dict, base: str) -> Dict:
     budget = entry.get("max_batch_tokens", 2048)
     gen = Generator(engine, max_batch_tokens=budget if budget == "auto" else int(budget), chunk=int(chunk) if chunk else None)
     params = SamplingParams(temperature=0.0, max_new_tokens=n_decode, ignore_eos=True)
-    warm = gen.submit(rng.integers(0, engine.spec.vocab, size=min(n_prompt, 64)).tolist(),
-                      SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True))
-    gen.run()                                                # compiles nothing, but warms libraries and captures
-    assert warm is not None
+    # warm-up: as many prompts as fill one step's budget (the library chooses its algorithm for a new
+    # number of rows at the first such step), a few decoded tokens each
+    per_step = budget if isinstance(budget, int) else 2048
+    if chunk:
+        per_step = min(per_step, int(chunk))
+    n_warm = max(1, min(live, -(-int(per_step) // n_prompt)))
+    for _ in range(n_warm):
+        gen.submit(rng.integers(0, engine.spec.vocab, size=n_prompt).tolist(),
+                   SamplingParams(temperature=0.0, max_new_tokens=20, ignore_eos=True))
+    gen.run()
     gen.stats = type(gen.stats)()
     rids = [gen.submit(rng.integers(0, engine.spec.vocab, size=n_prompt).tolist(), params) for _ in range(n_req)]
     torch.cuda.synchronize()

@@ -53,6 +53,37 @@ class Stream:
     pending: Optional[torch.Tensor] = None
     mirror: Optional[torch.Tensor] = None
 
+    # What every arrangement does with the stream, so that none has to know how deltas travel:
+    def normed(self, norm: "Norm", rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
+        """norm(x + what is pending) in the activation type.  All rows: the pending delta is added
+        into x on the way (one kernel).  With `rows`, only those rows are normed and x stays as it is."""
+        h = norm.forward(self.x, self.pending, rows, n_rows)
+        if rows is None and self.pending is not None:
+            self.pending, self.mirror = None, None
+        return h
+
+    def add(self, delta: torch.Tensor) -> None:
+        """x += delta, lazily: the delta stays pending until the next `normed` or `add` (a delta is
+        [N, hidden] in the activation type, or float32 partial sums [S, N, hidden])."""
+        self.settle()
+        self.pending, self.mirror = delta, None
+
+    def settle(self) -> None:
+        """Adds what is pending into x now."""
+        if self.pending is not None:
+            from .. import ops
+            ops.residual_add(self.x, self.pending)
+            self.pending, self.mirror = None, None
+
+    def with_mirror(self) -> "Stream":
+        """Settles the stream and makes sure that `mirror` = bfloat16(x) exists (one kernel for both)."""
+        if self.pending is not None or self.mirror is None:
+            from .. import ops
+            mirror = torch.empty(self.x.shape, dtype=torch.bfloat16, device=self.x.device)
+            ops.residual_add(self.x, self.pending, mirror)
+            self.pending, self.mirror = None, mirror
+        return self
+
 
 class Part:
     def tensor_decls(self) -> List[TensorDecl]:

@@ -46,15 +46,6 @@ class PreNormBlock(Block):
         part.fold_input_gain(norm.fold_gain())
         return True
 
-    @staticmethod
-    def _with_mirror(stream: Stream) -> Stream:
-        """Adds what is pending and makes sure the bfloat16 mirror of x exists."""
-        if stream.pending is not None or stream.mirror is None:
-            mirror = torch.empty(stream.x.shape, dtype=torch.bfloat16, device=stream.x.device)
-            ops.residual_add(stream.x, stream.pending, mirror)
-            stream.pending, stream.mirror = None, mirror
-        return stream
-
     def _fused(self, part, folded: bool, batch, cache=None) -> bool:
         return (folded and fused_decode_step(self.rt, batch) and hasattr(part, "decode_fused")
                 and part.can_decode_fused(batch))
@@ -71,13 +62,11 @@ class PreNormBlock(Block):
 
     def forward(self, stream: Stream, batch, cache) -> Stream:
         if self._fused(self.mixer, self.mixer_folded, batch):
-            self.mixer.decode_fused(self._with_mirror(stream), self.mixer_norm.spec.eps, batch, cache)
+            self.mixer.decode_fused(stream.with_mirror(), self.mixer_norm.spec.eps, batch, cache)
         else:
-            h = self.mixer_norm.forward(stream.x, stream.pending)       # x += pending; h = norm(x)
-            stream.pending, stream.mirror = self.mixer.forward(h, batch, cache), None
+            stream.add(self.mixer.forward(stream.normed(self.mixer_norm), batch, cache))   # (the add waits for the next norm)
         if self._fused(self.ffn, self.ffn_folded, batch):
-            self.ffn.decode_fused(self._with_mirror(stream), self.ffn_norm.spec.eps, batch)
+            self.ffn.decode_fused(stream.with_mirror(), self.ffn_norm.spec.eps, batch)
         else:
-            h = self.ffn_norm.forward(stream.x, stream.pending)
-            stream.pending, stream.mirror = self.ffn.forward(h, batch), None
+            stream.add(self.ffn.forward(stream.normed(self.ffn_norm), batch))
         return stream

@@ -89,5 +89,5 @@ class DecoderModel(Part):
             stream = self.blocks[i].forward(stream, batch, caches[run])
         if batch.n_logits == 0:
             return None
-        h = self.final_norm.forward(stream.x, stream.pending, batch.logit_rows, batch.n_logits)
+        h = stream.normed(self.final_norm, batch.logit_rows, batch.n_logits)
         return linear(h, self.head, out_dtype=torch.float32, packed=self.head_packed)

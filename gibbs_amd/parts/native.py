@@ -96,7 +96,10 @@ class NativePlan:
 
     def __del__(self):
         if getattr(self, "handle", None):
-            L.library().gibbs_plan_destroy(self.handle)
+            try:
+                L.library().gibbs_plan_destroy(self.handle)
+            except TypeError:              # (the interpreter is shutting down: the module is gone already)
+                pass
             self.handle = None
 
     @classmethod

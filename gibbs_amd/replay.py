@@ -63,9 +63,13 @@ def main(argv=None) -> int:
     from .engine import Engine
     from .engine.engine import DEFAULT_PAGE_SIZE
 
+    from .config import config_from_dict, read_config_json
+    from .weights import table_of
     page = args.page_size or DEFAULT_PAGE_SIZE
+    # a trace may be as long as the model allows (generation's default context limit is shorter)
+    longest = config_from_dict(read_config_json(args.model), tensors=table_of(args.model)).model_spec().max_position
     engine = Engine(args.model, dtype=args.dtype, max_tokens=pool_tokens_for(args.max_tokens, page),
-                    max_requests=args.max_requests, page_size=page)
+                    max_requests=args.max_requests, page_size=page, ctx=longest)
     print("trace_run: ready", file=sys.stderr, flush=True)
     replay(engine, sys.stdin, args.out)
     return 0

@@ -370,6 +370,46 @@ def test_trace_run_program(dirs, dtype, tmp_path):
     H.assert_close(read(4), pa[53:70], dtype, "step 4")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program_four_ways(dirs, dtype, tmp_path):
+    """The program itself (a subprocess, JSON lines in, files out) over the four ways of running the same
+    requests of Tiny B: whole; most in one step and the last 32 tokens one by one; portions of changing
+    size down to two tokens; mixed, up to four live requests in a pool so small that pages are used
+    again (--max-tokens 4 x 128).  Every wanted place against the plain implementation."""
+    from tests.test_engine_gpu import mixed_schedule, portions
+    d = dirs["B"]
+    vocab = H.TINY["B"]["vocab_size"]
+    seqs = {f"q{i}": H.tokens(900 + i, n, vocab) for i, n in enumerate([100, 45, 90, 64, 81, 50, 77, 96])}
+    assert sum(-(-len(s) // 16) for s in seqs.values()) > 512 // 16, "the pool must be too small to avoid reuse"
+    first = seqs["q0"]
+    ways = {
+        "whole": [([(r, ids, list(range(len(ids))))], [r]) for r, ids in seqs.items()],
+        "tail": [([("q0", first[:68], list(range(68)))], [])] + [([("q0", [t], [0])], []) for t in first[68:]] + [([], ["q0"])],
+        "portions": [([("q0", first[a:b], list(range(b - a)))], []) for a, b in portions(100, [7, 2, 13, 3, 2, 33, 5, 2, 17])],
+        "mixed": mixed_schedule(seqs, np.random.default_rng(12)),
+    }
+    for way, steps in ways.items():
+        out = tmp_path / way
+        proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", d, "--dtype", dtype,
+                               "--out", str(out), "--max-tokens", "512"], input=trace_lines(steps), capture_output=True,
+                              text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(len(steps))]
+        at, got, want = {}, [], []
+        for i, (entries, ends) in enumerate(steps):
+            wanted = sum(len(w) for _, _, w in entries)
+            if wanted:
+                got.append(np.fromfile(out / f"{i}.f32", dtype="<f4").reshape(wanted, vocab))
+                want += [H.plain_logits(d, seqs[r])[at.get(r, 0) + w] for r, _, places in entries for w in places]
+            for r, toks, _ in entries:
+                at[r] = at.get(r, 0) + len(toks)
+            for r in ends:
+                at.pop(r, None)
+        places = len(want)
+        H.assert_close(np.concatenate(got), np.stack(want), dtype, f"trace_run {way}", model="B")
+        assert places >= 100, way
+
+
 def test_command_line(dirs, tmp_path):
     env = dict(os.environ)
     run = lambda *a: subprocess.run([sys.executable, os.path.join(ROOT, "bin", "gibbs"), *a], capture_output=True,

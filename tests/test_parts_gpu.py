@@ -931,3 +931,87 @@ def test_positions_that_are_no_rotation_and_values_wider_than_keys(name, dtype, 
             got.setdefault(r, []).append(out[at:at + b - a]); at += b - a
     for r, ids in seqs.items():
         H.assert_close(np.concatenate(got[r]), wide_plain(cfg, weights, ids), name, f"toy positions / wide values request {r}")
+
+
+# --------------------------------------------------------------------------- another arrangement of a block's parts
+def test_an_arrangement_from_outside_uses_the_stream_protocol(tmp_path):
+    """A block in which mixer and feed-forward read the same normed rows and both add to the stream
+    (x += mixer(norm(x)) + ffn(norm(x))), registered from here: it hands its deltas to the residual
+    stream through `Stream.normed` / `Stream.add` and knows nothing of how they travel (pending
+    deltas, float32 partial sums, the bfloat16 mirror).  Both precisions, portions and single tokens."""
+    from gibbs_amd import Engine, Entry
+    from gibbs_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                  register_architecture)
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.parts import Block, DecoderModel, register_arrangement
+    from gibbs_amd.weights import write_random_model
+
+    @register_arrangement("toy_parallel")
+    class Parallel(Block):
+        def parts(self):
+            return [self.mixer_norm, self.mixer, self.ffn]          # (one norm: the second is not used)
+
+        def forward(self, stream, batch, cache):
+            h = stream.normed(self.mixer_norm)
+            stream.add(self.mixer.forward(h, batch, cache))
+            stream.add(self.ffn.forward(h, batch))
+            return stream
+
+    class ParallelConfig(ArchConfig):
+        architecture = "ToyParallelForCausalLM"
+
+        def __init__(self, cfg):
+            self.cfg = dict(cfg)
+
+        @classmethod
+        def from_dict(cls, cfg, tensors=None):
+            return cls(cfg)
+
+        def to_dict(self):
+            return dict(self.cfg)
+
+        def model_spec(self):
+            c, layers = self.cfg, []
+            for i, kind in enumerate(c["mixers"]):
+                p = f"b{i}"
+                if kind == "conv":
+                    mixer = MixerSpec("short_conv", {"width": c["width"], "kernel": 3, "bias": False},
+                                      {"in_proj": f"{p}.in", "conv": f"{p}.taps", "out_proj": f"{p}.out"})
+                else:
+                    mixer = MixerSpec("attention", {"heads": 2, "kv_heads": 1, "head_dim": 16, "scale": 0.25, "qk_norm": None,
+                                                    "window": None},
+                                      {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o"},
+                                      PositionSpec("rope", {"theta": 1e4, "rotary_dim": 16, "precision": "f32"}))
+                ffn = FeedForwardSpec("glu", {"inter": c["ff"], "activation": "silu"}, {"gate": f"{p}.g", "up": f"{p}.u", "down": f"{p}.d"})
+                norm = NormSpec("rms", c["eps"], f"{p}.n")
+                layers.append(LayerSpec(p, "toy_parallel", norm, mixer, norm, ffn))
+            return ModelSpec(self.architecture, c["width"], c["vocab"], tuple(layers), tuple(range(len(layers))), "tok",
+                             NormSpec("rms", c["eps"], "out_norm"), None, 128)
+    register_architecture("ToyParallelForCausalLM", ParallelConfig)
+    cfg = {"architectures": ["ToyParallelForCausalLM"], "width": 48, "ff": 80, "vocab": 61, "mixers": ["conv", "attn", "conv"],
+           "eps": 1e-5}
+    config = ParallelConfig(cfg)
+    folder = str(tmp_path / "parallel")
+    write_random_model(folder, config, DecoderModel(config.model_spec()).tensor_decls(), seed=6, std=0.2, gain_std=0.2)
+    w, _ = P.load_model_dir(folder)
+    ids = H.tokens(8, 50, 61)
+    T = len(ids)
+    x = P.embedding(w["tok"], ids)
+    for i, kind in enumerate(cfg["mixers"]):
+        p = f"b{i}"
+        h = P.rms_norm(x, w[f"{p}.n"], cfg["eps"])
+        if kind == "conv":
+            a = P.short_conv_mixer(h, w[f"{p}.in"], w[f"{p}.taps"], w[f"{p}.out"])
+        else:
+            inv = P.rope_inv_freq(16, 1e4)
+            q = P.rope_half_split(P.linear(h, w[f"{p}.q"]).reshape(T, 2, 16), range(T), inv)
+            k = P.rope_half_split(P.linear(h, w[f"{p}.k"]).reshape(T, 1, 16), range(T), inv)
+            a = P.linear(P.causal_attention(q, k, P.linear(h, w[f"{p}.v"]).reshape(T, 1, 16), 0.25).reshape(T, 32), w[f"{p}.o"])
+        x = x + a + P.swiglu_ffn(h, w[f"{p}.g"], w[f"{p}.u"], w[f"{p}.d"])
+    want = P.linear(P.rms_norm(x, w["out_norm"], cfg["eps"]), w["tok"])
+    for name in ("float32", "bfloat16"):
+        eng = Engine(folder, dtype=name, max_tokens=128, max_requests=1, page_size=8)
+        assert eng.plan is None and [type(b).__name__ for b in eng.model.blocks] == ["Parallel"] * 3
+        got = [eng.step([Entry("r", ids[a:b], list(range(b - a)))]).cpu().numpy()
+               for a, b in [(0, 21), (21, 23), (23, 24), (24, 25), (25, 49), (49, 50)]]
+        H.assert_close(np.concatenate(got), want, name, f"parallel arrangement {name}")
