@@ -3,6 +3,12 @@ on one MI355X (batch 8, 2,048-token prompts, context 4096), with prefill speed a
 decode at batch 1 and 64 beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
+                    [--batch B] [--prompt-len P --context C] [--suite bench/SUITE.json]
+
+`--prompt-len` / `--context` move the same measurement to longer contexts (16k, 32k, 100k; the timed
+prefill stays at 2,048 tokens); `--suite` runs the rows of a suite file of `gibbs --bench` afterwards
+(the serving workloads of the 350M and 2.6B shapes in bench/lfm2.json) and puts them into the line
+under `rows`.
 
 A "step" is one decode step of the whole batch.  W untimed steps, then runs of exactly K timed steps
 between device synchronisations: the median of 3 runs counts (src/bench.rs:274-296).  Before a timed
@@ -20,6 +26,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -48,7 +55,7 @@ def shape_for(layers: int) -> dict:
     return cfg
 
 
-def build_engine(dtype: str, layers: int, max_requests: int):
+def build_engine(dtype: str, layers: int, max_requests: int, context: int = CONTEXT):
     import torch
 
     from gibbs_amd import Engine
@@ -59,8 +66,8 @@ def build_engine(dtype: str, layers: int, max_requests: int):
     decls = DecoderModel(cfg.model_spec()).tensor_decls()
     compute = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0")
-    return Engine(config=cfg, weights=weights, dtype=dtype, max_tokens=max_requests * CONTEXT,
-                  max_requests=max_requests, ctx=CONTEXT)
+    return Engine(config=cfg, weights=weights, dtype=dtype, max_tokens=max_requests * context,
+                  max_requests=max_requests, ctx=context)
 
 
 def seeded_prompt(seed: int, n: int, vocab: int):
@@ -84,9 +91,10 @@ def time_prefill(engine, runs: int = 3):
     return sorted(times[1:])[len(times[1:]) // 2]
 
 
-def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, profile: bool = False):
+def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, profile: bool = False,
+                prompt_len: int = PROMPT_LEN):
     """Median seconds for exactly `steps` decode steps of `batch` requests that each hold a
-    2,048-token prompt (greedy sampling on the device), the requests' lengths at the middle of that
+    `prompt_len`-token prompt (greedy sampling on the device), the requests' lengths at the middle of that
     run, and, with `profile`, the kernels of one more run by their share of its device time."""
     import torch
 
@@ -95,7 +103,7 @@ def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, p
     rids = [f"d{i}" for i in range(batch)]
     first = []
     for i, rid in enumerate(rids):
-        logits = engine.step([(rid, seeded_prompt(i, PROMPT_LEN, vocab), [PROMPT_LEN - 1])])
+        logits = engine.step([(rid, seeded_prompt(i, prompt_len, vocab), [prompt_len - 1])])
         first.append(int(logits.argmax(-1).item()))
     loop = DecodeLoop(engine, rids, first)
     if warmup > 0:
@@ -135,15 +143,44 @@ def kernel_shares(run, most: int = 8):
     total = sum(us for _, _, us in rows)
     if total <= 0:
         return None
-    merged = {}                                                # instantiations of one kernel count together
+    merged = {}
     for name, calls, us in rows:
-        short = name.replace("(anonymous namespace)::", "").replace("void ", "").split("<")[0].split("(")[0].strip()
-        entry = merged.setdefault(short or name[:60], [0, 0.0])
+        short = name.replace("(anonymous namespace)::", "").replace("void ", "").split("(")[0].strip()
+        mangled = re.match(r"_Z(?:N\d+_GLOBAL__N_1)?(\d+)", short)      # a name the profiler left mangled: keep the identifier
+        if mangled:
+            start = mangled.end()
+            short = short[start:start + int(mangled.group(1))]
+        entry = merged.setdefault(short[:72] or name[:72], [0, 0.0])
         entry[0] += int(calls)
         entry[1] += us
     ranked = sorted(merged.items(), key=lambda kv: -kv[1][1])[:most]
     return [{"name": name, "calls": calls, "us": round(us, 1), "share": round(us / total, 4)}
             for name, (calls, us) in ranked]
+
+
+def suite_rows(path: str) -> list:
+    """The rows of a `gibbs --bench` suite file, measured here one after the other (a row that fails
+    is reported with its error)."""
+    import gc
+
+    import torch
+
+    from gibbs_amd import bench_suite as S
+    with open(path) as f:
+        suite = json.load(f)
+    base = os.path.dirname(os.path.abspath(path))
+    rows = []
+    for m in suite["models"]:
+        entry = dict(S.DEFAULTS, **suite.get("defaults", {}), **m)
+        ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
+        entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
+        try:
+            rows.append({"serve": S.serve, "products": S.products}.get(entry.get("workload", "decode"), S.measure)(entry, base))
+        except Exception as exc:
+            rows.append({"model": entry["name"], "error": f"{type(exc).__name__}: {exc}"})
+        gc.collect()
+        torch.cuda.empty_cache()
+    return rows
 
 
 PARITY_PROMPT, PARITY_DECODE = 64, 8
@@ -200,6 +237,9 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the shape has (named in config)")
     ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens every request holds before decoding starts")
+    ap.add_argument("--context", type=int, default=None, help="context limit (default 4096, or what --prompt-len needs)")
+    ap.add_argument("--suite", help="a suite file of `gibbs --bench` whose rows are run afterwards and reported under `rows`")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate")
     ap.add_argument("--no-kernels", action="store_true", help="skip the kernels' shares of the decode step")
@@ -210,19 +250,23 @@ def main() -> int:
     if args.steps < 1 or args.warmup < 0:
         print("--steps must be at least 1 and --warmup at least 0")
         return 2
-    if PROMPT_LEN + args.warmup + (RUNS + 1) * args.steps + 1 > CONTEXT:
-        print(f"--warmup + {RUNS + 1} x --steps must stay below {CONTEXT - PROMPT_LEN - 1} (context {CONTEXT})")
+    need = args.prompt_len + args.warmup + (RUNS + 1) * args.steps + 1
+    context = args.context or max(CONTEXT, -(-need // 1024) * 1024)
+    if args.prompt_len < 1 or need > context:
+        print(f"--prompt-len + --warmup + {RUNS + 1} x --steps must stay below the context ({context})")
         return 2
 
     from gibbs_amd import roofline as R
     gate = None if args.no_parity else parity()
-    engine = build_engine(args.dtype, args.layers, max_requests=max(64, args.batch))
+    engine = build_engine(args.dtype, args.layers, max_requests=args.batch if args.no_points else max(64, args.batch),
+                          context=context)
 
     prefill_s = time_prefill(engine)
     prefill_flops = R.prefill_flops(engine, PROMPT_LEN)
     peak = R.PEAK_FLOPS[args.dtype]
 
-    dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels)
+    dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels,
+                                    prompt_len=args.prompt_len)
     ms_per_step = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     # bytes of a decode step at the middle of the timed span
@@ -232,18 +276,18 @@ def main() -> int:
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            d, _, _ = time_decode(engine, b, args.steps, args.warmup)
+            d, _, _ = time_decode(engine, b, args.steps, args.warmup, prompt_len=args.prompt_len)
             points[f"decode_b{b}"] = round(b * args.steps / d, 1)
 
     cfg = engine.config
     line = {
-        "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B shape, 2,048-token prompts, context 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (LFM2-1.2B shape, {args.prompt_len:,}-token prompts, context {context})",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "LFM2-1.2B shape, random weights", "global_batch": args.batch, "seq_len": CONTEXT,
-            "parallelism": "single GPU", "prompt_len": PROMPT_LEN, "layers": args.layers,
+            "model": "LFM2-1.2B shape, random weights", "global_batch": args.batch, "seq_len": context,
+            "parallelism": "single GPU", "prompt_len": args.prompt_len, "layers": args.layers,
             "layers_of_shape": FULL_LAYERS, "attention_layers": len(cfg.full_attn_idxs),
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "ff_dim": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
@@ -256,6 +300,9 @@ def main() -> int:
                      "frac": round(achieved / (R.HBM_BYTES_PER_S / 1e9), 4)},
         "points": points, "parity": gate, "top_kernels": top,
     }
+    if args.suite:
+        del engine
+        line["rows"] = suite_rows(args.suite)
     print(json.dumps(line))
     return 0
 
