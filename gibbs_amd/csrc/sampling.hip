@@ -289,6 +289,78 @@ GIBBS_EXPORT int gibbs_repetition_penalty(float* logits, int M, int V, long ld, 
   GIBBS_LAUNCH_STATUS("repetition_penalty");
 }
 
+// The end of a decode step that runs as a captured graph, in one kernel (one workgroup per row): the row's
+// next token (the first largest logit; or, with logits null, the token that a sampling kernel has put
+// into ids already) is logged, the row's position and cached length move on by one, its next draw is
+// loaded, and the token's embedding is written as the row of the next step's residual stream (and of its
+// bfloat16 mirror), so that the next step starts at its first layer.
+//   log[steps[i] * n + i] = ids[i];  pos[i] += 1;  ctx[i] += 1;  u[i] = u_all[(steps[i] + 1) * n + i];  steps[i] += 1
+template <typename T>
+__global__ __launch_bounds__(THREADS) void decode_tail_kernel(const float* __restrict__ logits, int V, long ld,
+                                                              int* __restrict__ ids, int* __restrict__ pos, int* __restrict__ ctx,
+                                                              int* __restrict__ log, int* __restrict__ steps, int n, int capacity,
+                                                              float* __restrict__ u, const float* __restrict__ u_all,
+                                                              const T* __restrict__ table, int vocab, int hidden,
+                                                              float* __restrict__ x, bf16* __restrict__ mirror) {
+  __shared__ float sv[THREADS / WAVE];
+  __shared__ int si[THREADS / WAVE];
+  __shared__ int s_token;
+  const int i = blockIdx.x;
+  int token = 0;
+  if (logits) {
+    const float* row = logits + (size_t)i * ld;
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    walk_row(row, V, [&](float v, int j) {
+      if (better(v, j, bv, bi)) { bv = v; bi = j; }
+    });
+    block_best(bv, bi, sv, si);
+    token = (bi == 0x7fffffff) ? 0 : bi;
+  }
+  if (threadIdx.x == 0) {
+    if (logits) ids[i] = token;
+    else token = ids[i];
+    const int step = steps[i];
+    if (step < capacity) log[(size_t)step * n + i] = token;
+    pos[i] += 1;
+    ctx[i] += 1;
+    if (u && step + 1 < capacity) u[i] = u_all[(size_t)(step + 1) * n + i];
+    steps[i] = step + 1;
+    s_token = token;
+  }
+  if (!x) return;
+  __syncthreads();
+  token = s_token;
+  token = token < 0 ? 0 : (token >= vocab ? vocab - 1 : token);   // never read outside the table
+  const T* src = table + (size_t)token * hidden;
+  for (int e = threadIdx.x; e < hidden; e += THREADS) {
+    const float v = to_float(src[e]);
+    x[(size_t)i * hidden + e] = v;
+    if (mirror) mirror[(size_t)i * hidden + e] = (bf16)v;
+  }
+}
+
+// logits: [n, V] float32 (row stride ld) or null (ids hold the tokens); steps: [n] steps done per row; u, u_all:
+// draws (or null); table: [vocab, hidden] in table_dtype; x: [n, hidden] float32 and mirror: [n, hidden]
+// bfloat16 for the next step (or null: no embedding).
+GIBBS_EXPORT int gibbs_decode_tail(const float* logits, int V, long ld, int* ids, int* pos, int* ctx, int* log, int* steps,
+                                   int n, int capacity, float* u, const float* u_all, const void* table, int table_dtype,
+                                   int vocab, int hidden, float* x, void* mirror, hipStream_t stream) {
+  GIBBS_REQUIRE(n > 0 && capacity > 0, "decode_tail: batch %d, log of %d steps", n, capacity);
+  GIBBS_REQUIRE(!logits || (V > 0 && ld >= V), "decode_tail: bad logits V=%d ld=%ld", V, ld);
+  GIBBS_REQUIRE(!x || (table && hidden > 0 && vocab > 0), "decode_tail: an embedding needs the token table");
+  GIBBS_REQUIRE(!u || u_all, "decode_tail: draws without their table");
+  if (table_dtype == GIBBS_F32)
+    decode_tail_kernel<float><<<n, THREADS, 0, stream>>>(logits, V, ld, ids, pos, ctx, log, steps, n, capacity, u, u_all,
+                                                         (const float*)table, vocab, hidden, x, (bf16*)mirror);
+  else if (table_dtype == GIBBS_BF16)
+    decode_tail_kernel<bf16><<<n, THREADS, 0, stream>>>(logits, V, ld, ids, pos, ctx, log, steps, n, capacity, u, u_all,
+                                                        (const bf16*)table, vocab, hidden, x, (bf16*)mirror);
+  else
+    return gibbs_fail("decode_tail: unknown table dtype %d", table_dtype);
+  GIBBS_LAUNCH_STATUS("decode_tail");
+}
+
 GIBBS_EXPORT int gibbs_argmax(const float* logits, int* out, int M, int V, long ld, hipStream_t stream) {
   GIBBS_REQUIRE(M >= 0 && V > 0 && ld >= V, "argmax: bad sizes M=%d V=%d ld=%ld", M, V, ld);
   if (M == 0) return 0;

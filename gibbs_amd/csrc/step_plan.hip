@@ -81,6 +81,7 @@ struct Plan {
   const void* table = nullptr;
   int table_dtype = GIBBS_BF16;
   Matrix head;
+  const void* head_folded = nullptr;   // the head in tile order with the final norm's gain multiplied in (bfloat16), or null
   NormP final_norm;
   int fused_rows = 64;      // steps of at most this many decoded tokens take the fused decode kernels
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
@@ -109,6 +110,12 @@ struct GibbsStepArgs {
   long workspace_bytes;
   float* logits;           // [n_logits, vocab] float32 out
   hipStream_t stream;
+  // A step that continues a captured decode loop: the rows' embeddings are there already (the end of the
+  // previous step wrote them), as the float32 stream x_in [n_rows, hidden] and, for steps that take the fused
+  // decode kernels, its bfloat16 mirror.  Null: the step embeds its ids itself.
+  float* x_in;
+  void* mirror_in;
+  int all_rows_wanted;     // logit_rows is 0, 1, ..., n_rows - 1
 };
 
 namespace {
@@ -428,9 +435,13 @@ struct Exec {
   // ------------------------------------------------------------------------------------------- the step
   void run() {
     const int N = a.n_rows, H = p.hidden;
-    float* x = (float*)take((long)N * H * 4);
-    void* mirror = fused_step ? take((long)N * H * 2) : nullptr;
-    RUN(gibbs_embed(p.table, p.table_dtype, a.ids, x, mirror, N, H, p.vocab, a.stream));
+    float* x = a.x_in;
+    void* mirror = fused_step ? a.mirror_in : nullptr;
+    if (!x) {
+      x = (float*)take((long)N * H * 4);
+      mirror = fused_step ? take((long)N * H * 2) : nullptr;
+      RUN(gibbs_embed(p.table, p.table_dtype, a.ids, x, mirror, N, H, p.vocab, a.stream));
+    }
     Pending pending;
     for (const BlockP& b : p.blocks) {
       const bool mixer_fused = fused_step && (b.mixer == MIX_CONV ? b.conv.fusable : b.attn.fusable);
@@ -457,7 +468,12 @@ struct Exec {
       }
       if (!ok()) return;
     }
-    if (a.n_logits > 0) {
+    if (a.n_logits > 0 && fused_step && a.all_rows_wanted && a.n_logits == N && N <= 32 && p.head_folded && mirror &&
+        pending.parts == 0) {
+      // decoded tokens, every row wanted, the stream settled with its mirror at hand: the final norm is the
+      // head product's RMS prologue (its gain is folded into the head's tile-ordered copy)
+      RUN(gibbs_skinny_store_f32(mirror, p.head_folded, a.logits, N, p.vocab, H, H, 0, p.vocab, 1, p.final_norm.eps, a.stream));
+    } else if (a.n_logits > 0) {
       void* h = norm(x, pending, p.final_norm, a.logit_rows, a.n_logits);
       const int M = a.n_logits, V = p.vocab;
       // the head: float32 logits straight into the caller's buffer
@@ -474,7 +490,7 @@ struct Exec {
       give(h);
     }
     give(pending.data);
-    give(mirror);
+    give(mirror);      // (buffers of the caller's are not the arena's: giving them back does nothing)
     give(x);
   }
 #undef RUN
@@ -494,8 +510,8 @@ int check_args(const Plan* p, const GibbsStepArgs* a) {
 
 // ------------------------------------------------------------------------------------------------- building a plan
 GIBBS_EXPORT void* gibbs_plan_create(int dtype, int hidden, int vocab, const void* table, int table_dtype, const void* head,
-                                     const void* head_packed, const float* final_gain, float final_eps, int fused_rows,
-                                     int own_gemm) {
+                                     const void* head_packed, const void* head_folded, const float* final_gain,
+                                     float final_eps, int fused_rows, int own_gemm) {
   if ((dtype != GIBBS_BF16 && dtype != GIBBS_F32) || hidden <= 0 || vocab <= 0 || !table || !head) {
     gibbs_fail("plan: bad model sizes or no token table");
     return nullptr;
@@ -504,6 +520,7 @@ GIBBS_EXPORT void* gibbs_plan_create(int dtype, int hidden, int vocab, const voi
   Plan* p = new Plan();
   p->dtype = dtype; p->hidden = hidden; p->vocab = vocab; p->table = table; p->table_dtype = table_dtype;
   p->head.w = head; p->head.packed = head_packed; p->head.O = vocab; p->head.I = hidden;
+  p->head_folded = (dtype == GIBBS_BF16 && hidden % 8 == 0) ? head_folded : nullptr;
   p->final_norm = NormP{final_gain, final_eps};
   p->fused_rows = fused_rows; p->own_gemm = own_gemm;
   return p;
@@ -589,17 +606,4 @@ GIBBS_EXPORT int gibbs_plan_step(const void* plan, const GibbsStepArgs* args) {
   Exec e(*(const Plan*)plan, *args, false);
   e.run();
   return e.status;
-}
-
-// The end of a captured decode step: the next tokens from the logits (greedy, or drawn with u) into ids,
-// then positions and cached lengths move on by one and the step is logged.
-GIBBS_EXPORT int gibbs_plan_decode_tail(const float* logits, int n, int vocab, int* ids, int* pos, int* ctx, int* log, int* counter,
-                                        int capacity, const float* temperature, const float* top_p, const int* top_k, float* u,
-                                        const float* u_all, hipStream_t stream) {
-  if (temperature) {
-    if (gibbs_sample(logits, ids, n, vocab, vocab, temperature, top_p, top_k, u, stream)) return 1;
-    return gibbs_advance(pos, ctx, ids, log, counter, u, u_all, n, capacity, stream);
-  }
-  if (gibbs_argmax(logits, ids, n, vocab, vocab, stream)) return 1;
-  return gibbs_advance(pos, ctx, ids, log, counter, nullptr, nullptr, n, capacity, stream);
 }

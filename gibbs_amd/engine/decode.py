@@ -4,7 +4,10 @@ device and fed back on the device, the whole step replayed as one captured HIP g
 The step is the engine's own: `model.forward` over a `StepBatch` whose metadata lives in static
 device buffers.  What changes between steps (positions, cached lengths, the sampled ids, the random
 draws) is updated by a kernel at the end of the step, so a replay needs no host work; pages for all
-steps of a `run` are reserved, and the block tables uploaded, before the first of them.
+steps of a `run` are reserved, and the block tables uploaded, before the first of them.  With the
+native step that same kernel also writes the sampled tokens' embeddings as the next step's residual
+rows, so a step is: layers, head (the final norm as its prologue), one kernel for argmax, log, advance
+and embedding.
 """
 from __future__ import annotations
 
@@ -82,9 +85,17 @@ class DecodeLoop:
             n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
             cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
             tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
-            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True)
+            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True, all_rows_wanted=True)
         self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
-        self.counter = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.counter = torch.zeros(b, dtype=torch.int32, device=dev)          # steps done, per row
+        # native step: the rows of the residual stream (and their bfloat16 mirror) live here from one step to
+        # the next; the end of a step writes the next tokens' embeddings into them
+        self.x = self.mirror = None
+        if engine.plan is not None:
+            hidden = engine.spec.hidden
+            self.x = torch.zeros((b, hidden), dtype=torch.float32, device=dev)
+            if engine.dtype == torch.bfloat16:
+                self.mirror = torch.zeros((b, hidden), dtype=torch.bfloat16, device=dev)
         if not self.greedy:
             self.temperature = torch.zeros(b, dtype=torch.float32, device=dev)
             self.top_p = torch.zeros(b, dtype=torch.float32, device=dev)
@@ -133,11 +144,18 @@ class DecodeLoop:
         self.steps_done = 0
         self.pending = 0
         self._prepared = None
+        self._embed()
         if not self.greedy:
             dev = engine.device
             self.temperature.copy_(torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32))
             self.top_p.copy_(torch.tensor([p.resolved_top_p for p in self.params], dtype=torch.float32))
             self.top_k.copy_(torch.tensor([p.top_k for p in self.params], dtype=torch.int32))
+
+    def _embed(self) -> None:
+        """The embeddings of the tokens in `ids` into the loop's residual rows (the first step after binding;
+        every later step finds what the end of the step before it wrote)."""
+        if self.x is not None:
+            ops.embed(self.engine.model.table, self.batch.ids, self.n, out=self.x, mirror=self.mirror)
 
     # ------------------------------------------------------------------ host side
     def _fill_tables(self) -> None:
@@ -170,14 +188,15 @@ class DecodeLoop:
 
     # ------------------------------------------------------------------ one step on the device
     def _step(self) -> None:
-        logits = self.engine.forward(self.batch, self._workspace)
+        b = self.batch
+        logits = self.engine.forward(b, self._workspace, self.x, self.mirror)
+        table = self.engine.model.table if self.x is not None else None
         if self.greedy:
-            ops.argmax(logits, out=self.batch.ids)
-            ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, None, None, self.n)
+            ops.decode_tail(logits, b.ids, b.pos, b.ctx, self.log, self.counter, None, None, self.n, table, self.x, self.mirror)
         else:
-            ops.sample(logits, self.temperature, self.top_p, self.top_k, self.u, out=self.batch.ids)
-            ops.advance(self.batch.pos, self.batch.ctx, self.batch.ids, self.log, self.counter, self.u, self.u_all,
-                        self.n)
+            ops.sample(logits, self.temperature, self.top_p, self.top_k, self.u, out=b.ids)
+            ops.decode_tail(None, b.ids, b.pos, b.ctx, self.log, self.counter, self.u, self.u_all, self.n, table, self.x,
+                            self.mirror)
 
     def prepare(self, n_steps: int) -> None:
         """Everything a `run(n_steps)` needs before its first replay, so that a caller who times
@@ -206,7 +225,7 @@ class DecodeLoop:
         if self.graph is None and self.engine.plan is not None:
             # the native step's activations: a buffer of the loop's own, which the captured graphs replay
             # over (the engine's own may be replaced by a larger one when another step needs more)
-            need = self.engine.plan.workspace_bytes(self.batch)
+            need = self.engine.plan.workspace_bytes(self.batch, self.x, self.mirror)
             if self._workspace is None or self._workspace.numel() < need:
                 self._workspace = torch.empty(need, dtype=torch.uint8, device=self.engine.device)
         if self.graph is None:
@@ -218,6 +237,7 @@ class DecodeLoop:
             self._step()
             torch.cuda.synchronize()
             self._dev.copy_(state[0]); self.counter.copy_(state[1]); self.log.copy_(state[2]); arena.copy_(state[3])
+            self._embed()
             if not self.greedy:
                 self.u.copy_(self.u_all[self.steps_done])
             g = torch.cuda.CUDAGraph()

@@ -150,11 +150,13 @@ class Engine:
         widths = [int(info[1 + g]) for g in range(cache.n_groups)]
         return self._stager.stage_native(lib, cache.core, operands, info, widths, int(want_cu[-1]))
 
-    def forward(self, batch: StepBatch, workspace: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def forward(self, batch: StepBatch, workspace: Optional[torch.Tensor] = None, x_in: Optional[torch.Tensor] = None,
+                mirror_in: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """The model's forward pass over a staged batch: one native call when the model has a plan
-        (`workspace`: see `NativePlan.step`), else through the parts."""
+        (`workspace`, `x_in`, `mirror_in`: see `NativePlan.step`), else through the parts."""
         if self.plan is not None:
-            return self.plan.step(batch, workspace)
+            return self.plan.step(batch, workspace, x_in, mirror_in)
+        assert x_in is None, "only the native step takes the rows' embeddings from its caller"
         return self.model.forward(batch, self._views)
 
     def step(self, entries: Sequence[Entry]) -> Optional[torch.Tensor]:

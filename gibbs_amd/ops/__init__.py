@@ -272,6 +272,18 @@ def skinny_store(x: torch.Tensor, w: torch.Tensor, rms_eps: Optional[float] = No
     return out
 
 
+def skinny_store_f32(x: torch.Tensor, w, rms_eps: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """`skinny_store` with float32 output (logits): y = s * (x @ w^T) for at most 64 rows."""
+    n, i, ldx = _skinny_check(x, w, "skinny_store_f32")
+    o = w.shape[0]
+    if out is None:
+        out = torch.empty((n, o), dtype=torch.float32, device=x.device)
+    assert out.shape == (n, o) and out.dtype == torch.float32 and out.is_contiguous()
+    call("gibbs_skinny_store_f32", ptr(x), ptr(_w(w)), ptr(out), n, o, i, ldx, w.stride(0), o, int(rms_eps is not None),
+         float(rms_eps or 0.0), stream())
+    return out
+
+
 def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor, mirror: torch.Tensor) -> None:
     """stream_x += x_in @ w^T (float32 residual stream, in place); mirror = bfloat16(stream_x)."""
     n, i, ldx = _skinny_check(x_in, w, "skinny_residual")
@@ -646,18 +658,32 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
     return out
 
 
-def advance(pos: torch.Tensor, ctx: torch.Tensor, ids: torch.Tensor, log: torch.Tensor, counter: torch.Tensor,
-            u: Optional[torch.Tensor], u_all: Optional[torch.Tensor], n: int) -> None:
-    """End of a decode step on the device: logs the tokens in `ids`, moves pos and ctx on by one,
-    loads the next step's draws and counts the step."""
-    require_cuda(pos, ctx, ids, log, counter, u, u_all)
-    for t, what in ((pos, "pos"), (ctx, "ctx"), (ids, "ids")):
+def decode_tail(logits: Optional[torch.Tensor], ids: torch.Tensor, pos: torch.Tensor, ctx: torch.Tensor, log: torch.Tensor,
+                steps: torch.Tensor, u: Optional[torch.Tensor], u_all: Optional[torch.Tensor], n: int,
+                table: Optional[torch.Tensor] = None, x: Optional[torch.Tensor] = None,
+                mirror: Optional[torch.Tensor] = None) -> None:
+    """End of a decode step on the device, one kernel: with `logits` the rows' next tokens are their first
+    largest logits (else `ids` hold them already); the tokens are logged (log[steps[i], i]), pos and ctx move
+    on by one, the next draws are loaded, steps[i] counts; with `table` and `x` the tokens' embeddings become
+    the rows of the next step's residual stream x [n, hidden] (float32) and of its bfloat16 `mirror`."""
+    require_cuda(logits, ids, pos, ctx, log, steps, u, u_all, table, x, mirror)
+    for t, what in ((pos, "pos"), (ctx, "ctx"), (ids, "ids"), (steps, "steps")):
         _i32(t, n, what)
-    _i32(counter, 1, "counter")
     assert log.dtype == torch.int32 and log.is_contiguous() and log.numel() % n == 0
     capacity = log.numel() // n
+    v = ld = 0
+    if logits is not None:
+        assert logits.dtype == torch.float32 and logits.dim() == 2 and logits.shape[0] == n and logits.stride(1) == 1
+        v, ld = logits.shape[1], logits.stride(0) if n > 1 else logits.shape[1]
     if u is not None:
         assert u.dtype == torch.float32 and u.numel() >= n and u_all is not None
         assert u_all.dtype == torch.float32 and u_all.is_contiguous() and u_all.numel() >= capacity * n
-    call("gibbs_advance", ptr(pos), ptr(ctx), ptr(ids), ptr(log), ptr(counter), ptr(u), ptr(u_all), n, capacity,
-         stream())
+    vocab = hidden = 0
+    if x is not None:
+        assert table is not None and table.dim() == 2 and table.is_contiguous()
+        vocab, hidden = table.shape
+        assert x.dtype == torch.float32 and x.shape == (n, hidden) and x.is_contiguous()
+        assert mirror is None or (mirror.dtype == torch.bfloat16 and mirror.shape == (n, hidden) and mirror.is_contiguous())
+    call("gibbs_decode_tail", ptr(logits), v, ld, ptr(ids), ptr(pos), ptr(ctx), ptr(log), ptr(steps), n, capacity, ptr(u),
+         ptr(u_all), ptr(table), dtype_code(table.dtype) if table is not None else 0, vocab, hidden, ptr(x),
+         ptr(mirror) if x is not None else None, stream())

@@ -54,7 +54,10 @@ _SIGNATURES = {
                          c_void_p],
     "gibbs_attention_plain": [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p, c_void_p],
-    "gibbs_advance": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p],
+    "gibbs_decode_tail": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
+                          c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
+    "gibbs_skinny_store_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_int, c_float,
+                               c_void_p],
     "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
@@ -69,7 +72,8 @@ _SIGNATURES = {
 
 
 _PLAN_SIGNATURES = {
-    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int], c_void_p),
+    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int],
+                          c_void_p),
     "gibbs_plan_destroy": ([c_void_p], None),
     "gibbs_plan_add_block": ([c_void_p, c_void_p, c_float, c_void_p, c_float], c_int),
     "gibbs_plan_set_conv": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
@@ -80,8 +84,6 @@ _PLAN_SIGNATURES = {
     "gibbs_plan_set_glu": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
     "gibbs_plan_workspace": ([c_void_p, c_void_p], c_long),
     "gibbs_plan_step": ([c_void_p, c_void_p], c_int),
-    "gibbs_plan_decode_tail": ([c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                c_void_p, c_void_p, c_void_p, c_void_p, c_void_p], c_int),
 }
 
 

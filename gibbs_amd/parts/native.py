@@ -29,7 +29,8 @@ class StepArgs(ctypes.Structure):
                 ("slot", c_void_p), ("logit_rows", c_void_p), ("tables", c_void_p * MAX_GROUPS),
                 ("widths", c_int * MAX_GROUPS), ("n_rows", c_int), ("n_req", c_int), ("n_logits", c_int),
                 ("max_q", c_int), ("max_seq", c_int), ("lead_single", c_int), ("workspace", c_void_p),
-                ("workspace_bytes", c_long), ("logits", c_void_p), ("stream", c_void_p)]
+                ("workspace_bytes", c_long), ("logits", c_void_p), ("stream", c_void_p), ("x_in", c_void_p),
+                ("mirror_in", c_void_p), ("all_rows_wanted", c_int)]
 
 
 def _ptr(t) -> Optional[int]:
@@ -115,11 +116,12 @@ class NativePlan:
         gain, eps = model.final_norm.native_norm()
         handle = lib.gibbs_plan_create(L.dtype_code(rt.act_dtype), model.spec.hidden, model.spec.vocab, model.table.data_ptr(),
                                        L.dtype_code(model.table.dtype), model.head.data_ptr(), _ptr(model.head_packed),
-                                       _ptr(gain), float(eps), int(rt.fused_decode_rows), int(not lin.USE_LIBRARY_GEMM))
+                                       _ptr(model.head_folded), _ptr(gain), float(eps), int(rt.fused_decode_rows),
+                                       int(not lin.USE_LIBRARY_GEMM))
         if not handle:
             raise KernelError(lib.gibbs_last_error().decode(errors="replace"))
         builder = PlanBuilder(handle, rt)
-        builder.keep += [model.table, model.head, model.head_packed, gain]
+        builder.keep += [model.table, model.head, model.head_packed, model.head_folded, gain]
         plan = cls(handle, builder, model.spec.vocab, rt.device)
         for run, i in enumerate(model.spec.order):
             block = model.blocks[i]
@@ -128,8 +130,10 @@ class NativePlan:
         return plan
 
     # ------------------------------------------------------------------ one step
-    def _fill(self, batch) -> StepArgs:
+    def _fill(self, batch, x_in=None, mirror_in=None) -> StepArgs:
         a = self._args
+        a.x_in, a.mirror_in = _ptr(x_in), _ptr(mirror_in)
+        a.all_rows_wanted = int(batch.all_rows_wanted)
         a.ids, a.pos, a.row_req = batch.ids.data_ptr(), batch.pos.data_ptr(), batch.row_req.data_ptr()
         a.cu, a.ctx, a.slot = batch.cu.data_ptr(), batch.ctx.data_ptr(), batch.slot.data_ptr()
         a.logit_rows = batch.logit_rows.data_ptr() if batch.n_logits else None
@@ -142,19 +146,26 @@ class NativePlan:
         a.stream = L.stream()
         return a
 
-    def workspace_bytes(self, batch) -> int:
+    def workspace_bytes(self, batch, x_in=None, mirror_in=None) -> int:
         lib = L.library()
-        need = lib.gibbs_plan_workspace(self.handle, ctypes.byref(self._fill(batch)))
+        need = lib.gibbs_plan_workspace(self.handle, ctypes.byref(self._fill(batch, x_in, mirror_in)))
         if need < 0:
             raise KernelError(lib.gibbs_last_error().decode(errors="replace"))
         return int(need)
 
-    def step(self, batch, workspace: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    def step(self, batch, workspace: Optional[torch.Tensor] = None, x_in: Optional[torch.Tensor] = None,
+             mirror_in: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Queues the whole step; returns float32 logits [wanted rows, vocab] (None if none are wanted).
         `workspace`: a byte buffer of the caller's that outlives the step's kernels (a captured graph
-        replays over it); default: the plan's own, which grows when a step needs more."""
+        replays over it); default: the plan's own, which grows when a step needs more.  `x_in` (float32
+        [rows, hidden]) and `mirror_in` (its bfloat16 copy): the rows' embeddings, when the end of the
+        previous step has written them already (the step then starts at its first layer and updates
+        them in place)."""
         lib = L.library()
-        a = self._fill(batch)
+        if x_in is not None:
+            assert x_in.dtype == torch.float32 and x_in.is_contiguous() and x_in.shape[0] == batch.n_rows
+            assert mirror_in is None or (mirror_in.dtype == torch.bfloat16 and mirror_in.shape == x_in.shape and mirror_in.is_contiguous())
+        a = self._fill(batch, x_in, mirror_in)
         need = lib.gibbs_plan_workspace(self.handle, ctypes.byref(a))
         if need < 0:
             raise KernelError(lib.gibbs_last_error().decode(errors="replace"))

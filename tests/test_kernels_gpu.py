@@ -707,3 +707,87 @@ def test_attention_block_table_segments():
                                          k_gain=None, eps=0.0, inv_freq=None, rotary_dim=0, variant="half_split",
                                          n_splits=ns)
         close(got, ref, dtype, f"fused decode over segments, {ns} slices", bf16=1e-2)
+
+
+def test_decode_tail_one_kernel():
+    """The end of a captured decode step: next tokens (first largest logit, NaN never wins), the log, positions,
+    cached lengths, draws and per-row step counts, and the tokens' embeddings as the next step's rows."""
+    from gibbs_amd import ops
+    n, V, hidden, cap = 5, 1001, 72, 4
+    logits = rnd(n, V, seed=3)
+    logits[1, 7] = logits[1, 900] = 50.0           # a tie: the first wins
+    logits[2, 3] = float("nan")
+    table = rnd(V, hidden, dtype=torch.bfloat16, seed=4)
+    ids, pos, ctx = i32([9] * n), i32([10, 20, 30, 40, 50]), i32([10, 20, 30, 40, 50])
+    log, steps = torch.full((cap, n), -1, dtype=torch.int32, device=DEV), i32([0, 1, 2, 3, 4])
+    u, u_all = torch.zeros(n, device=DEV), rnd(cap, n, seed=5)
+    x, mirror = torch.zeros(n, hidden, device=DEV), torch.zeros(n, hidden, dtype=torch.bfloat16, device=DEV)
+    ops.decode_tail(logits, ids, pos, ctx, log, steps, u, u_all, n, table, x, mirror)
+    want = torch.nan_to_num(logits, nan=-float("inf")).argmax(-1).int()
+    want[1] = 7
+    assert torch.equal(ids, want) and pos.tolist() == [11, 21, 31, 41, 51] and ctx.tolist() == pos.tolist()
+    assert steps.tolist() == [1, 2, 3, 4, 5]
+    for r in range(n):
+        assert [int(log[s, r]) for s in range(cap)] == [int(want[r]) if s == r else -1 for s in range(cap)]   # row 4: beyond the log
+        assert float(u[r]) == (float(u_all[r + 1, r]) if r + 1 < cap else 0.0)
+    assert torch.equal(x, table[want.long()].float()) and torch.equal(mirror, table[want.long()])
+    # tokens that a sampling kernel has put into ids; no embedding asked for
+    ids2, steps2 = i32([4, 3, 2, 1, 0]), i32([0] * n)
+    ops.decode_tail(None, ids2, pos, ctx, log, steps2, None, None, n)
+    assert log[0].tolist() == [4, 3, 2, 1, 0] and pos.tolist() == [12, 22, 32, 42, 52] and ids2.tolist() == [4, 3, 2, 1, 0]
+
+
+@pytest.mark.parametrize("n,o,i", [(1, 331, 72), (9, 1000, 256), (32, 4096, 512)])
+def test_skinny_store_f32_logits(n, o, i):
+    from gibbs_amd import ops
+    x = rnd(n, i, dtype=torch.bfloat16, scale=2.0, seed=1)
+    w = rnd(o, i, dtype=torch.bfloat16, scale=i ** -0.5, seed=2)
+    for weights in (w, ops.PackedWeight(w)):
+        out = ops.skinny_store_f32(x, weights, rms_eps=1e-5)
+        assert out.dtype == torch.float32
+        scale = torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5)
+        close(out, (x.double() * scale) @ w.double().T, torch.float32, "skinny_store_f32 with rms prologue", f32=2e-5)
+        close(ops.skinny_store_f32(x, weights), x.double() @ w.double().T, torch.float32, "skinny_store_f32", f32=2e-5)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh", "gelu", "relu"])
+def test_activations_of_the_gated_kernels(dtype, activation):
+    """The activation table in the stand-alone kernel (both precisions, vector and scalar variants) and in the
+    epilogue of the fused decode product."""
+    from gibbs_amd import ops
+    act = {"silu": F.silu, "gelu_tanh": lambda g: F.gelu(g, approximate="tanh"), "gelu": F.gelu, "relu": F.relu}[activation]
+    for f in (200, 203):
+        gu = rnd(7, 2 * f, dtype=dtype, scale=2.0, seed=f)
+        close(ops.glu(gu, activation), act(gu[:, :f].double()) * gu[:, f:].double(), dtype, f"glu {activation} {f}")
+    if dtype == torch.bfloat16:
+        x = rnd(5, 96, dtype=dtype, seed=1)
+        w = rnd(2 * 48, 96, dtype=dtype, scale=0.2, seed=2)
+        want = act(x.double() @ w[:48].double().T) * (x.double() @ w[48:].double().T)
+        close(ops.skinny_glu(x, w, activation=activation), want, dtype, f"skinny_glu {activation}")
+    with pytest.raises(ops.KernelError, match="not implemented"):
+        ops.glu(rnd(2, 8, dtype=dtype), "softsign")
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_attention_plain_with_score_slopes(dtype):
+    """A linear bias on the scores by distance: slope[h] * (key position - query position)."""
+    from gibbs_amd import ops
+    nh, nkv, hd, page = 6, 2, 32, 8
+    seq_lens = [70, 9]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 24, seed=3)
+    rows = [(0, list(range(60, 70))), (1, [8])]
+    pos, row_req = i32([p for _, ps in rows for p in ps]), i32([r for r, ps in rows for _ in ps])
+    n = pos.numel()
+    q = rnd(n, nh * hd, dtype=dtype, seed=9)
+    slopes = torch.tensor([0.5 ** (h + 1) for h in range(nh)], dtype=torch.float32, device=DEV)
+    out = ops.attention_plain(q, n, nh, nkv, hd, kp, vp, table, 2, pos, row_req, hd ** -0.5, slopes=slopes)
+    at = 0
+    for r, ps in rows:
+        kk, vv = ks[r].double().repeat_interleave(nh // nkv, 1), vs[r].double().repeat_interleave(nh // nkv, 1)
+        for i, p in enumerate(ps):
+            s = torch.einsum("hd,lhd->hl", q[at + i].double().view(nh, hd), kk[:p + 1]) * hd ** -0.5
+            s = s + slopes.double()[:, None] * (torch.arange(p + 1, device=DEV) - p)[None, :]
+            want = torch.einsum("hl,lhd->hd", s.softmax(-1), vv[:p + 1])
+            close(out[at + i].view(nh, hd), want, dtype, f"slopes request {r} position {p}", f32=2e-5, bf16=1e-2)
+        at += len(ps)
