@@ -44,9 +44,8 @@ struct FusedArgs {
   long ldw, ldx;
   long group_stride;  // rows of W between row groups
   float eps;          // rms prologue
-  // STORE / GLU / CONV: bfloat16 output [N, ldy]; STORE may write float32 instead (Yf: logits)
+  // STORE / GLU / CONV: bfloat16 output [N, ldy]
   bf16* Y;
-  float* Yf;
   long ldy;
   // RESIDUAL
   float* x;   // [N, O] float32, updated in place
@@ -300,10 +299,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       scale = 1.0f / sqrtf(tot / (float)a.I + a.eps);
     }
     const bool full = o + 3 < a.O;
-    if (EPI == EPI_STORE && a.Yf) {
-      float* y = a.Yf + (size_t)n * a.ldy + o;
-      for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = sum[0][t][i] * scale;
-    } else if (EPI == EPI_STORE) {
+    if (EPI == EPI_STORE) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       if (full && a.ldy % 4 == 0) {
         *(bf16x4*)y = bf16x4{(bf16)(sum[0][t][0] * scale), (bf16)(sum[0][t][1] * scale), (bf16)(sum[0][t][2] * scale),
@@ -448,20 +444,6 @@ GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N
   if (rms) launch_nt<1, true, EPI_STORE>(a, stream);
   else launch_nt<1, false, EPI_STORE>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_store");
-}
-
-// The same with float32 output (the head product of a step of decoded tokens: the final norm as the RMS
-// prologue, its gain folded into W, logits out).
-GIBBS_EXPORT int gibbs_skinny_store_f32(const void* X, const void* W, float* Y, int N, int O, int I, long ldx, long ldw,
-                                        long ldy, int rms, float eps, hipStream_t stream) {
-  if (check_common("skinny_store_f32", X, W, N, O, I, ldx, ldw)) return 1;
-  GIBBS_REQUIRE(ldy >= O && Y, "skinny_store_f32: output rows shorter than %d", O);
-  FusedArgs a{};
-  a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
-  a.Yf = Y; a.ldy = ldy;
-  if (rms) launch_nt<1, true, EPI_STORE>(a, stream);
-  else launch_nt<1, false, EPI_STORE>(a, stream);
-  GIBBS_LAUNCH_STATUS("skinny_store_f32");
 }
 
 // x[n, o] += sum_k X[n, k] W[o, k];  xb[n, o] = bfloat16(x[n, o]).  x: [N, O] float32, xb: [N, O] bfloat16.

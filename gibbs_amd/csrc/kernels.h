@@ -60,8 +60,6 @@ int gibbs_attention_decode_fused(const void* qkv, void* kpages, void* vpages, vo
 int gibbs_argmax(const float* logits, int* out, int M, int V, long ld, hipStream_t stream);
 int gibbs_sample(const float* logits, int* out, int M, int V, long ld, const float* temperature, const float* top_p,
                  const int* top_k, const float* u, hipStream_t stream);
-int gibbs_skinny_store_f32(const void* X, const void* W, float* Y, int N, int O, int I, long ldx, long ldw, long ldy,
-                           int rms, float eps, hipStream_t stream);
 int gibbs_decode_tail(const float* logits, int V, long ld, int* ids, int* pos, int* ctx, int* log, int* steps, int n,
                       int capacity, float* u, const float* u_all, const void* table, int table_dtype, int vocab, int hidden,
                       float* x, void* mirror, hipStream_t stream);

@@ -81,7 +81,6 @@ struct Plan {
   const void* table = nullptr;
   int table_dtype = GIBBS_BF16;
   Matrix head;
-  const void* head_folded = nullptr;   // the head in tile order with the final norm's gain multiplied in (bfloat16), or null
   NormP final_norm;
   int fused_rows = 64;      // steps of at most this many decoded tokens take the fused decode kernels
   int own_gemm = 0;         // products above the few-row kernels' range: 0 the library's, 1 the tiled kernel
@@ -115,7 +114,6 @@ struct GibbsStepArgs {
   // decode kernels, its bfloat16 mirror.  Null: the step embeds its ids itself.
   float* x_in;
   void* mirror_in;
-  int all_rows_wanted;     // logit_rows is 0, 1, ..., n_rows - 1
 };
 
 namespace {
@@ -468,12 +466,7 @@ struct Exec {
       }
       if (!ok()) return;
     }
-    if (a.n_logits > 0 && fused_step && a.all_rows_wanted && a.n_logits == N && N <= 32 && p.head_folded && mirror &&
-        pending.parts == 0) {
-      // decoded tokens, every row wanted, the stream settled with its mirror at hand: the final norm is the
-      // head product's RMS prologue (its gain is folded into the head's tile-ordered copy)
-      RUN(gibbs_skinny_store_f32(mirror, p.head_folded, a.logits, N, p.vocab, H, H, 0, p.vocab, 1, p.final_norm.eps, a.stream));
-    } else if (a.n_logits > 0) {
+    if (a.n_logits > 0) {
       void* h = norm(x, pending, p.final_norm, a.logit_rows, a.n_logits);
       const int M = a.n_logits, V = p.vocab;
       // the head: float32 logits straight into the caller's buffer
@@ -510,8 +503,8 @@ int check_args(const Plan* p, const GibbsStepArgs* a) {
 
 // ------------------------------------------------------------------------------------------------- building a plan
 GIBBS_EXPORT void* gibbs_plan_create(int dtype, int hidden, int vocab, const void* table, int table_dtype, const void* head,
-                                     const void* head_packed, const void* head_folded, const float* final_gain,
-                                     float final_eps, int fused_rows, int own_gemm) {
+                                     const void* head_packed, const float* final_gain, float final_eps, int fused_rows,
+                                     int own_gemm) {
   if ((dtype != GIBBS_BF16 && dtype != GIBBS_F32) || hidden <= 0 || vocab <= 0 || !table || !head) {
     gibbs_fail("plan: bad model sizes or no token table");
     return nullptr;
@@ -520,7 +513,6 @@ GIBBS_EXPORT void* gibbs_plan_create(int dtype, int hidden, int vocab, const voi
   Plan* p = new Plan();
   p->dtype = dtype; p->hidden = hidden; p->vocab = vocab; p->table = table; p->table_dtype = table_dtype;
   p->head.w = head; p->head.packed = head_packed; p->head.O = vocab; p->head.I = hidden;
-  p->head_folded = (dtype == GIBBS_BF16 && hidden % 8 == 0) ? head_folded : nullptr;
   p->final_norm = NormP{final_gain, final_eps};
   p->fused_rows = fused_rows; p->own_gemm = own_gemm;
   return p;

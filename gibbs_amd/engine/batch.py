@@ -44,7 +44,6 @@ class StepBatch:
     max_q: int = 0
     max_seq: int = 0
     lead_single: int = 0         # requests at the head of the batch that bring one token each (decoded tokens)
-    all_rows_wanted: bool = False  # logit_rows is 0, 1, ..., n_rows - 1 (every row's logits, in order)
     decode_graph: bool = False   # metadata lives in static buffers that a captured graph replays over
 
 
@@ -107,8 +106,7 @@ class BatchStager:
             q_lens=q_lens, ctx_lens=view[int(offsets[4]):int(offsets[4]) + n].tolist(),
             slots=view[int(offsets[5]):int(offsets[5]) + n].tolist(),
             max_q=int(offsets[7 + len(widths)]), max_seq=int(offsets[8 + len(widths)]),
-            lead_single=leading_single(q_lens),
-            all_rows_wanted=n_logits == rows and bool((view[int(offsets[6]):int(offsets[6]) + rows] == np.arange(rows)).all()))
+            lead_single=leading_single(q_lens))
 
     def stage(self, ids: np.ndarray, pos: np.ndarray, row_req: np.ndarray, cu: np.ndarray, ctx: np.ndarray,
               slot: np.ndarray, logit_rows: np.ndarray, tables: Sequence[np.ndarray]) -> StepBatch:
@@ -135,5 +133,4 @@ class BatchStager:
             tables=[s.view(t.shape) for s, t in zip(sec[7:], tables)],
             q_lens=q_lens.tolist(), ctx_lens=ctx.tolist(), slots=slot.tolist(),
             max_q=int(q_lens.max()) if n_req else 0, max_seq=int((ctx + q_lens).max()) if n_req else 0,
-            lead_single=leading_single(q_lens.tolist()),
-            all_rows_wanted=logit_rows.size == ids.size and bool((logit_rows == np.arange(ids.size)).all()))
+            lead_single=leading_single(q_lens.tolist()))

@@ -6,8 +6,7 @@ device buffers.  What changes between steps (positions, cached lengths, the samp
 draws) is updated by a kernel at the end of the step, so a replay needs no host work; pages for all
 steps of a `run` are reserved, and the block tables uploaded, before the first of them.  With the
 native step that same kernel also writes the sampled tokens' embeddings as the next step's residual
-rows, so a step is: layers, head (the final norm as its prologue), one kernel for argmax, log, advance
-and embedding.
+rows, so a step is: layers, final norm, head, and one kernel for argmax, log, advance and embedding.
 """
 from __future__ import annotations
 
@@ -85,7 +84,7 @@ class DecodeLoop:
             n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
             cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
             tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
-            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True, all_rows_wanted=True)
+            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True)
         self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
         self.counter = torch.zeros(b, dtype=torch.int32, device=dev)          # steps done, per row
         # native step: the rows of the residual stream (and their bfloat16 mirror) live here from one step to

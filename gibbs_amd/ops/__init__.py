@@ -272,18 +272,6 @@ def skinny_store(x: torch.Tensor, w: torch.Tensor, rms_eps: Optional[float] = No
     return out
 
 
-def skinny_store_f32(x: torch.Tensor, w, rms_eps: Optional[float] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """`skinny_store` with float32 output (logits): y = s * (x @ w^T) for at most 64 rows."""
-    n, i, ldx = _skinny_check(x, w, "skinny_store_f32")
-    o = w.shape[0]
-    if out is None:
-        out = torch.empty((n, o), dtype=torch.float32, device=x.device)
-    assert out.shape == (n, o) and out.dtype == torch.float32 and out.is_contiguous()
-    call("gibbs_skinny_store_f32", ptr(x), ptr(_w(w)), ptr(out), n, o, i, ldx, w.stride(0), o, int(rms_eps is not None),
-         float(rms_eps or 0.0), stream())
-    return out
-
-
 def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor, mirror: torch.Tensor) -> None:
     """stream_x += x_in @ w^T (float32 residual stream, in place); mirror = bfloat16(stream_x)."""
     n, i, ldx = _skinny_check(x_in, w, "skinny_residual")

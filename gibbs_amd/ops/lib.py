@@ -56,8 +56,6 @@ _SIGNATURES = {
                               c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_void_p, c_void_p],
     "gibbs_decode_tail": [c_void_p, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
                           c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p],
-    "gibbs_skinny_store_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_int, c_float,
-                               c_void_p],
     "gibbs_attention_decode": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
@@ -72,8 +70,7 @@ _SIGNATURES = {
 
 
 _PLAN_SIGNATURES = {
-    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int],
-                          c_void_p),
+    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int], c_void_p),
     "gibbs_plan_destroy": ([c_void_p], None),
     "gibbs_plan_add_block": ([c_void_p, c_void_p, c_float, c_void_p, c_float], c_int),
     "gibbs_plan_set_conv": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,

@@ -72,14 +72,6 @@ class DecoderModel(Part):
         self.head = weights[self.spec.head] if self.spec.head is not None else self.table
         self.head_packed = ops.PackedWeight(self.head) if rt.act_dtype == torch.bfloat16 else None
         self.final_norm.bind(weights, rt)
-        # for steps of decoded tokens: a tile-ordered copy of the head with the final norm's gain multiplied into
-        # its columns, so that the norm becomes the head product's RMS prologue (the norm keeps its gain for
-        # every other step)
-        self.head_folded = None
-        gain = getattr(self.final_norm, "gain", None)
-        if (rt.act_dtype == torch.bfloat16 and rt.fold_gains and hasattr(self.final_norm, "native_norm") and gain is not None
-                and self.spec.hidden % 8 == 0):
-            self.head_folded = ops.PackedWeight((self.head.float() * gain[None, :]).to(torch.bfloat16))
         for b in self.blocks:
             b.bind(weights, rt)
 
@@ -97,9 +89,5 @@ class DecoderModel(Part):
             stream = self.blocks[i].forward(stream, batch, caches[run])
         if batch.n_logits == 0:
             return None
-        if (self.head_folded is not None and fused_decode_step(self.rt, batch) and batch.all_rows_wanted and batch.n_rows <= 32
-                and stream.pending is None and stream.mirror is not None):
-            # every row wanted, the stream settled with its mirror at hand: the final norm as the head product's prologue
-            return ops.skinny_store_f32(stream.mirror, self.head_folded, rms_eps=self.final_norm.spec.eps)
         h = stream.normed(self.final_norm, batch.logit_rows, batch.n_logits)
         return linear(h, self.head, out_dtype=torch.float32, packed=self.head_packed)

@@ -30,7 +30,7 @@ class StepArgs(ctypes.Structure):
                 ("widths", c_int * MAX_GROUPS), ("n_rows", c_int), ("n_req", c_int), ("n_logits", c_int),
                 ("max_q", c_int), ("max_seq", c_int), ("lead_single", c_int), ("workspace", c_void_p),
                 ("workspace_bytes", c_long), ("logits", c_void_p), ("stream", c_void_p), ("x_in", c_void_p),
-                ("mirror_in", c_void_p), ("all_rows_wanted", c_int)]
+                ("mirror_in", c_void_p)]
 
 
 def _ptr(t) -> Optional[int]:
@@ -116,12 +116,11 @@ class NativePlan:
         gain, eps = model.final_norm.native_norm()
         handle = lib.gibbs_plan_create(L.dtype_code(rt.act_dtype), model.spec.hidden, model.spec.vocab, model.table.data_ptr(),
                                        L.dtype_code(model.table.dtype), model.head.data_ptr(), _ptr(model.head_packed),
-                                       _ptr(model.head_folded), _ptr(gain), float(eps), int(rt.fused_decode_rows),
-                                       int(not lin.USE_LIBRARY_GEMM))
+                                       _ptr(gain), float(eps), int(rt.fused_decode_rows), int(not lin.USE_LIBRARY_GEMM))
         if not handle:
             raise KernelError(lib.gibbs_last_error().decode(errors="replace"))
         builder = PlanBuilder(handle, rt)
-        builder.keep += [model.table, model.head, model.head_packed, model.head_folded, gain]
+        builder.keep += [model.table, model.head, model.head_packed, gain]
         plan = cls(handle, builder, model.spec.vocab, rt.device)
         for run, i in enumerate(model.spec.order):
             block = model.blocks[i]
@@ -133,7 +132,6 @@ class NativePlan:
     def _fill(self, batch, x_in=None, mirror_in=None) -> StepArgs:
         a = self._args
         a.x_in, a.mirror_in = _ptr(x_in), _ptr(mirror_in)
-        a.all_rows_wanted = int(batch.all_rows_wanted)
         a.ids, a.pos, a.row_req = batch.ids.data_ptr(), batch.pos.data_ptr(), batch.row_req.data_ptr()
         a.cu, a.ctx, a.slot = batch.cu.data_ptr(), batch.ctx.data_ptr(), batch.slot.data_ptr()
         a.logit_rows = batch.logit_rows.data_ptr() if batch.n_logits else None

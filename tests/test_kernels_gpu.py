@@ -737,19 +737,6 @@ def test_decode_tail_one_kernel():
     assert log[0].tolist() == [4, 3, 2, 1, 0] and pos.tolist() == [12, 22, 32, 42, 52] and ids2.tolist() == [4, 3, 2, 1, 0]
 
 
-@pytest.mark.parametrize("n,o,i", [(1, 331, 72), (9, 1000, 256), (32, 4096, 512)])
-def test_skinny_store_f32_logits(n, o, i):
-    from gibbs_amd import ops
-    x = rnd(n, i, dtype=torch.bfloat16, scale=2.0, seed=1)
-    w = rnd(o, i, dtype=torch.bfloat16, scale=i ** -0.5, seed=2)
-    for weights in (w, ops.PackedWeight(w)):
-        out = ops.skinny_store_f32(x, weights, rms_eps=1e-5)
-        assert out.dtype == torch.float32
-        scale = torch.rsqrt(x.double().pow(2).mean(-1, keepdim=True) + 1e-5)
-        close(out, (x.double() * scale) @ w.double().T, torch.float32, "skinny_store_f32 with rms prologue", f32=2e-5)
-        close(ops.skinny_store_f32(x, weights), x.double() @ w.double().T, torch.float32, "skinny_store_f32", f32=2e-5)
-
-
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("activation", ["silu", "gelu_tanh", "gelu", "relu"])
 def test_activations_of_the_gated_kernels(dtype, activation):
