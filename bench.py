@@ -175,7 +175,7 @@ def suite_rows(path: str) -> list:
         ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
         entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
         try:
-            rows.append({"serve": S.serve, "products": S.products}.get(entry.get("workload", "decode"), S.measure)(entry, base))
+            rows.append({"serve": S.serve, "products": S.products, "mixed": S.mixed}.get(entry.get("workload", "decode"), S.measure)(entry, base))
         except Exception as exc:
             rows.append({"model": entry["name"], "error": f"{type(exc).__name__}: {exc}"})
         gc.collect()

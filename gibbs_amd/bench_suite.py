@@ -19,6 +19,10 @@ model entry inherits the defaults; the keys that mean something here:
                     `max_requests` live at a time (default: all), prompts cut into portions of at
                     most `chunk` tokens (default: none) under `max_batch_tokens` (default 2048) per
                     step; the row reports generated and prompt tokens a second over the whole run;
+                    or "mixed": `batch` requests with `prefill_tokens` cached tokens each decode one token
+                    per step beside a prompt portion of `portion` tokens of one more request, through
+                    `Engine.step` (no captured graph: what a scheduler step costs); the row reports the
+                    wall time of a step and the time after which the host is through with queueing it;
                     or "products": every distinct matrix of the model's layers against `rows`
                     (default 2048) rows of activations, the library's product and the hand-written
                     tiled kernel side by side (`only`: "library" or "own" keeps one of them, for a
@@ -242,6 +246,37 @@ def products(entry: Dict, base: str) -> Dict:
     return {"model": entry["name"], "workload": "products", "dtype": "bfloat16", "rows": rows, "products": cells}
 
 
+def mixed(entry: Dict, base: str) -> Dict:
+    """Steps that hold decoded tokens beside a prompt portion, one after the other without waiting for
+    their logits: wall time per step, and how long the host needs to queue one."""
+    import numpy as np
+    import torch
+    n_dec, portion, cached, steps = (int(entry.get(k, d)) for k, d in (("batch", 64), ("portion", 64), ("prefill_tokens", 512),
+                                                                         ("steps", 16)))
+    ctx = -(-(cached + (steps + 4) * max(portion, 1) + 64) // 64) * 64
+    engine = _load(entry, base, batch=n_dec + 1, ctx=ctx)
+    rng = np.random.default_rng(0)
+    vocab = engine.spec.vocab
+    rids = [f"d{i}" for i in range(n_dec)]
+    for r in rids:
+        engine.step([(r, rng.integers(0, vocab, cached).tolist(), [])])
+    engine.step([("p", rng.integers(0, vocab, cached).tolist(), [])])
+    feeds = [[(r, [int(t)], [0]) for r, t in zip(rids, rng.integers(0, vocab, n_dec))]
+             + ([("p", rng.integers(0, vocab, portion).tolist(), [portion - 1])] if portion else []) for _ in range(steps + 3)]
+    for f in feeds[:3]:
+        engine.step(f)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for f in feeds[3:]:
+        engine.step(f)
+    host = time.perf_counter() - t0
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return {"model": entry["name"], "workload": "mixed", "dtype": entry["dtype"], "decoding": n_dec, "portion": portion,
+            "rows": n_dec + portion, "cached_tokens": cached, "native_step": engine.plan is not None,
+            "ms_per_step": round(1e3 * wall / steps, 4), "host_ms_per_step": round(1e3 * host / steps, 4)}
+
+
 def _serve_row(entry, n_req, live, n_prompt, n_decode, chunk, done, wall, generated, st) -> dict:
     return {"model": entry["name"], "workload": "serve", "dtype": entry["dtype"], "requests": n_req, "live": live,
             "prompt_tokens": n_prompt, "decode_tokens": n_decode, "chunk": chunk,
@@ -276,7 +311,7 @@ def run_suite(path: str) -> int:
         entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
         try:
             workload = entry.get("workload", "decode")
-            row = {"serve": serve, "products": products}.get(workload, measure)(entry, base)
+            row = {"serve": serve, "products": products, "mixed": mixed}.get(workload, measure)(entry, base)
         except Exception as e:     # one model's failure is reported; the others still run (bench.rs:751)
             print(f"gibbs --bench: {entry['name']}: {type(e).__name__}: {e}", file=sys.stderr)
             failed = True
