@@ -8,6 +8,7 @@
 // blocks alone cannot fill the chip, k is also split over workgroups (`k_splits`), each writing
 // its float32 partial Y[s] for the consumer to add in a fixed order.
 #include "common.h"
+#include "packed_layout.h"
 
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -21,7 +22,7 @@ constexpr int WAVES = 8;
 template <int NT, int FT, int OUT>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ W, const bf16* __restrict__ X,
                                                           void* __restrict__ Yv, int N, int O, int I, long ldw,
-                                                          long ldx, long ldy, int k_per_block, long split_stride) {
+                                                          long ldx, long ldy, int k_per_block, long split_stride, bool pair) {
   static_assert(FT <= WAVES, "wave f finishes tile f");
   // More than 16 rows of X: a wave brings its part of X in through LDS (its own region: no barrier),
   // 128 contiguous bytes or more of a row per request instead of the 64 that a lane group of an MFMA
@@ -45,20 +46,24 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
   const int k_begin = kb0 + wave * per_wave * 32;
   const int k_end = min(kb1, k_begin + per_wave * 32);
 
-  // ldw == 0: W is in tile order (pack_weight): [ceil(O/16)][ceil(I/32)][64 lanes][8], a wave's A
-  // operand 1 KB of consecutive memory
+  // ldw == 0: W is in tile order (packed_layout.h; which of the two orders follows from O), a wave's A
+  // operand 1 KB of consecutive memory (pair layout read here by 16 features: 8 pieces of 128 bytes)
   const bool packed = ldw == 0;
-  const int ktiles = (I + 31) / 32;
+  const bool pairs = packed && pair;
+  const int ktiles = pairs ? (I + 63) / 64 : (I + 31) / 32;
   bool row_ok[FT];
   const bf16* wrow[FT];
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     row_ok[f] = o0 + f * 16 + r < O;
-    wrow[f] = packed ? W + ((size_t)(o0 / 16 + f) * ktiles) * 512 + lane * 8
-                     : W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
+    wrow[f] = pairs    ? W + ((size_t)(2 * (o0 / 16 + f) + r / 8) * ktiles) * 512 + (g * 16 + r % 8) * 8
+              : packed ? W + ((size_t)(o0 / 16 + f) * ktiles) * 512 + lane * 8
+                       : W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
   }
   const int kstride = packed ? 512 : 32;
   const int koff = packed ? 0 : g * 8;
+  // elements from wrow to the lane's A operand of 32-k tile j
+  auto a_off = [&](int j) { return pairs ? (size_t)(j >> 1) * 512 + (j & 1) * 64 : (size_t)j * kstride; };
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -112,7 +117,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
         const int kk = k + u * 32;
 #pragma unroll
         for (int f = 0; f < FT; ++f)
-          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
+          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + a_off(kk / 32)) : zero;
       }
 #pragma unroll
       for (int t = 0; t < NT; ++t)
@@ -129,7 +134,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
         const bool k_ok = kk + g * 8 < k_end;
 #pragma unroll
         for (int f = 0; f < FT; ++f)
-          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + (size_t)(kk / 32) * kstride) : zero;
+          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + a_off(kk / 32)) : zero;
 #pragma unroll
         for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
       }
@@ -191,17 +196,17 @@ void launch(int out, int ft, int n_out, int k_splits, hipStream_t s, const bf16*
     if (ft == 4) {
       dim3 grid(ceil_div(n_out, 64), k_splits);
       if (out == OUT_BF16)
-        gemm_skinny_kernel<NT, 4, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+        gemm_skinny_kernel<NT, 4, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss, ldw == 0 && pair_layout(O));
       else
-        gemm_skinny_kernel<NT, 4, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+        gemm_skinny_kernel<NT, 4, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss, ldw == 0 && pair_layout(O));
       return;
     }
   }
   dim3 grid(ceil_div(n_out, 16), k_splits);
   if (out == OUT_BF16)
-    gemm_skinny_kernel<NT, 1, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+    gemm_skinny_kernel<NT, 1, OUT_BF16><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss, ldw == 0 && pair_layout(O));
   else
-    gemm_skinny_kernel<NT, 1, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss);
+    gemm_skinny_kernel<NT, 1, OUT_F32><<<grid, WAVES * WAVE, 0, s>>>(W, X, Y, N, O, I, ldw, ldx, ldy, kpb, ss, ldw == 0 && pair_layout(O));
 }
 }  // namespace
 

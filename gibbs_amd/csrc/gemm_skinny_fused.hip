@@ -6,10 +6,18 @@
 //   v_mfma_f32_16x16x32_bf16, the workgroup's waves splitting k and meeting in LDS, as in
 //   gemm_skinny.  On top of that:
 //
-//   packed W      W may come in MFMA-tile order (`pack_weight`: [row group][16-row tile][32-k tile][lane][8],
-//                  zero-padded): a wave's load of an A operand is then 1 KB of consecutive memory, 8 requests
-//                  of 128 bytes instead of 16 of 64, which is worth a fifth of the time of these products
-//                  (the compute unit's memory pipe is bound by requests in flight, not by bytes).
+//   packed W      W may come in MFMA-tile order (packed_layout.h: 16-row tiles, or 8-row tiles of two k tiles
+//                  for matrices of few rows, zero-padded): a wave's load of an A operand is then 1 KB of
+//                  consecutive memory, 8 requests of 128 bytes instead of 16 of 64, which is worth a fifth of
+//                  the time of these products (the compute unit's memory pipe is bound by requests in flight,
+//                  not by bytes).
+//   8 features     Where 16 features per workgroup would leave compute units idle, a workgroup takes 8, and the
+//                  other 8 rows of its A operands hold the same 8 features at the NEXT 32 values of k: the
+//                  operand's product with X at k fills rows 0..7 of one accumulator, its product with X at
+//                  k + 32 rows 8..15 of a second one, and the two halves are added at the end.  One load of
+//                  1 KB then serves two MFMA steps, and it is consecutive memory in the pair layout (two
+//                  workgroups that read alternate 128-byte pieces of the same tiles were measured a quarter
+//                  slower than one that reads them whole).
 //   prologue RMS   the rows of X are the bfloat16 mirror of the residual stream; the workgroup sums
 //                  their squares from the B operands it loads anyway and scales its outputs by
 //                  1/sqrt(mean(x^2) + eps).  The norm's gain is folded into W when weights are bound.
@@ -23,7 +31,9 @@
 //                  CONV      bx = B * x;  cv = bias + taps . [state, bx];  y = C * cv;  state shifts
 //                            (every row is one decoded token of a different request)
 #include "activation.h"
+#include "packed_layout.h"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -36,8 +46,8 @@ constexpr int MAX_TAPS = 8;
 struct FusedArgs {
   int rotate;     // 1: workgroups start at different k (see the kernel)
   const bf16* W;
-  int packed;        // W is in tile order
-  int ktiles;        // packed: 32-k tiles per 16-row tile
+  int packed;        // W is in tile order: 1 = 16-row tiles, 2 = 8-row tiles of two k tiles (packed_layout.h)
+  int ktiles;        // packed: 32-k tiles per 16-row tile (pair layout: 64-k pairs per 8-row tile)
   long group_tiles;  // packed: 16-row tiles per row group
   const bf16* X;   // [N, I] bfloat16 (the mirror of the residual stream when rms)
   int N, O, I;     // O: features per row group
@@ -66,13 +76,14 @@ struct FusedArgs {
 // FT: tiles of ROWS features that a workgroup computes from the same B operands (more rows of X
 // than one or two MFMA tiles: X is re-read from L2 by every workgroup, so a workgroup should use
 // each B operand for more of W).  Wave f sums tile f over the waves and runs its epilogue.
-template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC>
+template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC, bool STAGE, bool BP = false>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
   static_assert(FT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only");
-  // More than 16 rows of X: a wave brings its part of X in through LDS, 128 contiguous bytes or more of
-  // a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory pipe
-  // of a compute unit is bound by requests in flight).  The wave's region is its own: no barrier.
-  constexpr bool STAGE = NT >= 2;
+  // STAGE (more than a few rows of X): a wave brings its part of X in through LDS, 128 contiguous bytes or
+  // more of a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory
+  // pipe of a compute unit is bound by requests in flight, and from 8 rows on X is as many requests as W
+  // for a workgroup of 8 features).  The wave's region is its own: no barrier.
+  static_assert(STAGE || NT == 1, "more than 16 rows of X are staged");
   constexpr int U = (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);  // MFMA steps per iteration
   constexpr int CH = 4 * U;                    // 16-byte chunks of a row per iteration
   constexpr int RED_BYTES = WAVES * FT * RG * NT * WAVE * 16;
@@ -84,36 +95,67 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int r = lane % 16, g = lane / 16;
   const int o0 = blockIdx.x * ROWS * FT;
-  // the wave's share of k, in whole MFMA steps of 32
-  const int steps = (a.I + 31) / 32;
+  // the wave's share of k, in whole MFMA steps of 32 (workgroups of 8 features: in pairs of steps)
+  constexpr bool PAIR = ROWS == 8;
+  constexpr int KU = PAIR ? 64 : 32;
+  static_assert(!PAIR || FT == 1, "8 features: one tile per workgroup");
+  // BP (8 features and at most 8 rows of X): the B operands are pairs as well, rows 8..15 holding the same 8 rows
+  // of X at the next 32 values of k.  One MFMA then does two steps: the upper left 8 x 8 block of its result is
+  // the product at k, the lower right one the product at k + 32 (the other two blocks mix the two and are
+  // dropped).  A load of X is 8 requests of 128 bytes instead of two loads of 8 requests of 64.
+  static_assert(!BP || (PAIR && NT == 1 && !STAGE), "paired B operands: 8 features, one tile of rows, not staged");
+  const int steps = (a.I + KU - 1) / KU;
   const int per_wave = (steps + WAVES - 1) / WAVES;
-  const int k_begin = wave * per_wave * 32;
-  const int k_end = min(a.I, k_begin + per_wave * 32);
+  const int k_begin = wave * per_wave * KU;
+  const int k_end = min(a.I, k_begin + per_wave * KU);
 
+  // Where a lane's A operands lie: wrow + a_off(step), the step being the number of the 32-k tile (pairs: of
+  // the 64-k pair) from the start of k.  One expression for all layouts, so that no branch stands between loads:
+  //   j = min(step * a_unit + koff, a_limit);  offset = (j >> a_sh) * a_mul + (j & a_sh) * 64 - koff
+  //   16-row tiles: tile j, 512 elements each.  Pair layout read by 16 features: pair j / 2, half j % 2.
+  //   Row-major: element j of the row (a_unit elements per step).
   bool row_ok[FT];
   const bf16* wrow[FT][RG];
+  int koff = 0, a_unit = 1, a_sh = 0, a_mul = 512;
+  int a_limit = (k_end - 1) / KU;
+  const int r8 = r % 8, half = r / 8;
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     row_ok[f] = r < ROWS && o0 + f * ROWS + r < a.O;
 #pragma unroll
-    for (int q = 0; q < RG; ++q)
-      if (a.packed) {
-        // 16-row tile of the feature tile, and this lane's place in it (8-row workgroups take half a tile)
-        const int o_tile = (o0 + f * ROWS) / 16;
-        const int in_tile = ROWS == 16 ? lane : g * 16 + ((o0 / 8) % 2) * 8 + (r % 8);
-        wrow[f][q] = a.W + (((size_t)q * a.group_tiles + o_tile) * a.ktiles) * 512 + in_tile * 8;
+    for (int q = 0; q < RG; ++q) {
+      if (a.packed == 2) {
+        // 8-row tiles of two k tiles: [row group][8-row tile][pair][g][half][r8][8]
+        const size_t tiles8 = 2 * a.group_tiles;
+        if (PAIR) {
+          wrow[f][q] = a.W + ((q * tiles8 + o0 / 8) * a.ktiles) * 512 + lane * 8;
+        } else {
+          const size_t o8 = min((size_t)(o0 + f * ROWS) / 8 + half, tiles8 - 1);   // (beyond the last tile: unused rows)
+          wrow[f][q] = a.W + ((q * tiles8 + o8) * a.ktiles) * 512 + (g * 16 + r8) * 8;
+          a_sh = 1;
+        }
+      } else if (a.packed) {
+        // 16-row tiles (never read by workgroups of 8 features: the layout follows the number of rows)
+        const int o_tile = min((o0 + f * ROWS) / 16, (int)a.group_tiles - 1);   // (beyond the last tile: unused rows)
+        wrow[f][q] = a.W + (((size_t)q * a.group_tiles + o_tile) * a.ktiles) * 512 + lane * 8;
       } else {
-        wrow[f][q] = a.W + ((size_t)q * a.group_stride + (row_ok[f] ? o0 + f * ROWS + r : 0)) * a.ldw + g * 8;
+        const int row = PAIR ? (o0 + r8 < a.O ? o0 + r8 : 0) : (row_ok[f] ? o0 + f * ROWS + r : 0);
+        koff = (PAIR ? half * 32 : 0) + g * 8;
+        wrow[f][q] = a.W + ((size_t)q * a.group_stride + row) * a.ldw + koff;
+        a_unit = KU; a_limit = a.I - 8; a_mul = 1;
       }
+    }
   }
-  const int kstride = a.packed ? 512 : 32;  // elements between a lane's A operands of consecutive MFMA steps
-  const int koff = a.packed ? 0 : g * 8;    // packed tiles are whole (zero-padded)
+  auto a_off = [&](int step) {
+    const int j = min(step * a_unit + koff, a_limit);
+    return (long)(j >> a_sh) * a_mul + (j & a_sh) * 64 - koff;
+  };
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    x_ok[t] = t * 16 + r < a.N;
-    xrow[t] = a.X + (size_t)(x_ok[t] ? t * 16 + r : 0) * a.ldx + g * 8;
+    x_ok[t] = BP ? r8 < a.N : t * 16 + r < a.N;
+    xrow[t] = a.X + (size_t)(x_ok[t] ? (BP ? r8 : t * 16 + r) : 0) * a.ldx + (BP ? half * 32 : 0) + g * 8;
   }
   // What the epilogue reads besides the product is asked for now: the product hides the latency
   // (the state row hangs on a slot index, two dependent loads).  Wave 0 writes the outputs; its lane
@@ -155,14 +197,17 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 
   floatx4 acc[FT][RG][NT];
-  float ss[NT];
+  floatx4 acc_hi[PAIR ? RG : 1][NT];   // 8 features: the products with X at k + 32 (rows 8..15 hold the features)
+  floatx4 gram[NT];   // RMS: X X^T of the tile's rows (its diagonal is the rows' sums of squares)
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    ss[t] = 0.f;
+    gram[t] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int f = 0; f < FT; ++f)
 #pragma unroll
       for (int q = 0; q < RG; ++q) acc[f][q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int q = 0; q < (PAIR ? RG : 1); ++q) acc_hi[q][t] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -193,97 +238,156 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   // ranges and wraps around (the order of a feature's additions is fixed by its workgroup).
   const int n_iter = (k_end - k_begin + 32 * U - 1) / (32 * U);
   const int first_iter = (STAGE && n_iter > 0 && a.rotate) ? (int)(blockIdx.x % n_iter) : 0;
-  for (int it = 0; it < n_iter; ++it) {
-    const int k = k_begin + ((it + first_iter) % n_iter) * 32 * U;
-    bf16x8 av[U][FT][RG], bv[U][NT];
+  auto k_of = [&](int it) { return k_begin + ((it + first_iter) % n_iter) * 32 * U; };
+
+  // Operands live in registers for one iteration of U MFMA steps.  As soon as a step's operands have been
+  // used, the same registers are asked for the next iteration's step: a wave keeps U steps of loads in
+  // flight all the time instead of waiting for an iteration's loads, working on them and asking again.
+  // Every load is unconditional and its value is used as it comes (a load under a branch of its own, or a
+  // select right behind it, makes the wave wait for all its loads in flight at once): addresses are clamped
+  // into the matrices.  Rows of X beyond N give columns of the product that nobody stores.  Where k is beyond
+  // the wave's range, which only the last stretch of the range can be, the rows of X are made zero before
+  // they are used, so that whatever W holds there adds nothing.
+  constexpr int UA = PAIR ? U / 2 : U;   // A operands per iteration (8 features: one serves two MFMA steps)
+  constexpr int UB = BP ? U / 2 : U;     // B operands per iteration
+  static_assert(U % 2 == 0, "pairs of MFMA steps");
+  const int xoff = (BP ? half * 32 : 0) + g * 8;   // a lane's k within a B operand
+  bf16x8 av[UA][FT][RG], bv[UB][NT], sv[NT][LPT];
+  auto load_a = [&](int k, int u) {   // u: the iteration's A operand
+    const long off = a_off(k / KU + u);
+#pragma unroll
+    for (int f = 0; f < FT; ++f)
+#pragma unroll
+      for (int q = 0; q < RG; ++q) av[u][f][q] = *(const bf16x8*)(wrow[f][q] + off);
+  };
+  auto load_b = [&](int k, int u) {
+    const int kc = min(k + u * (BP ? 64 : 32) + xoff, a.I - 8) - xoff;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) bv[u][t] = *(const bf16x8*)(xrow[t] + kc);
+  };
+  auto load_s = [&](int k) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int kc = min(k + s_chunk[i] * 8, a.I - 8) - s_chunk[i] * 8;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) sv[t][i] = *(const bf16x8*)(srow[t][i] + kc);
+    }
+  };
+  // One iteration on the operands of stretch k; `more`: the next stretch k_next is asked for.  `ragged`: k may
+  // run beyond the wave's range within this stretch.
+  auto iteration = [&](int k, int k_next, auto more, auto ragged) {
     if (STAGE) {
-      bf16x8 sv[NT][LPT];
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int i = 0; i < LPT; ++i) {
+        const bool k_ok = !ragged || k + s_chunk[i] * 8 < k_end;
 #pragma unroll
-        for (int i = 0; i < LPT; ++i)
-          sv[t][i] = (s_ok[t][i] && k + s_chunk[i] * 8 < k_end) ? *(const bf16x8*)(srow[t][i] + k) : zero;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kk = k + u * 32;
-#pragma unroll
-        for (int f = 0; f < FT; ++f)
-#pragma unroll
-          for (int q = 0; q < RG; ++q)
-            av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
+        for (int t = 0; t < NT; ++t) stage[(t * LPT + i) * WAVE + lane] = k_ok ? sv[t][i] : zero;
       }
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) stage[(t * LPT + i) * WAVE + lane] = sv[t][i];
+      if (more) load_s(k_next);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int t = 0; t < NT; ++t) bv[u][t] = stage[t * 16 * CH + read_slot[u]];
+    }
+    if constexpr (BP) {
+#pragma unroll
+      for (int u = 0; u < UB; ++u) {
+        bf16x8 b = bv[u][0];
+        if (ragged && !(k + u * 64 + xoff < k_end)) b = zero;
+        if (RMS) gram[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, b, gram[0], 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][0][q], b, acc[0][q][0], 0, 0, 0);
+        if (more) {
+          load_a(k_next, u);
+          load_b(k_next, u);
+        }
+      }
     } else {
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kk = k + u * 32;
-        const bool k_ok = kk + g * 8 < k_end;
-#pragma unroll
-        for (int f = 0; f < FT; ++f)
-#pragma unroll
-          for (int q = 0; q < RG; ++q)
-            av[u][f][q] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f][q] + (size_t)(kk / 32) * kstride) : zero;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) bv[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
-      }
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
       for (int t = 0; t < NT; ++t) {
-        if (RMS) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const float v = (float)bv[u][t][e];
-            ss[t] = fmaf(v, v, ss[t]);
-          }
-        }
+        bf16x8 b = bv[u][t];
+        if (!STAGE && ragged && !(k + u * 32 + g * 8 < k_end)) b = zero;
+        if (RMS) gram[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, b, gram[t], 0, 0, 0);
 #pragma unroll
         for (int f = 0; f < FT; ++f)
 #pragma unroll
-          for (int q = 0; q < RG; ++q)
-            acc[f][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][f][q], bv[u][t], acc[f][q][t], 0, 0, 0);
+          for (int q = 0; q < RG; ++q) {
+            if (PAIR && u % 2 == 1)
+              acc_hi[q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u / 2][f][q], b, acc_hi[q][t], 0, 0, 0);
+            else
+              acc[f][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[PAIR ? u / 2 : u][f][q], b, acc[f][q][t], 0, 0, 0);
+          }
       }
+      if (more) {
+        if (!PAIR) load_a(k_next, u);
+        else if (u % 2 == 1) load_a(k_next, u / 2);
+        if (!STAGE) load_b(k_next, u);
+      }
+    }
+    }
+  };
+  if (n_iter > 0) {
+    int k = k_of(0);
+    if (STAGE) load_s(k);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (u < UA) load_a(k, u);
+      if (!STAGE && u < UB) load_b(k, u);
+    }
+    // (with the rotated start of the staged variant the range's last stretch may come at any iteration)
+    for (int it = 0; it + 1 < n_iter; ++it) {
+      const int k_next = k_of(it + 1);
+      if (STAGE) iteration(k, k_next, std::true_type{}, std::true_type{});
+      else iteration(k, k_next, std::true_type{}, std::false_type{});
+      k = k_next;
+    }
+    iteration(k, 0, std::false_type{}, std::true_type{});
   }
   if (STAGE) __syncthreads();  // the staging regions become the reduction buffer
 
-  // sum of squares of row n = t*16 + r: over the 4 lane groups, then over the waves
+  // sum of squares of row n = t*16 + r: element (r, r) of the Gram matrix, which lane (r, r / 4) holds as its
+  // element r % 4 (a lane holds rows g*4 .. g*4+3 of column r); then over the waves
   if (RMS) {
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      ss[t] += __shfl_xor(ss[t], 16, WAVE);
-      ss[t] += __shfl_xor(ss[t], 32, WAVE);
-      if (g == 0) red_ss[wave][t][r] = ss[t];
+      const int i = r % 4;
+      const float d = i == 0 ? gram[t][0] : (i == 1 ? gram[t][1] : (i == 2 ? gram[t][2] : gram[t][3]));
+      if (g == r / 4) red_ss[wave][t][r] = d;   // (paired B operands: rows 8..15 are rows 0..7 at k + 32)
     }
   }
   // the waves' partial products meet in LDS; wave f adds those of tile f in the order of the waves
+  // (8 features: lanes g < 2 hold them in the first accumulator, lanes g >= 2 in the second; lane l < 32 then
+  // adds what lane l + 32 left)
 #pragma unroll
   for (int f = 0; f < FT; ++f)
 #pragma unroll
     for (int q = 0; q < RG; ++q)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) red[wave][f][q][t][lane] = acc[f][q][t];
+      for (int t = 0; t < NT; ++t) red[wave][f][q][t][lane] = (PAIR && !BP && g >= 2) ? acc_hi[PAIR ? q : 0][t] : acc[f][q][t];
   __syncthreads();
   if (wave >= FT) return;
   const int tile = wave;
+  // (paired B operands: the second half of feature (g, i) and row r is at rows + 8, columns + 8 of the tile)
+  const int partner = BP ? (lane + 40) & 63 : (lane & 31) + 32;
   floatx4 sum[RG][NT];
 #pragma unroll
   for (int q = 0; q < RG; ++q)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) sum[q][t] = red[0][tile][q][t][lane];
+    for (int t = 0; t < NT; ++t) {
+      sum[q][t] = red[0][tile][q][t][lane];
+      if (PAIR) sum[q][t] += red[0][tile][q][t][partner];
+    }
 #pragma unroll(RG * NT <= 2 ? WAVES : 1)
   for (int w = 1; w < WAVES; ++w)
 #pragma unroll
     for (int q = 0; q < RG; ++q)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) sum[q][t] += red[w][tile][q][t][lane];
+      for (int t = 0; t < NT; ++t) {
+        sum[q][t] += red[w][tile][q][t][lane];
+        if (PAIR) sum[q][t] += red[w][tile][q][t][partner];
+      }
 
   // D[feature g*4 + i][row r] of tile t: lane holds 4 consecutive features of one row
 #pragma unroll
@@ -295,7 +399,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     if (RMS) {
       float tot = 0.f;
 #pragma unroll
-      for (int w = 0; w < WAVES; ++w) tot += red_ss[w][t][r];
+      for (int w = 0; w < WAVES; ++w) tot += red_ss[w][t][r] + (BP ? red_ss[w][t][(r + 8) & 15] : 0.f);
       scale = 1.0f / sqrtf(tot / (float)a.I + a.eps);
     }
     const bool full = o + 3 < a.O;
@@ -374,32 +478,38 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 }
 
-template <int NT, int RG, bool RMS, int EPI, int KC>
+template <int NT, bool ST, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
-  constexpr int rows8_below = 256;   // tiles of 16 features below which a workgroup takes 8 (one per compute unit)
   constexpr int tiles2_from = 192;   // pairs of tiles from which a workgroup takes two (measured at 33 to 64 rows)
   if constexpr (NT >= 3 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
     // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
     if (a.O / 32 >= tiles2_from) {
-      gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(a);
+      gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(a);
       return;
     }
   }
   // few features: halve the rows per workgroup so that every compute unit gets one
-  if ((NT <= 2 || EPI == EPI_CONV) && a.O / 16 < rows8_below) {
-    gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+  if ((NT <= 2 || EPI == EPI_CONV) && pair_layout(a.O)) {
+    if constexpr (NT == 1 && !ST) {
+      if (a.N <= 8) {   // the rows of X fit half a tile: paired B operands
+        gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+        return;
+      }
+    }
+    gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
   } else {
-    gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
   }
 }
 
 template <int RG, bool RMS, int EPI, int KC = 0>
 void launch_nt(const FusedArgs& a, hipStream_t s) {
+  // (up to 16 rows of X come straight into the B operands: staging 5 to 16 rows through LDS was measured, slower)
   const int nt = ceil_div(a.N, 16);
-  if (nt == 1) launch_rows<1, RG, RMS, EPI, KC>(a, s);
-  else if (nt == 2) launch_rows<2, RG, RMS, EPI, KC>(a, s);
-  else if (nt == 3) launch_rows<3, RG, RMS, EPI, KC>(a, s);
-  else launch_rows<4, RG, RMS, EPI, KC>(a, s);
+  if (nt == 1) launch_rows<1, false, RG, RMS, EPI, KC>(a, s);
+  else if (nt == 2) launch_rows<2, true, RG, RMS, EPI, KC>(a, s);
+  else if (nt == 3) launch_rows<3, true, RG, RMS, EPI, KC>(a, s);
+  else launch_rows<4, true, RG, RMS, EPI, KC>(a, s);
 }
 
 template <bool RMS>
@@ -420,18 +530,17 @@ int check_common(const char* what, const void* X, const void* W, int N, int O, i
   return 0;
 }
 
-// A row stride of 0 says that W is in tile order (pack_weight).
+// A row stride of 0 says that W is in tile order; which of the two follows from the rows of a group (packed_layout.h).
 void note_layout(FusedArgs& a) {
   a.rotate = 1;
-  if (a.ldw != 0) return;
-  a.packed = 1;
-  a.ktiles = ceil_div(a.I, 32);
   a.group_tiles = ceil_div(a.O, 16);
+  if (a.ldw != 0) return;
+  a.packed = pair_layout(a.O) ? 2 : 1;
+  a.ktiles = a.packed == 2 ? ceil_div(a.I, 64) : ceil_div(a.I, 32);
 }
 }  // namespace
 
-// In all of these, ldw == 0 means that W is in tile order: [row group][ceil(O/16)][ceil(I/32)][64 lanes][8],
-// lane (r, g) of a tile holding W[tile row * 16 + r][k tile * 32 + g * 8 .. + 8], zeros beyond O and I.
+// In all of these, ldw == 0 means that W is in tile order (packed_layout.h), each row group by itself.
 //
 // Y[n, o] = scale_n * sum_k X[n, k] W[o, k], bfloat16 out; scale_n = 1/sqrt(mean_k X[n,k]^2 + eps) if rms.
 GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N, int O, int I, long ldx, long ldw,

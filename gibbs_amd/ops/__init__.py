@@ -166,23 +166,36 @@ def one_off_work() -> int:
     return int(library().gibbs_gemm_library_timings())
 
 
+def pair_layout(rows: int) -> bool:
+    """Whether a packed matrix of `rows` rows (per row group) is in the pair layout; the rule is the library's."""
+    return -(-rows // 16) < library().gibbs_pair_layout_below_tiles()
+
+
 class PackedWeight:
-    """A matrix [groups * rows, inner] (bfloat16) in the order the few-row products read it:
-    [group][ceil(rows/16)][ceil(inner/32)][64 lanes][8], lane (r, g) of a tile holding
-    W[tile row * 16 + r][k tile * 32 + g * 8 .. + 8], zeros beyond rows and inner.  A wave's load of
-    an MFMA A operand is then 1 KB of consecutive memory (8 requests of 128 bytes instead of 16 of
-    64), which is worth a fifth of the time of a weight-streaming product.  `shape`, `dtype` and
-    `stride(0) == 0` let it stand where the row-major matrix does."""
+    """A matrix [groups * rows, inner] (bfloat16) in the order the few-row products read it, each row group
+    by itself, zeros beyond rows and inner.  A wave's load of an MFMA A operand is then 1 KB of consecutive
+    memory (8 requests of 128 bytes instead of 16 of 64), which is worth a fifth of the time of a
+    weight-streaming product.  Two orders (csrc/packed_layout.h), chosen by the rows of a group:
+    16-row tiles, [group][ceil(rows/16)][ceil(inner/32)][64 lanes][8], lane (r, g) of a tile holding
+    W[tile row * 16 + r][k tile * 32 + g * 8 .. + 8]; and, for matrices of so few rows that workgroups take 8
+    features each, 8-row tiles of two k tiles, [group][2 ceil(rows/16)][ceil(inner/64)][g][half][r8][8] with
+    W[tile * 8 + r8][pair * 64 + half * 32 + g * 8 .. + 8].  `shape`, `dtype` and `stride(0) == 0` let it stand
+    where the row-major matrix does."""
 
     def __init__(self, w: torch.Tensor, groups: int = 1):
         assert w.dim() == 2 and w.dtype == torch.bfloat16 and w.shape[0] % groups == 0
         total, inner = w.shape
         rows = total // groups
-        rows_p, inner_p = -(-rows // 16) * 16, -(-inner // 32) * 32
+        self.pairs = pair_layout(rows)
+        rows_p = -(-rows // 16) * 16
+        inner_p = -(-inner // 64) * 64 if self.pairs else -(-inner // 32) * 32
         padded = torch.zeros((groups, rows_p, inner_p), dtype=w.dtype, device=w.device)
         padded[:, :rows, :inner] = w.reshape(groups, rows, inner)
-        tiles = padded.view(groups, rows_p // 16, 16, inner_p // 32, 4, 8).permute(0, 1, 3, 4, 2, 5)
-        self.data = tiles.contiguous()                     # [group][row tile][k tile][g][r][8]
+        if self.pairs:
+            tiles = padded.view(groups, rows_p // 8, 8, inner_p // 64, 2, 4, 8).permute(0, 1, 3, 5, 4, 2, 6)
+        else:
+            tiles = padded.view(groups, rows_p // 16, 16, inner_p // 32, 4, 8).permute(0, 1, 3, 4, 2, 5)
+        self.data = tiles.contiguous()                     # [group][row tile][k tile or pair][g]([half])[r][8]
         self.shape, self.dtype, self.groups, self.device = (total, inner), w.dtype, groups, w.device
 
     def dim(self) -> int:

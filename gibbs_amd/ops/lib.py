@@ -69,7 +69,7 @@ _SIGNATURES = {
 }
 
 
-_PLAN_SIGNATURES = {
+_VALUE_SIGNATURES = {
     "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int], c_void_p),
     "gibbs_plan_destroy": ([c_void_p], None),
     "gibbs_plan_add_block": ([c_void_p, c_void_p, c_float, c_void_p, c_float], c_int),
@@ -81,6 +81,7 @@ _PLAN_SIGNATURES = {
     "gibbs_plan_set_glu": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
     "gibbs_plan_workspace": ([c_void_p, c_void_p], c_long),
     "gibbs_plan_step": ([c_void_p, c_void_p], c_int),
+    "gibbs_pair_layout_below_tiles": ([], c_int),
 }
 
 
@@ -100,7 +101,7 @@ def library() -> ctypes.CDLL:
                     fn = getattr(lib, name)
                     fn.argtypes = argtypes
                     fn.restype = c_int
-                for name, (argtypes, restype) in _PLAN_SIGNATURES.items():
+                for name, (argtypes, restype) in _VALUE_SIGNATURES.items():
                     getattr(lib, name).argtypes, getattr(lib, name).restype = argtypes, restype
                 for name in ("gibbs_gemm_library_timings", "gibbs_gemm_library_plans"):
                     getattr(lib, name).argtypes, getattr(lib, name).restype = [], c_long

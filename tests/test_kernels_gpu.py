@@ -131,22 +131,36 @@ def test_gemm_skinny(n, o, i, splits, out_dtype):
 
 
 def test_packed_weight_layout():
-    """[group][16-row tile][32-k tile][lane = g * 16 + r][8] with zeros beyond the matrix."""
+    """Many rows: [group][16-row tile][32-k tile][lane = g * 16 + r][8]; few rows (workgroups of 8 features):
+    [group][8-row tile][pair of k tiles][g][half][r8][8]; zeros beyond the matrix."""
     from gibbs_amd import ops
+    rows = 4104                                             # 257 tiles of 16
+    assert not ops.pair_layout(rows) and not ops.pair_layout(4081) and ops.pair_layout(4080) and ops.pair_layout(40)
+    w = rnd(2 * rows, 72, dtype=torch.bfloat16)
+    p = ops.PackedWeight(w, groups=2)
+    assert p.shape == (2 * rows, 72) and p.stride(0) == 0 and tuple(p.data.shape) == (2, 257, 3, 4, 16, 8) and not p.pairs
+    for q, ot, kt, g, r in [(0, 0, 0, 0, 0), (1, 2, 1, 3, 7), (0, 256, 2, 0, 15), (1, 256, 2, 1, 3), (1, 256, 0, 2, 8)]:
+        row, k = ot * 16 + r, kt * 32 + g * 8
+        want = torch.zeros(8, dtype=torch.bfloat16, device=DEV)
+        if row < rows and k < 72:
+            want[:min(8, 72 - k)] = w[q * rows + row, k:k + 8]
+        assert torch.equal(p.data[q, ot, kt, g, r], want), (q, ot, kt, g, r)
     w = rnd(2 * 40, 72, dtype=torch.bfloat16)
     p = ops.PackedWeight(w, groups=2)
-    assert p.shape == (80, 72) and p.stride(0) == 0 and tuple(p.data.shape) == (2, 3, 3, 4, 16, 8)
-    for q, ot, kt, g, r in [(0, 0, 0, 0, 0), (1, 2, 1, 3, 7), (0, 1, 2, 0, 15), (1, 0, 2, 1, 3)]:
-        row, k = ot * 16 + r, kt * 32 + g * 8
+    assert p.shape == (80, 72) and p.stride(0) == 0 and tuple(p.data.shape) == (2, 6, 2, 4, 2, 8, 8) and p.pairs
+    for q, o8, pair, g, half, r8 in [(0, 0, 0, 0, 0, 0), (1, 4, 1, 0, 0, 7), (0, 2, 1, 1, 1, 5), (1, 5, 0, 3, 1, 3), (0, 4, 0, 2, 1, 7)]:
+        row, k = o8 * 8 + r8, pair * 64 + half * 32 + g * 8
         want = torch.zeros(8, dtype=torch.bfloat16, device=DEV)
         if row < 40 and k < 72:
             want[:min(8, 72 - k)] = w[q * 40 + row, k:k + 8]
-        assert torch.equal(p.data[q, ot, kt, g, r], want), (q, ot, kt, g, r)
+        assert torch.equal(p.data[q, o8, pair, g, half, r8], want), (q, o8, pair, g, half, r8)
     x = rnd(5, 72, dtype=torch.bfloat16, seed=2)
     for splits in (1, 2):
         w1 = rnd(50, 256, dtype=torch.bfloat16, seed=3)
         x1 = rnd(5, 256, dtype=torch.bfloat16, seed=4)
         assert torch.equal(ops.gemm_skinny(x1, ops.PackedWeight(w1), torch.float32, splits), ops.gemm_skinny(x1, w1, torch.float32, splits))
+        w2 = rnd(4200, 256, dtype=torch.bfloat16, seed=5)                    # 16-row tiles
+        assert torch.equal(ops.gemm_skinny(x1, ops.PackedWeight(w2), torch.float32, splits), ops.gemm_skinny(x1, w2, torch.float32, splits))
 
 
 def test_skinny_splits_cover_k():
