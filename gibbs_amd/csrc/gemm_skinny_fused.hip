@@ -84,7 +84,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   // pipe of a compute unit is bound by requests in flight, and from 8 rows on X is as many requests as W
   // for a workgroup of 8 features).  The wave's region is its own: no barrier.
   static_assert(STAGE || NT == 1, "more than 16 rows of X are staged");
-  constexpr int U = (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);  // MFMA steps per iteration
+  // MFMA steps per iteration (8 features and one tile of rows: an A operand serves two steps, so 8 steps are 4 loads a row group)
+  constexpr int U = (ROWS == 8 && NT == 1) ? 8 : (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);
   constexpr int CH = 4 * U;                    // 16-byte chunks of a row per iteration
   constexpr int RED_BYTES = WAVES * FT * RG * NT * WAVE * 16;
   constexpr int STAGE_BYTES = STAGE ? WAVES * NT * 16 * CH * 16 : 0;
@@ -157,45 +158,16 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     x_ok[t] = BP ? r8 < a.N : t * 16 + r < a.N;
     xrow[t] = a.X + (size_t)(x_ok[t] ? (BP ? r8 : t * 16 + r) : 0) * a.ldx + (BP ? half * 32 : 0) + g * 8;
   }
-  // What the epilogue reads besides the product is asked for now: the product hides the latency
-  // (the state row hangs on a slot index, two dependent loads).  Wave 0 writes the outputs; its lane
-  // holds features o_epi .. +3 of row t*16 + r.
+  // What the epilogue reads besides the product is asked for behind the first loads of the operands: the
+  // product hides the latency (the state row hangs on a slot index, two dependent loads, and wave 0 would
+  // start its share of W that much later if they came first).  Wave 0 writes the outputs; its lane holds
+  // features o_epi .. +3 of row t*16 + r.
   constexpr int KH = KC > 1 ? KC - 1 : 1;
   const int o_epi = o0 + g * 4;
   const bool epi_lane = wave == 0 && g * 4 < ROWS && o_epi < a.O;
   float pre_x[NT][4];          // RESIDUAL: the stream; CONV: unused
   float pre_hist[NT][KH][4];   // CONV: the state rows
   float pre_taps[KC > 1 ? KC : 1][4], pre_bias[4];
-  if (EPI == EPI_RESIDUAL) {
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = t * 16 + r;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pre_x[t][i] = (epi_lane && n < a.N && o_epi + i < a.O) ? a.x[(size_t)n * a.O + o_epi + i] : 0.f;
-    }
-  }
-  if (EPI == EPI_CONV && KC > 1) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const bool ok = epi_lane && o_epi + i < a.O;
-#pragma unroll
-      for (int j = 0; j < KC; ++j) pre_taps[j][i] = ok ? a.taps[(size_t)(o_epi + i) * KC + j] : 0.f;
-      pre_bias[i] = (ok && a.bias) ? a.bias[o_epi + i] : 0.f;
-    }
-#pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = t * 16 + r;
-      const bool row = epi_lane && n < a.N;
-      const float* st = a.state + (size_t)(row ? a.slot[n] : 0) * a.slot_stride;
-      const int before = row ? a.ctx[n] : 0;
-#pragma unroll
-      for (int j = 0; j < KH; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          pre_hist[t][j][i] = (row && o_epi + i < a.O && before - (KC - 1) + j >= 0) ? st[(size_t)j * a.O + o_epi + i] : 0.f;
-    }
-  }
-
   floatx4 acc[FT][RG][NT];
   floatx4 acc_hi[PAIR ? RG : 1][NT];   // 8 features: the products with X at k + 32 (rows 8..15 hold the features)
   floatx4 gram[NT];   // RMS: X X^T of the tile's rows (its diagonal is the rows' sums of squares)
@@ -329,13 +301,46 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     }
   };
   if (n_iter > 0) {
-    int k = k_of(0);
+    const int k = k_of(0);
     if (STAGE) load_s(k);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (u < UA) load_a(k, u);
       if (!STAGE && u < UB) load_b(k, u);
     }
+  }
+  if (EPI == EPI_RESIDUAL) {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pre_x[t][i] = (epi_lane && n < a.N && o_epi + i < a.O) ? a.x[(size_t)n * a.O + o_epi + i] : 0.f;
+    }
+  }
+  if (EPI == EPI_CONV && KC > 1) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool ok = epi_lane && o_epi + i < a.O;
+#pragma unroll
+      for (int j = 0; j < KC; ++j) pre_taps[j][i] = ok ? a.taps[(size_t)(o_epi + i) * KC + j] : 0.f;
+      pre_bias[i] = (ok && a.bias) ? a.bias[o_epi + i] : 0.f;
+    }
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      const int n = t * 16 + r;
+      const bool row = epi_lane && n < a.N;
+      const float* st = a.state + (size_t)(row ? a.slot[n] : 0) * a.slot_stride;
+      const int before = row ? a.ctx[n] : 0;
+#pragma unroll
+      for (int j = 0; j < KH; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          pre_hist[t][j][i] = (row && o_epi + i < a.O && before - (KC - 1) + j >= 0) ? st[(size_t)j * a.O + o_epi + i] : 0.f;
+    }
+  }
+
+  if (n_iter > 0) {
+    int k = k_of(0);
     // (with the rotated start of the staged variant the range's last stretch may come at any iteration)
     for (int it = 0; it + 1 < n_iter; ++it) {
       const int k_next = k_of(it + 1);
