@@ -23,6 +23,9 @@ model entry inherits the defaults; the keys that mean something here:
                     per step beside a prompt portion of `portion` tokens of one more request, through
                     `Engine.step` (no captured graph: what a scheduler step costs); the row reports the
                     wall time of a step and the time after which the host is through with queueing it;
+                    or "streams": a kernel that only reads `reads_mib` MiB, and the few-row product of every
+                    distinct matrix of the model's layers beside the pure read of its bytes, per kernel of a
+                    captured chain
                     or "products": every distinct matrix of the model's layers against `rows`
                     (default 2048) rows of activations, the library's product and the hand-written
                     tiled kernel side by side (`only`: "library" or "own" keeps one of them, for a
@@ -246,6 +249,75 @@ def products(entry: Dict, base: str) -> Dict:
     return {"model": entry["name"], "workload": "products", "dtype": "bfloat16", "rows": rows, "products": cells}
 
 
+def streams(entry: Dict, base: str) -> Dict:
+    """What a kernel that streams a given number of bytes takes inside a chain of dependent kernels (a captured
+    graph of 48 launches, the buffers taking turns through 1.5 GiB so that nothing stays cached): a kernel that
+    only reads (`reads_mib`), and the few-row products of the decode step for every distinct matrix of the
+    model (`rows` rows of X) with the pure read of the same bytes beside them."""
+    import torch
+
+    from . import ops
+    from .config import config_from_dict
+    from .parts import DecoderModel
+    dev, chain = "cuda:0", 48
+    pool = torch.empty(3 << 28, dtype=torch.bfloat16, device=dev).normal_()          # 1.5 GiB
+    pool_bytes = pool.numel() * 2
+    sums = torch.zeros(8192, device=dev)
+
+    def per_kernel(fn) -> float:
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / 20 / chain * 1e6
+
+    def read_us(nbytes: int) -> float:
+        nbytes = max(16, nbytes // 16 * 16)
+        step = (nbytes + (1 << 20)) // 256 * 256
+
+        def run():
+            for i in range(chain):
+                ops.probe_read(pool, (i * step) % (pool_bytes - nbytes) // 256 * 256, nbytes, sums)
+        return per_kernel(run)
+
+    row = {"model": entry["name"], "workload": "streams", "dtype": "bfloat16",
+           "reads": [{"mib": m, "us": round(read_us(int(m * (1 << 20))), 2)} for m in entry.get("reads_mib", [])]}
+    ident = entry.get("id")
+    if ident:
+        if not ident.startswith("random:"):
+            raise ValueError("the streams workload takes a configuration (random:CONFIG.json): only shapes matter")
+        with open(os.path.join(base, ident[len("random:"):])) as f:
+            cfg = config_from_dict(json.load(f))
+        model = DecoderModel(cfg.model_spec())
+        shapes: List[tuple] = []
+        for block in model.blocks:
+            for part in (block.mixer, block.ffn):
+                for shape in part.product_shapes():
+                    if shape not in shapes:
+                        shapes.append(shape)
+        n = int(entry.get("rows", 8))
+        cells = []
+        for o, i in shapes:
+            copies = max(2, min(chain, -(-(1 << 29) // (o * i * 2))))       # half a GiB of copies take turns
+            ws = [ops.PackedWeight(pool[c * o * i:(c + 1) * o * i].view(o, i)) for c in range(copies)]
+            x = torch.randn(n, i, device=dev).to(torch.bfloat16)
+            y = torch.empty(n, o, dtype=torch.bfloat16, device=dev)
+            us = per_kernel(lambda: [ops.skinny_store(x, ws[c % copies], None, out=y) for c in range(chain)])
+            cells.append({"out": o, "in": i, "mib": round(o * i * 2 / (1 << 20), 1), "product_us": round(us, 2),
+                          "read_us": round(read_us(o * i * 2), 2)})
+            del ws
+        row.update(rows=n, products=cells)
+    return row
+
+
 def mixed(entry: Dict, base: str) -> Dict:
     """Steps that hold decoded tokens beside a prompt portion, one after the other without waiting for
     their logits: wall time per step, and how long the host needs to queue one."""
@@ -303,15 +375,16 @@ def run_suite(path: str) -> int:
         entry = dict(DEFAULTS)
         entry.update(suite.get("defaults", {}))
         entry.update(m)
-        if "id" not in entry:
+        if "id" not in entry and not (entry.get("workload") == "streams" and "name" in entry):
             print("gibbs --bench: a model entry has no id", file=sys.stderr)
             failed = True
             continue
-        ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
-        entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
+        if "id" in entry:
+            ident = entry["id"][len("random:"):] if entry["id"].startswith("random:") else entry["id"]
+            entry.setdefault("name", os.path.splitext(os.path.basename(ident.rstrip("/")))[0])
         try:
             workload = entry.get("workload", "decode")
-            row = {"serve": serve, "products": products, "mixed": mixed}.get(workload, measure)(entry, base)
+            row = {"serve": serve, "products": products, "mixed": mixed, "streams": streams}.get(workload, measure)(entry, base)
         except Exception as e:     # one model's failure is reported; the others still run (bench.rs:751)
             print(f"gibbs --bench: {entry['name']}: {type(e).__name__}: {e}", file=sys.stderr)
             failed = True

@@ -41,6 +41,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
 
 enum { EPI_STORE = 0, EPI_RESIDUAL = 1, EPI_GLU = 2, EPI_CONV = 3 };
+
+// The operand with lanes r and r ^ 8 of every 16 exchanged (a rotation by 8 within the row of lanes).
+__device__ __forceinline__ bf16x8 swap_halves16(bf16x8 v) {
+  typedef int int4v __attribute__((ext_vector_type(4)));
+  int4v w = __builtin_bit_cast(int4v, v);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = __builtin_amdgcn_update_dpp(0, w[i], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+  return __builtin_bit_cast(bf16x8, w);
+}
 constexpr int MAX_TAPS = 8;
 
 struct FusedArgs {
@@ -104,7 +113,9 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   // of X at the next 32 values of k.  One MFMA then does two steps: the upper left 8 x 8 block of its result is
   // the product at k, the lower right one the product at k + 32 (the other two blocks mix the two and are
   // dropped).  A load of X is 8 requests of 128 bytes instead of two loads of 8 requests of 64.
-  static_assert(!BP || (PAIR && NT == 1 && !STAGE), "paired B operands: 8 features, one tile of rows, not staged");
+  // With 16 features the A operands are single steps: the step at k takes the pair as it is (columns 0..7 of the
+  // result are the rows of X), the step at k + 32 takes it with the halves of every 16 lanes exchanged.
+  static_assert(!BP || (NT == 1 && !STAGE && FT == 1), "paired B operands: one tile of rows and of features, not staged");
   const int steps = (a.I + KU - 1) / KU;
   const int per_wave = (steps + WAVES - 1) / WAVES;
   const int k_begin = wave * per_wave * KU;
@@ -267,12 +278,20 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
         bf16x8 b = bv[u][0];
         if (ragged && !(k + u * 64 + xoff < k_end)) b = zero;
         if (RMS) gram[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, b, gram[0], 0, 0, 0);
+        if constexpr (PAIR) {
 #pragma unroll
-        for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][0][q], b, acc[0][q][0], 0, 0, 0);
-        if (more) {
-          load_a(k_next, u);
-          load_b(k_next, u);
+          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][0][q], b, acc[0][q][0], 0, 0, 0);
+          if (more) load_a(k_next, u);
+        } else {
+#pragma unroll
+          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u][0][q], b, acc[0][q][0], 0, 0, 0);
+          if (more) load_a(k_next, 2 * u);
+          const bf16x8 b2 = swap_halves16(b);
+#pragma unroll
+          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u + 1][0][q], b2, acc[0][q][0], 0, 0, 0);
+          if (more) load_a(k_next, 2 * u + 1);
         }
+        if (more) load_b(k_next, u);
       }
     } else {
 #pragma unroll
@@ -375,7 +394,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   if (wave >= FT) return;
   const int tile = wave;
   // (paired B operands: the second half of feature (g, i) and row r is at rows + 8, columns + 8 of the tile)
-  const int partner = BP ? (lane + 40) & 63 : (lane & 31) + 32;
+  const int partner = BP ? (lane + 40) & 63 : (lane & 31) + 32;   // (8 features only)
   floatx4 sum[RG][NT];
 #pragma unroll
   for (int q = 0; q < RG; ++q)
@@ -503,6 +522,12 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
     }
     gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
   } else {
+    if constexpr (NT == 1 && !ST) {
+      if (a.N <= 8) {
+        gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+        return;
+      }
+    }
     gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
   }
 }

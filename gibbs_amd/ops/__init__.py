@@ -614,6 +614,15 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
     return out
 
 
+def probe_read(buffer: torch.Tensor, offset: int, nbytes: int, out: torch.Tensor, grid: int = 1024, block: int = 256) -> None:
+    """Reads `nbytes` of `buffer` from byte `offset` and leaves per-workgroup sums in `out` (float32 [grid]): the
+    yardstick for the weight-streaming kernels (measurement only)."""
+    require_cuda(buffer, out)
+    assert buffer.is_contiguous() and 0 <= offset and offset + nbytes <= buffer.numel() * buffer.element_size()
+    assert out.dtype == torch.float32 and out.numel() >= grid and out.is_contiguous()
+    call("gibbs_probe_read", buffer.data_ptr() + offset, nbytes, ptr(out), grid, block, stream())
+
+
 def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Index of the first largest value of each row (NaN never wins), int32 [M]."""
     require_cuda(logits)

@@ -64,6 +64,7 @@ _SIGNATURES = {
     "gibbs_gemm_library_init": [],
     "gibbs_gemm_library": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
+    "gibbs_probe_read": [c_void_p, c_long, c_void_p, c_int, c_int, c_void_p],
     "gibbs_repetition_penalty": [c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     "gibbs_sample": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
 }
