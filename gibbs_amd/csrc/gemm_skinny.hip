@@ -10,6 +10,9 @@
 #include "common.h"
 #include "packed_layout.h"
 
+int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
+                          long ldy, int rms, float eps, hipStream_t stream);
+
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
@@ -221,6 +224,8 @@ GIBBS_EXPORT int gibbs_gemm_skinny(const void* X, const void* W, void* Y, int ou
   GIBBS_REQUIRE(k_splits >= 1 && k_splits <= 1024, "gemm_skinny: %d k splits", k_splits);
   GIBBS_REQUIRE(k_splits == 1 || out_dtype == GIBBS_F32, "gemm_skinny: partial sums are float32");
   GIBBS_REQUIRE(out_dtype == GIBBS_F32 || out_dtype == GIBBS_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
+  // one tile of rows and whole sums: the kernel with the paired operands (gemm_skinny_fused.hip) does the same faster
+  if (k_splits == 1 && N <= 16) return gibbs_skinny_store_as(X, W, Y, out_dtype, N, O, I, ldx, ldw, ldy, 0, 0.f, stream);
   // each block's k range is a whole number of 128-element steps (what one wave does per iteration)
   int kpb = ceil_div(ceil_div(I, k_splits), 128) * 128;
   const int used = ceil_div(I, kpb);

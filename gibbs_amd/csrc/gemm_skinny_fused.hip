@@ -63,8 +63,10 @@ struct FusedArgs {
   long ldw, ldx;
   long group_stride;  // rows of W between row groups
   float eps;          // rms prologue
-  // STORE / GLU / CONV: bfloat16 output [N, ldy]
+  // STORE / GLU / CONV: bfloat16 output [N, ldy] (STORE: or float32, Yf)
   bf16* Y;
+  float* Yf;
+  int y_vec;
   long ldy;
   // RESIDUAL
   float* x;   // [N, O] float32, updated in place
@@ -427,7 +429,14 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       scale = 1.0f / sqrtf(tot / (float)a.I + a.eps);
     }
     const bool full = o + 3 < a.O;
-    if (EPI == EPI_STORE) {
+    if (EPI == EPI_STORE && a.Yf) {
+      float* y = a.Yf + (size_t)n * a.ldy + o;
+      if (full && a.y_vec) {
+        *(floatx4*)y = floatx4{sum[0][t][0] * scale, sum[0][t][1] * scale, sum[0][t][2] * scale, sum[0][t][3] * scale};
+      } else {
+        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = sum[0][t][i] * scale;
+      }
+    } else if (EPI == EPI_STORE) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       if (full && a.ldy % 4 == 0) {
         *(bf16x4*)y = bf16x4{(bf16)(sum[0][t][0] * scale), (bf16)(sum[0][t][1] * scale), (bf16)(sum[0][t][2] * scale),
@@ -573,13 +582,27 @@ void note_layout(FusedArgs& a) {
 // In all of these, ldw == 0 means that W is in tile order (packed_layout.h), each row group by itself.
 //
 // Y[n, o] = scale_n * sum_k X[n, k] W[o, k], bfloat16 out; scale_n = 1/sqrt(mean_k X[n,k]^2 + eps) if rms.
+int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
+                          long ldy, int rms, float eps, hipStream_t stream);
+
 GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N, int O, int I, long ldx, long ldw,
                                     long ldy, int rms, float eps, hipStream_t stream) {
+  return gibbs_skinny_store_as(X, W, Y, GIBBS_BF16, N, O, I, ldx, ldw, ldy, rms, eps, stream);
+}
+
+// The same with the output's type given: bfloat16 or float32 (Y: [N, ldy] of that type, 16-byte aligned rows for
+// the vector stores to be taken).
+int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
+                          long ldy, int rms, float eps, hipStream_t stream) {
   if (check_common("skinny_store", X, W, N, O, I, ldx, ldw)) return 1;
   GIBBS_REQUIRE(ldy >= O, "skinny_store: output rows shorter than %d", O);
+  GIBBS_REQUIRE(out_dtype == GIBBS_BF16 || out_dtype == GIBBS_F32, "skinny_store: unknown output dtype %d", out_dtype);
   FusedArgs a{};
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
-  a.Y = (bf16*)Y; a.ldy = ldy;
+  if (out_dtype == GIBBS_F32) a.Yf = (float*)Y;
+  else a.Y = (bf16*)Y;
+  a.ldy = ldy;
+  a.y_vec = ((uintptr_t)Y % 16) == 0 && ldy % 4 == 0;   // float32 rows that take 16-byte stores
   if (rms) launch_nt<1, true, EPI_STORE>(a, stream);
   else launch_nt<1, false, EPI_STORE>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_store");
