@@ -563,7 +563,9 @@ def rms_scale(x, eps):
 
 
 @pytest.mark.parametrize("n,o,i", [(1, 64, 128), (8, 3072, 2048), (16, 331 * 8, 1000), (17, 200, 512), (64, 96, 4096), (5, 40, 72),
-                                   (48, 8200, 512), (64, 3072, 2048)])      # two tiles a workgroup; many rows, one tile
+                                   (48, 8200, 512), (64, 3072, 2048),      # two tiles a workgroup; many rows, one tile
+                                   (3, 20, 104), (8, 1001, 1000), (7, 4100, 104), (8, 4099, 2048), (9, 4100, 72),
+                                   (12, 36, 200)])                          # paired operands with ragged ends, both layouts
 def test_skinny_store_with_rms_prologue(n, o, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=3.0), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -575,7 +577,8 @@ def test_skinny_store_with_rms_prologue(n, o, i):
 
 
 @pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96), (64, 2048, 2048),
-                                   (40, 1000, 4096)])                       # many rows: partial sums over k, then the add
+                                   (40, 1000, 4096),                        # many rows: partial sums over k, then the add
+                                   (7, 36, 200), (8, 4100, 136), (2, 12, 8)])
 def test_skinny_residual(n, o, i):
     from gibbs_amd import ops
     y, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -591,7 +594,8 @@ def test_skinny_residual(n, o, i):
 
 
 @pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024), (64, 6200, 256),
-                                   (36, 8192, 2048)])                       # two tiles a workgroup
+                                   (36, 8192, 2048),                        # two tiles a workgroup
+                                   (5, 4100, 104), (8, 52, 40), (11, 4090, 72)])
 def test_skinny_glu(n, f, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=2.0), rnd(2 * f, i, dtype=torch.bfloat16, scale=0.05, seed=1)
