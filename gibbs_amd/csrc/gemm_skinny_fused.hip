@@ -543,9 +543,13 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
 
 template <int RG, bool RMS, int EPI, int KC = 0>
 void launch_nt(const FusedArgs& a, hipStream_t s) {
-  // (up to 16 rows of X come straight into the B operands: staging 5 to 16 rows through LDS was measured, slower)
+  // Up to 8 rows of X come straight into paired B operands, 12 and more through LDS.  Between them neither is
+  // clearly better (measured at 9, 12 and 16 rows: staged products are 8 to 16 % faster at 16 rows, the same at
+  // 12, and up to 13 % slower at 9 for the widest matrices).
+  constexpr int stage_from = 12;
   const int nt = ceil_div(a.N, 16);
-  if (nt == 1) launch_rows<1, false, RG, RMS, EPI, KC>(a, s);
+  if (nt == 1 && a.N < stage_from) launch_rows<1, false, RG, RMS, EPI, KC>(a, s);
+  else if (nt == 1) launch_rows<1, true, RG, RMS, EPI, KC>(a, s);
   else if (nt == 2) launch_rows<2, true, RG, RMS, EPI, KC>(a, s);
   else if (nt == 3) launch_rows<3, true, RG, RMS, EPI, KC>(a, s);
   else launch_rows<4, true, RG, RMS, EPI, KC>(a, s);
