@@ -307,10 +307,11 @@ def decode_batch_steps(seqs, prompt_len, ends_early):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,live", [("M", 17), ("W", 33), ("M", 48), ("W", 64)])
+@pytest.mark.parametrize("name,live", [("W", 7), ("M", 9), ("W", 12), ("M", 17), ("W", 33), ("M", 48), ("W", 64)])
 def test_many_requests_decoding_side_by_side(tmp_path_factory, name, live, dtype):
-    """17 to 64 live requests that decode together (in bfloat16 the fused decode kernels with their rows
-    staged through LDS, two tiles of features per workgroup, the down projection cut along k), with
+    """7 to 64 live requests that decode together (in bfloat16 the fused decode kernels: up to 8 rows in
+    paired operands, 9 to 11 straight into the operands, from 12 on staged through LDS, from 33 on with
+    two tiles of features per workgroup and the down projection cut along k), with
     prompts of different lengths so that sequences cross page edges at different steps, one request
     ending mid-way: every decoded place against the plain implementation, and the bfloat16 fused
     path against the same engine on its general path without folded gains."""
