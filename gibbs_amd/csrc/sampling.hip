@@ -35,14 +35,14 @@ __device__ __forceinline__ void block_best(float& v, int& i, float* sv, int* si)
 }
 
 // Calls fn(value, index) for the elements of a row that fall to this thread: 16-byte loads over the
-// aligned middle of the row, single elements before and after it.
-template <typename F>
+// aligned middle of the row, single elements before and after it.  AHEAD: loads in flight per thread (a
+// workgroup that walks a row alone, on the step's critical path, wants the whole row asked for at once).
+template <int AHEAD = 4, typename F>
 __device__ __forceinline__ void walk_row(const float* row, int V, F fn) {
   const int head = min(V, (int)(((16 - ((uintptr_t)row & 15)) & 15) / 4));
   const int n4 = (V - head) / 4;
   for (int i = threadIdx.x; i < head; i += THREADS) fn(row[i], i);
   const float4* row4 = (const float4*)(row + head);
-  constexpr int AHEAD = 4;     // loads in flight per thread
   for (int j0 = threadIdx.x; j0 < n4; j0 += AHEAD * THREADS) {
     float4 v[AHEAD];
 #pragma unroll
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(THREADS) void decode_tail_kernel(const float* __res
     const float* row = logits + (size_t)i * ld;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    walk_row(row, V, [&](float v, int j) {
+    walk_row<16>(row, V, [&](float v, int j) {
       if (better(v, j, bv, bi)) { bv = v; bi = j; }
     });
     block_best(bv, bi, sv, si);
