@@ -538,7 +538,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
   if (a.n_splits > 1) {
     dim3 mgrid(n_rows, ceil_div(a.nh, 4));
-    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial, out, a.nh, a.hd, a.n_splits, a.ldo);
+    launch_attention_merge(mgrid, stream, partial, out, a.nh, a.hd, a.n_splits, a.ldo);
   }
   GIBBS_LAUNCH_STATUS("attention_decode");
 }

@@ -346,8 +346,8 @@ GIBBS_EXPORT int gibbs_attention_prefill(const void* q, const void* kpages, cons
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return gibbs_fail("attention_prefill: %s", hipGetErrorString(e));
     dim3 mgrid(n_rows, ceil_div(nh, 4));
-    attention_merge_kernel<<<mgrid, 256, 0, stream>>>(partial + (size_t)first_row * nh * n_splits * (hd + 2),
-                                                      oo + (size_t)first_row * ldo, nh, hd, n_splits, ldo);
+    launch_attention_merge(mgrid, stream, partial + (size_t)first_row * nh * n_splits * (hd + 2), oo + (size_t)first_row * ldo,
+                           nh, hd, n_splits, ldo);
   }
   GIBBS_LAUNCH_STATUS("attention_prefill");
 }
