@@ -9,6 +9,7 @@
 // its float32 partial Y[s] for the consumer to add in a fixed order.
 #include "common.h"
 #include "packed_layout.h"
+#include <type_traits>
 
 int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
                           long ldy, int rms, float eps, hipStream_t stream);
@@ -59,14 +60,20 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
 #pragma unroll
   for (int f = 0; f < FT; ++f) {
     row_ok[f] = o0 + f * 16 + r < O;
-    wrow[f] = pairs    ? W + ((size_t)(2 * (o0 / 16 + f) + r / 8) * ktiles) * 512 + (g * 16 + r % 8) * 8
-              : packed ? W + ((size_t)(o0 / 16 + f) * ktiles) * 512 + lane * 8
+    const size_t tile = min(o0 / 16 + f, (O + 15) / 16 - 1);   // (a tile beyond the last one: rows nobody stores)
+    wrow[f] = pairs    ? W + ((2 * tile + r / 8) * ktiles) * 512 + (g * 16 + r % 8) * 8
+              : packed ? W + (tile * ktiles) * 512 + lane * 8
                        : W + (size_t)(row_ok[f] ? o0 + f * 16 + r : 0) * ldw + g * 8;
   }
-  const int kstride = packed ? 512 : 32;
   const int koff = packed ? 0 : g * 8;
-  // elements from wrow to the lane's A operand of 32-k tile j
-  auto a_off = [&](int j) { return pairs ? (size_t)(j >> 1) * 512 + (j & 1) * 64 : (size_t)j * kstride; };
+  // elements from wrow to the lane's A operand of 32-k tile j, clamped into the wave's range (so that every load
+  // is unconditional; see gemm_skinny_fused.hip): packed, tile min(j, last tile); row-major, element
+  // min(32 j + koff, I - 8) of the row
+  const int a_limit = packed ? (k_end - 1) / 32 : I - 8;
+  auto a_off = [&](int j) -> long {
+    const int c = min(packed ? j : j * 32 + koff, a_limit);
+    return pairs ? (long)(c >> 1) * 512 + (c & 1) * 64 : (packed ? (long)c * 512 : (long)c - koff);
+  };
   const bf16* xrow[NT];
   bool x_ok[NT];
 #pragma unroll
@@ -105,50 +112,72 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
   // waves' ranges and wraps around, so that they do not ask the same L2 channels at the same time
   const int n_iter = (k_end - k_begin + 32 * U - 1) / (32 * U);
   const int first_iter = (STAGE && n_iter > 0) ? (int)(blockIdx.x % n_iter) : 0;
-  for (int it = 0; it < n_iter; ++it) {
-    const int k = k_begin + ((it + first_iter) % n_iter) * 32 * U;
-    bf16x8 a[U][FT], b[U][NT];
+  auto k_of = [&](int it) { return k_begin + ((it + first_iter) % n_iter) * 32 * U; };
+  // Loads are unconditional and roll, as in gemm_skinny_fused.hip: as soon as a step's operands have been used
+  // their registers are asked for the next stretch of k; rows of X beyond N give columns nobody stores, and
+  // where k runs beyond the wave's range the rows of X are made zero before they are used.
+  bf16x8 av[U][FT], bv[U][NT], sv[NT][LPT];
+  auto load_a = [&](int k, int u) {
+    const long off = a_off(k / 32 + u);
+#pragma unroll
+    for (int f = 0; f < FT; ++f) av[u][f] = *(const bf16x8*)(wrow[f] + off);
+  };
+  auto load_b = [&](int k, int u) {
+    const int kc = min(k + u * 32 + g * 8, I - 8) - g * 8;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) bv[u][t] = *(const bf16x8*)(xrow[t] + kc);
+  };
+  auto load_s = [&](int k) {
+#pragma unroll
+    for (int i = 0; i < LPT; ++i) {
+      const int kc = min(k + s_chunk[i] * 8, I - 8) - s_chunk[i] * 8;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) sv[t][i] = *(const bf16x8*)(srow[t][i] + kc);
+    }
+  };
+  auto iteration = [&](int k, int k_next, auto more) {
     if (STAGE) {
-      bf16x8 sv[NT][LPT];
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int i = 0; i < LPT; ++i) {
+        const bool k_ok = k + s_chunk[i] * 8 < k_end;
 #pragma unroll
-        for (int i = 0; i < LPT; ++i)
-          sv[t][i] = (s_ok[t][i] && k + s_chunk[i] * 8 < k_end) ? *(const bf16x8*)(srow[t][i] + k) : zero;
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kk = k + u * 32;
-#pragma unroll
-        for (int f = 0; f < FT; ++f)
-          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + a_off(kk / 32)) : zero;
+        for (int t = 0; t < NT; ++t) stage[(t * LPT + i) * WAVE + lane] = k_ok ? sv[t][i] : zero;
       }
-#pragma unroll
-      for (int t = 0; t < NT; ++t)
-#pragma unroll
-        for (int i = 0; i < LPT; ++i) stage[(t * LPT + i) * WAVE + lane] = sv[t][i];
+      if (more) load_s(k_next);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) b[u][t] = stage[t * 16 * CH + read_slot[u]];
-    } else {
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kk = k + u * 32;
-        const bool k_ok = kk + g * 8 < k_end;
-#pragma unroll
-        for (int f = 0; f < FT; ++f)
-          a[u][f] = (row_ok[f] && kk + koff < k_end) ? *(const bf16x8*)(wrow[f] + a_off(kk / 32)) : zero;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) b[u][t] = (x_ok[t] && k_ok) ? *(const bf16x8*)(xrow[t] + kk) : zero;
-      }
+        for (int t = 0; t < NT; ++t) bv[u][t] = stage[t * 16 * CH + read_slot[u]];
     }
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
-      for (int f = 0; f < FT; ++f)
+      for (int t = 0; t < NT; ++t) {
+        bf16x8 b = bv[u][t];
+        if (!STAGE && !(k + u * 32 + g * 8 < k_end)) b = zero;
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][f], b[u][t], acc[f][t], 0, 0, 0);
+        for (int f = 0; f < FT; ++f) acc[f][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][f], b, acc[f][t], 0, 0, 0);
+      }
+      if (more) {
+        load_a(k_next, u);
+        if (!STAGE) load_b(k_next, u);
+      }
+    }
+  };
+  if (n_iter > 0) {
+    int k = k_of(0);
+    if (STAGE) load_s(k);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      load_a(k, u);
+      if (!STAGE) load_b(k, u);
+    }
+    for (int it = 0; it + 1 < n_iter; ++it) {
+      const int k_next = k_of(it + 1);
+      iteration(k, k_next, std::true_type{});
+      k = k_next;
+    }
+    iteration(k, 0, std::false_type{});
   }
   if (STAGE) __syncthreads();  // the staging regions become the reduction buffer
 
