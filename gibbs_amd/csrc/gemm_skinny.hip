@@ -9,10 +9,8 @@
 // its float32 partial Y[s] for the consumer to add in a fixed order.
 #include "common.h"
 #include "packed_layout.h"
+#include "kernels.h"
 #include <type_traits>
-
-int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
-                          long ldy, int rms, float eps, hipStream_t stream);
 
 namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;

@@ -32,6 +32,7 @@
 //                            (every row is one decoded token of a different request)
 #include "activation.h"
 #include "packed_layout.h"
+#include "kernels.h"
 #include <stdlib.h>
 #include <type_traits>
 
@@ -586,9 +587,6 @@ void note_layout(FusedArgs& a) {
 // In all of these, ldw == 0 means that W is in tile order (packed_layout.h), each row group by itself.
 //
 // Y[n, o] = scale_n * sum_k X[n, k] W[o, k], bfloat16 out; scale_n = 1/sqrt(mean_k X[n,k]^2 + eps) if rms.
-int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
-                          long ldy, int rms, float eps, hipStream_t stream);
-
 GIBBS_EXPORT int gibbs_skinny_store(const void* X, const void* W, void* Y, int N, int O, int I, long ldx, long ldw,
                                     long ldy, int rms, float eps, hipStream_t stream) {
   return gibbs_skinny_store_as(X, W, Y, GIBBS_BF16, N, O, I, ldx, ldw, ldy, rms, eps, stream);

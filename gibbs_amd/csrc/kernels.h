@@ -64,3 +64,8 @@ int gibbs_decode_tail(const float* logits, int V, long ld, int* ids, int* pos, i
                       int capacity, float* u, const float* u_all, const void* table, int table_dtype, int vocab, int hidden,
                       float* x, void* mirror, hipStream_t stream);
 }
+
+// Inside the library only: gibbs_skinny_store with the output's type given (bfloat16 or float32); what
+// gibbs_gemm_skinny hands whole sums of up to 16 rows to (gemm_skinny_fused.hip).
+int gibbs_skinny_store_as(const void* X, const void* W, void* Y, int out_dtype, int N, int O, int I, long ldx, long ldw,
+                          long ldy, int rms, float eps, hipStream_t stream);
