@@ -238,6 +238,9 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   constexpr int UB = BP ? U / 2 : U;     // B operands per iteration
   static_assert(U % 2 == 0, "pairs of MFMA steps");
   const int xoff = (BP ? half * 32 : 0) + g * 8;   // a lane's k within a B operand
+  // (three and four tiles of rows: the staged rows of X are asked for behind the iteration's products instead of
+  // before them: their registers would cost a second resident workgroup, or spill)
+  constexpr bool ROLL_S = NT <= 2;
   bf16x8 av[UA][FT][RG], bv[UB][NT], sv[NT][LPT];
   auto load_a = [&](int k, int u) {   // u: the iteration's A operand
     const long off = a_off(k / KU + u);
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
         for (int t = 0; t < NT; ++t) stage[(t * LPT + i) * WAVE + lane] = k_ok ? sv[t][i] : zero;
       }
-      if (more) load_s(k_next);
+      if (ROLL_S && more) load_s(k_next);
 #pragma unroll
       for (int u = 0; u < U; ++u)
 #pragma unroll
@@ -321,6 +324,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       }
     }
     }
+    if (STAGE && !ROLL_S && more) load_s(k_next);
   };
   if (n_iter > 0) {
     const int k = k_of(0);
