@@ -521,7 +521,8 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
   constexpr int tiles2_from = 192;   // pairs of tiles from which a workgroup takes two (measured at 33 to 64 rows)
   if constexpr (NT >= 3 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
     // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
-    if (a.O / 32 >= tiles2_from) {
+    // (also where single tiles would need a second round of workgroups that pairs do not: 257 to 383 tiles)
+    if (a.O / 32 >= tiles2_from || (ceil_div(a.O, 16) > 256 && a.O / 32 >= 128)) {
       gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(a);
       return;
     }
