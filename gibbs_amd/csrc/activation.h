@@ -16,3 +16,10 @@ __device__ __forceinline__ float activate(float g, int act) {
     default: return g * (1.0f / (1.0f + expf(-g)));   // silu
   }
 }
+
+// The same for an epilogue whose result is rounded to bfloat16: silu by the hardware's exponential and reciprocal
+// (a few units in the last place of float32), so that the serial tail of a product kernel stays short.
+__device__ __forceinline__ float activate_to_bf16(float g, int act) {
+  if (act == ACT_SILU) return g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+  return activate(g, act);
+}

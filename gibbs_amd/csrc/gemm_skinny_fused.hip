@@ -64,6 +64,7 @@ struct FusedArgs {
   long ldw, ldx;
   long group_stride;  // rows of W between row groups
   float eps;          // rms prologue
+  float inv_I;        // 1 / I
   // STORE / GLU / CONV: bfloat16 output [N, ldy] (STORE: or float32, Yf)
   bf16* Y;
   float* Yf;
@@ -431,7 +432,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       float tot = 0.f;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) tot += red_ss[w][t][r] + (BP ? red_ss[w][t][(r + 8) & 15] : 0.f);
-      scale = 1.0f / sqrtf(tot / (float)a.I + a.eps);
+      scale = __builtin_amdgcn_rsqf(tot * a.inv_I + a.eps);   // (1 ulp: the outputs are rounded to bfloat16, or added to a stream that is)
     }
     const bool full = o + 3 < a.O;
     if (EPI == EPI_STORE && a.Yf) {
@@ -463,7 +464,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
         const float gt = sum[0][t][i] * scale, up = sum[RG > 1 ? 1 : 0][t][i] * scale;
-        y[i] = (bf16)(activate(gt, a.act) * up);
+        y[i] = (bf16)(activate_to_bf16(gt, a.act) * up);
       }
     } else if (KC > 1) {  // EPI_CONV, operands at hand
       float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
@@ -582,6 +583,7 @@ int check_common(const char* what, const void* X, const void* W, int N, int O, i
 // A row stride of 0 says that W is in tile order; which of the two follows from the rows of a group (packed_layout.h).
 void note_layout(FusedArgs& a) {
   a.rotate = 1;
+  a.inv_I = 1.0f / (float)a.I;
   a.group_tiles = ceil_div(a.O, 16);
   if (a.ldw != 0) return;
   a.packed = pair_layout(a.O) ? 2 : 1;
