@@ -169,7 +169,9 @@ __global__ __launch_bounds__(512) void gemm_bf16_256_kernel(const bf16* __restri
     // A(t) and W(t) have landed (this thread's part; the barrier covers the others'); the four loads of
     // A(t+1) may still be on their way
     asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    __syncthreads();
+    // (the bare barrier: __syncthreads() carries a fence, for which the compiler waits until no load is in flight;
+    // a tile's operands were read from LDS into registers before its products, which stand before this barrier)
+    __builtin_amdgcn_s_barrier();
     const int kb = min(t + 1, nt - 1) * TK, ka = min(t + 2, nt - 1) * TK;
     bf16* dB = sB + ((t + 1) & 1) * TILE_ELEMS;
     bf16* dA = sA + ((t + 2) % 3) * TILE_ELEMS;
