@@ -88,10 +88,11 @@ struct FusedArgs {
 // product), 0 for any other length or epilogue.
 // FT: tiles of ROWS features that a workgroup computes from the same B operands (more rows of X
 // than one or two MFMA tiles: X is re-read from L2 by every workgroup, so a workgroup should use
-// each B operand for more of W).  Wave f sums tile f over the waves and runs its epilogue.
+// each B operand for more of W).  Wave f * NT + t sums tile f of features and tile t of rows over the waves
+// and runs its epilogue.
 template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC, bool STAGE, bool BP = false>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
-  static_assert(FT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only");
+  static_assert(FT * NT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only; a wave per tile of the result");
   // STAGE (more than a few rows of X): a wave brings its part of X in through LDS, 128 contiguous bytes or
   // more of a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory
   // pipe of a compute unit is bound by requests in flight, and from 8 rows on X is as many requests as W
@@ -175,13 +176,16 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
   // What the epilogue reads besides the product is asked for behind the first loads of the operands: the
   // product hides the latency (the state row hangs on a slot index, two dependent loads, and wave 0 would
-  // start its share of W that much later if they came first).  Wave 0 writes the outputs; its lane holds
-  // features o_epi .. +3 of row t*16 + r.
+  // start its share of W that much later if they came first).  The tiles of the result are written by a wave
+  // each: wave f * NT + t has tile f of the features and tile t of the rows (one wave alone spent as long
+  // on four tiles of rows as the product itself took); its lane holds features o_epi .. +3 of row n_epi.
   constexpr int KH = KC > 1 ? KC - 1 : 1;
-  const int o_epi = o0 + g * 4;
-  const bool epi_lane = wave == 0 && g * 4 < ROWS && o_epi < a.O;
-  float pre_x[NT][4];          // RESIDUAL: the stream; CONV: unused
-  float pre_hist[NT][KH][4];   // CONV: the state rows
+  const int f_epi = wave / NT, t_epi = wave % NT;
+  const int o_epi = o0 + f_epi * ROWS + g * 4;
+  const int n_epi = t_epi * 16 + r;
+  const bool epi_lane = wave < FT * NT && g * 4 < ROWS && o_epi < a.O && n_epi < a.N;
+  float pre_x[4];          // RESIDUAL: the stream; CONV: unused
+  float pre_hist[KH][4];   // CONV: the state rows
   float pre_taps[KC > 1 ? KC : 1][4], pre_bias[4];
   floatx4 acc[FT][RG][NT];
   floatx4 acc_hi[PAIR ? RG : 1][NT];   // 8 features: the products with X at k + 32 (rows 8..15 hold the features)
@@ -338,11 +342,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
   if (EPI == EPI_RESIDUAL) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = t * 16 + r;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) pre_x[t][i] = (epi_lane && n < a.N && o_epi + i < a.O) ? a.x[(size_t)n * a.O + o_epi + i] : 0.f;
-    }
+    for (int i = 0; i < 4; ++i) pre_x[i] = (epi_lane && o_epi + i < a.O) ? a.x[(size_t)n_epi * a.O + o_epi + i] : 0.f;
   }
   if (EPI == EPI_CONV && KC > 1) {
 #pragma unroll
@@ -352,18 +352,13 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       for (int j = 0; j < KC; ++j) pre_taps[j][i] = ok ? a.taps[(size_t)(o_epi + i) * KC + j] : 0.f;
       pre_bias[i] = (ok && a.bias) ? a.bias[o_epi + i] : 0.f;
     }
+    const float* st = a.state + (size_t)(epi_lane ? a.slot[n_epi] : 0) * a.slot_stride;
+    const int before = epi_lane ? a.ctx[n_epi] : 0;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      const int n = t * 16 + r;
-      const bool row = epi_lane && n < a.N;
-      const float* st = a.state + (size_t)(row ? a.slot[n] : 0) * a.slot_stride;
-      const int before = row ? a.ctx[n] : 0;
+    for (int j = 0; j < KH; ++j)
 #pragma unroll
-      for (int j = 0; j < KH; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          pre_hist[t][j][i] = (row && o_epi + i < a.O && before - (KC - 1) + j >= 0) ? st[(size_t)j * a.O + o_epi + i] : 0.f;
-    }
+      for (int i = 0; i < 4; ++i)
+        pre_hist[j][i] = (epi_lane && o_epi + i < a.O && before - (KC - 1) + j >= 0) ? st[(size_t)j * a.O + o_epi + i] : 0.f;
   }
 
   if (n_iter > 0) {
@@ -389,7 +384,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       if (g == r / 4) red_ss[wave][t][r] = d;   // (paired B operands: rows 8..15 are rows 0..7 at k + 32)
     }
   }
-  // the waves' partial products meet in LDS; wave f adds those of tile f in the order of the waves
+  // the waves' partial products meet in LDS; wave f * NT + t adds those of its tile in the order of the waves
   // (8 features: lanes g < 2 hold them in the first accumulator, lanes g >= 2 in the second; lane l < 32 then
   // adds what lane l + 32 left)
 #pragma unroll
@@ -399,34 +394,29 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
       for (int t = 0; t < NT; ++t) red[wave][f][q][t][lane] = (PAIR && !BP && g >= 2) ? acc_hi[PAIR ? q : 0][t] : acc[f][q][t];
   __syncthreads();
-  if (wave >= FT) return;
-  const int tile = wave;
+  if (wave >= FT * NT) return;
   // (paired B operands: the second half of feature (g, i) and row r is at rows + 8, columns + 8 of the tile)
   const int partner = BP ? (lane + 40) & 63 : (lane & 31) + 32;   // (8 features only)
-  floatx4 sum[RG][NT];
+  floatx4 sum[RG];
 #pragma unroll
-  for (int q = 0; q < RG; ++q)
+  for (int q = 0; q < RG; ++q) {
+    sum[q] = red[0][f_epi][q][t_epi][lane];
+    if (PAIR) sum[q] += red[0][f_epi][q][t_epi][partner];
+  }
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      sum[q][t] = red[0][tile][q][t][lane];
-      if (PAIR) sum[q][t] += red[0][tile][q][t][partner];
-    }
-#pragma unroll(RG * NT <= 2 ? WAVES : 1)
   for (int w = 1; w < WAVES; ++w)
 #pragma unroll
-    for (int q = 0; q < RG; ++q)
-#pragma unroll
-      for (int t = 0; t < NT; ++t) {
-        sum[q][t] += red[w][tile][q][t][lane];
-        if (PAIR) sum[q][t] += red[w][tile][q][t][partner];
-      }
+    for (int q = 0; q < RG; ++q) {
+      sum[q] += red[w][f_epi][q][t_epi][lane];
+      if (PAIR) sum[q] += red[w][f_epi][q][t_epi][partner];
+    }
 
-  // D[feature g*4 + i][row r] of tile t: lane holds 4 consecutive features of one row
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    const int n = t * 16 + r;
-    const int o = o0 + tile * ROWS + g * 4;
-    if (n >= a.N || g * 4 >= ROWS || o >= a.O) continue;
+  // D[feature g*4 + i][row r] of the tile: lane holds 4 consecutive features of one row
+  {
+    const int t = t_epi;
+    const int n = n_epi;
+    const int o = o_epi;
+    if (n >= a.N || g * 4 >= ROWS || o >= a.O) return;
     float scale = 1.f;
     if (RMS) {
       float tot = 0.f;
@@ -438,17 +428,17 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     if (EPI == EPI_STORE && a.Yf) {
       float* y = a.Yf + (size_t)n * a.ldy + o;
       if (full && a.y_vec) {
-        *(floatx4*)y = floatx4{sum[0][t][0] * scale, sum[0][t][1] * scale, sum[0][t][2] * scale, sum[0][t][3] * scale};
+        *(floatx4*)y = floatx4{sum[0][0] * scale, sum[0][1] * scale, sum[0][2] * scale, sum[0][3] * scale};
       } else {
-        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = sum[0][t][i] * scale;
+        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = sum[0][i] * scale;
       }
     } else if (EPI == EPI_STORE) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       if (full && a.ldy % 4 == 0) {
-        *(bf16x4*)y = bf16x4{(bf16)(sum[0][t][0] * scale), (bf16)(sum[0][t][1] * scale), (bf16)(sum[0][t][2] * scale),
-                             (bf16)(sum[0][t][3] * scale)};
+        *(bf16x4*)y = bf16x4{(bf16)(sum[0][0] * scale), (bf16)(sum[0][1] * scale), (bf16)(sum[0][2] * scale),
+                             (bf16)(sum[0][3] * scale)};
       } else {
-        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = (bf16)(sum[0][t][i] * scale);
+        for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = (bf16)(sum[0][i] * scale);
       }
     } else if (EPI == EPI_RESIDUAL) {
       float* xp = a.x + (size_t)n * a.O + o;
@@ -456,14 +446,14 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         if (o + i >= a.O) break;
-        const float v = pre_x[t][i] + sum[0][t][i] * scale;
+        const float v = pre_x[i] + sum[0][i] * scale;
         xp[i] = v;
         bp[i] = (bf16)v;
       }
     } else if (EPI == EPI_GLU) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
-        const float gt = sum[0][t][i] * scale, up = sum[RG > 1 ? 1 : 0][t][i] * scale;
+        const float gt = sum[0][i] * scale, up = sum[RG > 1 ? 1 : 0][i] * scale;
         y[i] = (bf16)(activate_to_bf16(gt, a.act) * up);
       }
     } else if (KC > 1) {  // EPI_CONV, operands at hand
@@ -473,16 +463,16 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       for (int i = 0; i < 4; ++i) {
         if (o + i >= a.O) break;
         const int c = o + i;
-        const float bx = (sum[0][t][i] * scale) * (sum[RG > 2 ? 2 : 0][t][i] * scale);
-        const float cg = sum[RG > 1 ? 1 : 0][t][i] * scale;
+        const float bx = (sum[0][i] * scale) * (sum[RG > 2 ? 2 : 0][i] * scale);
+        const float cg = sum[RG > 1 ? 1 : 0][i] * scale;
         float cv = 0.f;
 #pragma unroll
-        for (int j = 0; j < KC - 1; ++j) cv = fmaf(pre_taps[j][i], pre_hist[t][j][i], cv);
+        for (int j = 0; j < KC - 1; ++j) cv = fmaf(pre_taps[j][i], pre_hist[j][i], cv);
         cv = fmaf(pre_taps[KC - 1][i], bx, cv);
         if (a.bias) cv += pre_bias[i];
         y[i] = (bf16)(cg * cv);
 #pragma unroll
-        for (int j = 0; j + 1 < KC - 1; ++j) st[(size_t)j * a.O + c] = pre_hist[t][j + 1][i];
+        for (int j = 0; j + 1 < KC - 1; ++j) st[(size_t)j * a.O + c] = pre_hist[j + 1][i];
         st[(size_t)(KC - 2) * a.O + c] = bx;
       }
     } else {  // EPI_CONV, any kernel length
@@ -492,8 +482,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
       bf16* y = a.Y + (size_t)n * a.ldy + o;
       for (int i = 0; i < 4 && o + i < a.O; ++i) {
         const int c = o + i;
-        const float bx = (sum[0][t][i] * scale) * (sum[RG > 2 ? 2 : 0][t][i] * scale);
-        const float cg = sum[RG > 1 ? 1 : 0][t][i] * scale;
+        const float bx = (sum[0][i] * scale) * (sum[RG > 2 ? 2 : 0][i] * scale);
+        const float cg = sum[RG > 1 ? 1 : 0][i] * scale;
         float hist[MAX_TAPS - 1];
         float cv = 0.f;
 #pragma unroll
