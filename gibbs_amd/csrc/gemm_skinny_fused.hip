@@ -68,7 +68,7 @@ struct FusedArgs {
   // STORE / GLU / CONV: bfloat16 output [N, ldy] (STORE: or float32, Yf)
   bf16* Y;
   float* Yf;
-  int y_vec;
+  int y_vec;   // a lane's four features take one store (rows and pointers are aligned for it)
   long ldy;
   // RESIDUAL
   float* x;   // [N, O] float32, updated in place
@@ -443,37 +443,55 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
     } else if (EPI == EPI_RESIDUAL) {
       float* xp = a.x + (size_t)n * a.O + o;
       bf16* bp = a.xb + (size_t)n * a.O + o;
+      float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (o + i >= a.O) break;
-        const float v = pre_x[i] + sum[0][i] * scale;
-        xp[i] = v;
-        bp[i] = (bf16)v;
+      for (int i = 0; i < 4; ++i) v[i] = pre_x[i] + sum[0][i] * scale;
+      if (full && a.y_vec) {   // (a lane's four features in one store each)
+        *(floatx4*)xp = floatx4{v[0], v[1], v[2], v[3]};
+        *(bf16x4*)bp = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+      } else {
+        for (int i = 0; i < 4 && o + i < a.O; ++i) { xp[i] = v[i]; bp[i] = (bf16)v[i]; }
       }
     } else if (EPI == EPI_GLU) {
       bf16* y = a.Y + (size_t)n * a.ldy + o;
-      for (int i = 0; i < 4 && o + i < a.O; ++i) {
+      bf16 v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
         const float gt = sum[0][i] * scale, up = sum[RG > 1 ? 1 : 0][i] * scale;
-        y[i] = (bf16)(activate_to_bf16(gt, a.act) * up);
+        v[i] = (bf16)(activate_to_bf16(gt, a.act) * up);
       }
+      if (full && a.y_vec) *(bf16x4*)y = bf16x4{v[0], v[1], v[2], v[3]};
+      else for (int i = 0; i < 4 && o + i < a.O; ++i) y[i] = v[i];
     } else if (KC > 1) {  // EPI_CONV, operands at hand
       float* st = a.state + (size_t)a.slot[n] * a.slot_stride;
       bf16* y = a.Y + (size_t)n * a.ldy + o;
+      float bx[4];
+      bf16 v[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if (o + i >= a.O) break;
-        const int c = o + i;
-        const float bx = (sum[0][i] * scale) * (sum[RG > 2 ? 2 : 0][i] * scale);
+        bx[i] = (sum[0][i] * scale) * (sum[RG > 2 ? 2 : 0][i] * scale);
         const float cg = sum[RG > 1 ? 1 : 0][i] * scale;
         float cv = 0.f;
 #pragma unroll
         for (int j = 0; j < KC - 1; ++j) cv = fmaf(pre_taps[j][i], pre_hist[j][i], cv);
-        cv = fmaf(pre_taps[KC - 1][i], bx, cv);
+        cv = fmaf(pre_taps[KC - 1][i], bx[i], cv);
         if (a.bias) cv += pre_bias[i];
-        y[i] = (bf16)(cg * cv);
+        v[i] = (bf16)(cg * cv);
+      }
+      if (full && a.y_vec) {
+        *(bf16x4*)y = bf16x4{v[0], v[1], v[2], v[3]};
 #pragma unroll
-        for (int j = 0; j + 1 < KC - 1; ++j) st[(size_t)j * a.O + c] = pre_hist[j + 1][i];
-        st[(size_t)(KC - 2) * a.O + c] = bx;
+        for (int j = 0; j + 1 < KC - 1; ++j)
+          *(floatx4*)(st + (size_t)j * a.O + o) = floatx4{pre_hist[j + 1][0], pre_hist[j + 1][1], pre_hist[j + 1][2], pre_hist[j + 1][3]};
+        *(floatx4*)(st + (size_t)(KC - 2) * a.O + o) = floatx4{bx[0], bx[1], bx[2], bx[3]};
+      } else {
+        for (int i = 0; i < 4 && o + i < a.O; ++i) {
+          const int c = o + i;
+          y[i] = v[i];
+#pragma unroll
+          for (int j = 0; j + 1 < KC - 1; ++j) st[(size_t)j * a.O + c] = pre_hist[j + 1][i];
+          st[(size_t)(KC - 2) * a.O + c] = bx[i];
+        }
       }
     } else {  // EPI_CONV, any kernel length
       const int K = a.K;
@@ -614,6 +632,7 @@ GIBBS_EXPORT int gibbs_skinny_residual(const void* X, const void* W, float* x, v
   FusedArgs a{};
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = O; a.I = I; a.ldw = ldw; a.ldx = ldx; note_layout(a);
   a.x = x; a.xb = (bf16*)xb;
+  a.y_vec = O % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)xb % 8) == 0;
   launch_nt<1, false, EPI_RESIDUAL>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_residual");
 }
@@ -627,6 +646,7 @@ GIBBS_EXPORT int gibbs_skinny_glu(const void* X, const void* W, void* Y, int N, 
   FusedArgs a{};
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = F; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.group_stride = F; a.Y = (bf16*)Y; a.ldy = ldy; a.act = act;
+  a.y_vec = ldy % 4 == 0 && ((uintptr_t)Y % 8) == 0;
   if (rms) launch_nt<2, true, EPI_GLU>(a, stream);
   else launch_nt<2, false, EPI_GLU>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_glu");
@@ -644,6 +664,7 @@ GIBBS_EXPORT int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N,
   a.W = (const bf16*)W; a.X = (const bf16*)X; a.N = N; a.O = C; a.I = I; a.ldw = ldw; a.ldx = ldx; a.eps = eps; note_layout(a);
   a.group_stride = C; a.Y = (bf16*)Y; a.ldy = C;
   a.taps = taps; a.bias = bias; a.state = state; a.slot_stride = slot_stride; a.slot = slot; a.ctx = ctx; a.K = K;
+  a.y_vec = C % 4 == 0 && slot_stride % 4 == 0 && ((uintptr_t)Y % 8) == 0 && ((uintptr_t)state % 16) == 0;
   if (rms) launch_conv<true>(a, stream);
   else launch_conv<false>(a, stream);
   GIBBS_LAUNCH_STATUS("skinny_conv");
