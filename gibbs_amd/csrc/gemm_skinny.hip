@@ -179,16 +179,15 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_kernel(const bf16* _
   }
   if (STAGE) __syncthreads();  // the staging regions become the reduction buffer
 
-  // the waves' sums meet in LDS; wave f adds those of tile f in the order of the waves
+  // the waves' sums meet in LDS; the tiles of the result (FT of features by NT of rows) go round the waves, each
+  // adding its tiles' parts in the order of the waves
 #pragma unroll
   for (int f = 0; f < FT; ++f)
 #pragma unroll
     for (int t = 0; t < NT; ++t) red[wave][f][t][lane] = acc[f][t];
   __syncthreads();
-  if (wave >= FT) return;
-  const int tile = wave;
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
+  for (int unit = wave; unit < FT * NT; unit += WAVES) {
+    const int tile = unit / NT, t = unit % NT;
     floatx4 sum = red[0][tile][t][lane];
 #pragma unroll
     for (int w = 1; w < WAVES; ++w) sum += red[w][tile][t][lane];
