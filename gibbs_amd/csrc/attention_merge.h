@@ -32,6 +32,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
         av[j][c] = ps[s * stride + 2 + (e < hd ? e : 0)];
       }
     }
+    __builtin_amdgcn_sched_barrier(0);   // every load is asked for before the first value is used: one round trip
     float M = -INFINITY;
 #pragma unroll
     for (int j = 0; j < MERGE_AT_ONCE; ++j)
