@@ -94,6 +94,10 @@ struct DecodeArgs {
   int rot, variant;       // 0 half split, 1 interleaved
   const float2* cs_table; // [table_len, rot/2] (cos, sin) of the first positions, or null
   int table_len;
+  // A row's whole block table fits the staging area in LDS (no window, the caller's bound on the keys): its first
+  // n_ids page ids are asked for at once, before the row's position is known (one dependent load less in front
+  // of the first keys).  A row that is beyond the bound after all takes the ids of its slice as it would without.
+  int ids_whole, n_ids;
 };
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -136,6 +140,15 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   const int e0 = sub * EPL;
   const bool active = e0 < hd;
 
+  // (row_req null: row n is request n, as in a step of decoded tokens alone)
+  const int* table = a.table + (size_t)(a.row_req ? a.row_req[row] : row) * a.max_pages;
+  constexpr int PRE = (SEG_PAGES + NW * WAVE - 1) / (NW * WAVE);
+  int pre_page[PRE];
+#pragma unroll
+  for (int i = 0; i < PRE; ++i) {
+    const int j = threadIdx.x + i * NW * WAVE;
+    pre_page[i] = (a.ids_whole && j < a.n_ids) ? table[j] : 0;
+  }
   const int p = a.pos[row];
   const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
   const int len = p + 1 - lo;
@@ -144,7 +157,6 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   per = (per + UNIT - 1) / UNIT * UNIT;
   const int k0 = lo + split * per;
   const int k1 = min(k0 + per, p + 1);
-  const int* table = a.table + (size_t)a.row_req[row] * a.max_pages;
   const bf16* qrow = qkv + (size_t)row * a.ldq;
 
   // Everything that does not hang on earlier arithmetic is asked for first: the query heads, the
@@ -163,14 +175,45 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
     knew_raw = *(const uint4*)(qrow + (size_t)(a.nh + kvh) * hd + e0);
     vnew_raw = *(const uint4*)(qrow + (size_t)(a.nh + a.nkv + kvh) * hd + e0);
   }
-  constexpr int PRE = (SEG_PAGES + NW * WAVE - 1) / (NW * WAVE);
-  const int first_page0 = a.page_shift >= 0 ? k0 >> a.page_shift : k0 / a.page_size;
-  const int seg1_0 = min(k1, (first_page0 + SEG_PAGES) * a.page_size);
-  int pre_page[PRE];
+  const bool whole = a.ids_whole && p < a.n_ids * a.page_size;
+  const int first_page0 = whole ? 0 : (a.page_shift >= 0 ? k0 >> a.page_shift : k0 / a.page_size);
+  const int seg1_0 = whole ? k1 : min(k1, (first_page0 + SEG_PAGES) * a.page_size);
+  if (!whole) {
+#pragma unroll
+    for (int i = 0; i < PRE; ++i) {
+      const int j = threadIdx.x + i * NW * WAVE;
+      pre_page[i] = (j < SEG_PAGES && (first_page0 + j) * a.page_size < seg1_0) ? table[first_page0 + j] : 0;
+    }
+  }
+
+  // The first segment's page ids go to LDS, and the loads of the wave's first tile of keys are asked for, before
+  // the queries and the row's own key are prepared: the preparation (rotation factors that hang on the position,
+  // norms, rotation) runs while those loads are on their way.
 #pragma unroll
   for (int i = 0; i < PRE; ++i) {
     const int j = threadIdx.x + i * NW * WAVE;
-    pre_page[i] = (j < SEG_PAGES && (first_page0 + j) * a.page_size < seg1_0) ? table[first_page0 + j] : 0;
+    if (j < SEG_PAGES && (whole ? j < a.n_ids : (first_page0 + j) * a.page_size < seg1_0)) s_pages[j] = pre_page[i];
+  }
+  __syncthreads();  // the first segment's ids are in LDS
+  // a key's and a value's 16 bytes of this lane; first_page: the page whose id is s_pages[0]
+  auto fetch = [&](int key, int seg1, int first_page, uint4& kr, uint4& vr) {
+    kr = vr = make_uint4(0, 0, 0, 0);
+    if (key < seg1 && !(RAW && key == p) && active) {
+      const int lp = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
+      const int page = min(max(s_pages[lp - first_page], 0), a.num_pages - 1);  // never read outside the pool
+      const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
+      kr = *(const uint4*)(kpages + off);
+      vr = *(const uint4*)(vpages + off);
+    }
+  };
+  constexpr int LPT = MM ? TILE / KPW : 1;   // loads of K (and of V) per tile of the matrix-core walk
+  uint4 kreg[LPT], vreg[LPT];
+  if constexpr (MM) {
+    // (the matrix-core walk has one segment: the launcher sees to it that a slice's ids fit the staging area)
+    if (wave * TILE < seg1_0 - k0) {
+#pragma unroll
+      for (int i = 0; i < LPT; ++i) fetch(k0 + wave * TILE + i * KPW + grp, seg1_0, first_page0, kreg[i], vreg[i]);
+    }
   }
 
   Rot8 rt;
@@ -230,19 +273,19 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   // The slice's page ids go to LDS first (one round trip for all of them, instead of a dependent
   // table load in front of every key's loads); the loads of the next two keys are issued before the
   // current key is worked on, so that memory latency overlaps the arithmetic.
+  __syncthreads();  // the queries and the row's own key and value are in LDS
   for (int seg0 = k0; seg0 < k1; seg0 += SEG_PAGES * a.page_size) {
-    const int first_page = a.page_shift >= 0 ? seg0 >> a.page_shift : seg0 / a.page_size;
-    const int seg1 = min(k1, (first_page + SEG_PAGES) * a.page_size);
-    if (seg0 != k0) __syncthreads();  // the previous segment's ids are no longer read
+    const int first_page = seg0 == k0 ? first_page0 : (a.page_shift >= 0 ? seg0 >> a.page_shift : seg0 / a.page_size);
+    const int seg1 = seg0 == k0 ? seg1_0 : min(k1, (first_page + SEG_PAGES) * a.page_size);
+    if (seg0 != k0) {
+      __syncthreads();  // the previous segment's ids are no longer read
 #pragma unroll
-    for (int i = 0; i < PRE; ++i) {
-      const int j = threadIdx.x + i * NW * WAVE;
-      if (j < SEG_PAGES && (first_page + j) * a.page_size < seg1) {
-        const int page = seg0 == k0 ? pre_page[i] : table[first_page + j];
-        s_pages[j] = page;
+      for (int i = 0; i < PRE; ++i) {
+        const int j = threadIdx.x + i * NW * WAVE;
+        if (j < SEG_PAGES && (first_page + j) * a.page_size < seg1) s_pages[j] = table[first_page + j];
       }
+      __syncthreads();
     }
-    __syncthreads();  // the ids, and at the first segment the queries and the row's own key and value, are in LDS
     if (seg0 == k0) {
       if constexpr (MM) {
         // B operands of S^T = K Q^T: column lr is query head g0 + lr, d = s*32 + g4*8 .. +8
@@ -277,16 +320,6 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
         *(uint4*)(vpages + off) = make_uint4(vw[0], vw[1], vw[2], vw[3]);
       }
     }
-    auto fetch = [&](int key, uint4& kr, uint4& vr) {
-      kr = vr = make_uint4(0, 0, 0, 0);
-      if (key < seg1 && !(RAW && key == p) && active) {
-        const int lp = a.page_shift >= 0 ? key >> a.page_shift : key / a.page_size;
-        const int page = min(max(s_pages[lp - first_page], 0), a.num_pages - 1);  // never read outside the pool
-        const size_t off = (((size_t)page * a.nkv + kvh) * a.page_size + (key - lp * a.page_size)) * hd + e0;
-        kr = *(const uint4*)(kpages + off);
-        vr = *(const uint4*)(vpages + off);
-      }
-    };
     if constexpr (MM) {
       // The wave's tiles of the slice: keys k0 + j*32 .. +32 for j = wave, wave + NW, ...  A tile travels
       // memory -> registers (one tile ahead) -> the wave's own patch of LDS (no barrier: only this wave
@@ -295,18 +328,14 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
       // transposing reads of the tile as it was stored.
       bf16 (*tK)[LDT] = reinterpret_cast<bf16 (*)[LDT]>(s_tiles + (size_t)wave * 2 * TILE * LDT);
       bf16 (*tV)[LDT] = tK + TILE;
-      constexpr int LPT = TILE / KPW;   // loads of K (and of V) per tile
-      uint4 kreg[LPT], vreg[LPT];
       auto fetch_tile = [&](int t0) {
 #pragma unroll
-        for (int i = 0; i < LPT; ++i) fetch(t0 + i * KPW + grp, kreg[i], vreg[i]);
+        for (int i = 0; i < LPT; ++i) fetch(t0 + i * KPW + grp, seg1, first_page, kreg[i], vreg[i]);
       };
       const float scale2 = a.scale * 1.44269504088896340736f;
       const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
       const int n_tiles = (seg1 - k0 + TILE - 1) / TILE;
-      int j = wave;
-      if (j < n_tiles) fetch_tile(k0 + j * TILE);
-      for (; j < n_tiles; j += NW) {
+      for (int j = wave; j < n_tiles; j += NW) {   // (the wave's first tile was asked for before the preparation)
         const int t0 = k0 + j * TILE;
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the reads of the previous tile are through
         if (active) {
@@ -381,10 +410,10 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
       // the wave's first key of this segment keeps the global stride pattern k0 + (NW it + wave) KPW + grp
       int key = k0 + wave * KPW + grp;
       if (key < seg0) key += (seg0 - key + NW * KPW - 1) / (NW * KPW) * (NW * KPW);
-      fetch(key, kraw[0], vraw[0]);
-      fetch(key + NW * KPW, kraw[1], vraw[1]);
+      fetch(key, seg1, first_page, kraw[0], vraw[0]);
+      fetch(key + NW * KPW, seg1, first_page, kraw[1], vraw[1]);
       for (; key < seg1; key += NW * KPW) {
-        fetch(key + 2 * NW * KPW, kraw[2], vraw[2]);
+        fetch(key + 2 * NW * KPW, seg1, first_page, kraw[2], vraw[2]);
         __builtin_amdgcn_sched_barrier(0);  // the loads above stay ahead of the arithmetic below
         float kf[EPL], vf[EPL];
         if (RAW && key == p) {
@@ -529,6 +558,9 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   const bool mm_can = a.hd % 16 == 0 && a.hd <= 128 && longest / a.page_size + 2 <= SEG_PAGES;
   GIBBS_REQUIRE(kind != 2 || mm_can, "attention_decode: the matrix-core kernel takes head sizes in steps of 16 up to 128 and key slices of at most %d pages (head size %d, %ld keys a slice)", SEG_PAGES - 2, a.hd, longest);
   const bool mm = kind == 2 || (kind == 0 && mm_can);
+  const long ids = (bound + a.page_size - 1) / a.page_size;
+  a.ids_whole = a.window == 0 && ids <= SEG_PAGES;
+  a.n_ids = (int)min(ids, (long)a.max_pages);
   if (lanes <= 2) launch_waves<2, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);
   else if (lanes <= 4) launch_waves<4, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);
   else if (lanes <= 8) launch_waves<8, RAW>(waves, mm, gt, grid, stream, q, kpages, vpages, partial, out, a);

@@ -333,6 +333,10 @@ struct Exec {
     return out;
   }
 
+  // A step of one token per request: row n is request n, and the attention need not look that up (a dependent
+  // load less in front of its page ids).
+  bool rows_are_requests() const { return a.max_q == 1 && a.n_rows == a.n_req; }
+
   // decoded tokens from the raw projection: q/k norm, rotation, the cache write and attention in one kernel
   void* attend_decoded(const AttnP& t, const void* qkv) {
     const int N = a.n_rows;
@@ -341,7 +345,7 @@ struct Exec {
     float* partial = n_splits > 1 ? (float*)take(gibbs_attention_decode_workspace(N, t.nh, t.hd, n_splits) * 4) : nullptr;
     void* out = take((long)N * t.nh * t.hd * 2);
     RUN(gibbs_attention_decode_fused(qkv, t.kpages, t.vpages, out, partial, t.q_gain, t.k_gain, t.qk_eps, t.inv_freq, t.rot,
-                                     t.variant, t.cos_sin, t.cos_sin ? t.table_len : 0, a.pos, a.row_req, a.tables[t.group],
+                                     t.variant, t.cos_sin, t.cos_sin ? t.table_len : 0, a.pos, rows_are_requests() ? nullptr : a.row_req, a.tables[t.group],
                                      a.widths[t.group], t.page_size, t.num_pages, N, t.nh, t.nkv, t.hd,
                                      (long)(t.nh + 2 * t.nkv) * t.hd, (long)t.nh * t.hd, t.scale, t.window, n_splits, waves, 0,
                                      a.max_seq, a.stream));
