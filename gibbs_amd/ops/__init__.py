@@ -342,7 +342,7 @@ def skinny_conv(x: torch.Tensor, w_in: torch.Tensor, taps: torch.Tensor, bias: O
 
 def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
                            vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor,
-                           row_req: torch.Tensor, scale: float, *, q_gain: Optional[torch.Tensor],
+                           row_req: Optional[torch.Tensor], scale: float, *, q_gain: Optional[torch.Tensor],
                            k_gain: Optional[torch.Tensor], eps: float, inv_freq: Optional[torch.Tensor],
                            rotary_dim: int, variant: str, window: Optional[int] = None,
                            max_seq: int = 0, n_splits: Optional[int] = None,
@@ -361,7 +361,11 @@ def attention_decode_fused(qkv: torch.Tensor, n_rows: int, nh: int, nkv: int, hd
     num_pages, page_size = _check_pages(kpages, nkv, hd, qkv.dtype)
     assert _check_pages(vpages, nkv, hd, qkv.dtype) == (num_pages, page_size)
     assert table.dim() == 2 and table.shape[0] >= n_req
-    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos")
+    if row_req is not None:   # (None: row n is request n)
+        _i32(row_req, n_rows, "row_req")
+    else:
+        assert n_rows <= table.shape[0], "rows without a row-to-request map are requests"
     for g in (q_gain, k_gain):
         assert g is None or (g.dtype == torch.float32 and g.shape == (hd,) and g.is_contiguous())
     if inv_freq is not None:
@@ -534,12 +538,14 @@ def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, 
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
-                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: torch.Tensor,
+                     vpages: torch.Tensor, table: torch.Tensor, n_req: int, pos: torch.Tensor, row_req: Optional[torch.Tensor],
                      scale: float, window: Optional[int] = None, max_seq: int = 0, n_splits: Optional[int] = None,
                      out: Optional[torch.Tensor] = None, waves: Optional[int] = None, kind: str = "auto") -> torch.Tensor:
     """bfloat16 paged attention for rows with few queries and long caches (decoded tokens): the
     keys of each (row, kv head) are cut into `n_splits` slices that run as workgroups of their own
-    and are merged afterwards.  Same operands and result as `attention_plain`."""
+    and are merged afterwards.  Same operands and result as `attention_plain`; `row_req` None says that row n is
+    request n.  `max_seq`, if given, bounds the keys of every row; it steers how the kernel asks for page ids and
+    cuts slices (a row beyond it is still right as long as a slice's page ids fit the kernel's staging area)."""
     require_cuda(q, kpages, vpages, table, pos, row_req)
     if q.dtype != torch.bfloat16:
         raise KernelError("attention_decode is the bfloat16 kernel; the float32 path uses attention_plain")
@@ -549,7 +555,11 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
     num_pages, page_size = _check_pages(kpages, nkv, hd, q.dtype)
     assert _check_pages(vpages, nkv, hd, q.dtype) == (num_pages, page_size)
     assert table.dim() == 2 and table.shape[0] >= n_req
-    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos"); _i32(row_req, n_rows, "row_req")
+    _i32(table, n_req, "block table"); _i32(pos, n_rows, "pos")
+    if row_req is not None:   # (None: row n is request n)
+        _i32(row_req, n_rows, "row_req")
+    else:
+        assert n_rows <= table.shape[0], "rows without a row-to-request map are requests"
     if n_splits is None or waves is None:
         auto_splits, auto_waves = decode_splits(n_rows, nkv, nh // nkv, max_seq, hd, kind, page_size)
         n_splits = auto_splits if n_splits is None else n_splits

@@ -334,6 +334,31 @@ def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves,
     close(out, plain, dtype, "decode vs plain kernel", bf16=1e-2)
 
 
+@pytest.mark.parametrize("kind", ["valu", "mfma"])
+@pytest.mark.parametrize("n_splits", [1, 4])
+@pytest.mark.parametrize("bound", [0, 64, 700])
+def test_attention_decode_rows_as_requests_and_rows_beyond_the_bound(bound, n_splits, kind):
+    """Without a row-to-request map row n is request n; and the caller's bound on the keys only steers the
+    kernel (it asks for a row's page ids before it knows the row's position when the whole table fits its
+    staging area): rows beyond the bound take the ids of their slice afterwards and are as right."""
+    from gibbs_amd import ops
+    dtype, nh, nkv, hd, page = torch.bfloat16, 8, 2, 64, 8
+    seq_lens = [700, 1, 33, 16, 300]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, 180, seed=11)
+    positions = [l - 1 for l in seq_lens]
+    pos = i32(positions)
+    q = rnd(5, nh * hd, dtype=dtype, seed=12)
+    scale = 1 / math.sqrt(hd)
+    out = ops.attention_decode(q, 5, nh, nkv, hd, kp, vp, table, 5, pos, None, scale, None, max_seq=bound,
+                               n_splits=n_splits, waves=4, kind=kind)
+    mapped = ops.attention_decode(q, 5, nh, nkv, hd, kp, vp, table, 5, pos, i32([0, 1, 2, 3, 4]), scale, None, max_seq=bound,
+                                  n_splits=n_splits, waves=4, kind=kind)
+    assert torch.equal(out, mapped)
+    for r in range(5):
+        want = attention_reference(q[r:r + 1].view(1, nh, hd), ks[r], vs[r], [positions[r]], scale, None)
+        close(out[r].view(1, nh, hd), want, dtype, f"decode attention row {r}", bf16=1e-2)
+
+
 @pytest.mark.parametrize("n_splits", [1, 3, 7])
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
                                                    (32, 8, 64, 16, None), (4, 2, 128, 16, None), (2, 2, 96, 64, 100),
