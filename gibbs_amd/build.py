@@ -24,8 +24,11 @@ LIB_NAME = "libgibbs_hip.so"
 ARCH = "gfx950"
 # packed-fp32 instructions are kept off for every kernel (the host pass warns that it does
 # not know the feature; that is harmless).
+# A kernel's first 16 dwords of scalar arguments arrive in registers with the wave (gfx950 preloads them) instead
+# of by a load that everything else in the kernel waits for; arguments passed as a struct are not preloaded.
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fvisibility=hidden",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result",
+               "-mllvm", "-amdgpu-kernarg-preload-count=16"]
 
 
 HOST_SRC = os.path.join(CSRC, "host")

@@ -91,7 +91,14 @@ struct FusedArgs {
 // each B operand for more of W).  Wave f * NT + t sums tile f of features and tile t of rows over the waves
 // and runs its epilogue.
 template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC, bool STAGE, bool BP = false>
-__global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedArgs a) {
+__global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const bf16* W, const bf16* X, int N, int O, int I, int packed,
+                                                                         int ktiles, int rotate, long group_tiles, long ldw,
+                                                                         long ldx, FusedArgs rest) {
+  // What the first loads need comes as 16 dwords of scalar arguments, which arrive in registers with the wave;
+  // the rest of the arguments is a struct, which the kernel loads as it needs it.
+  FusedArgs a = rest;
+  a.W = W; a.X = X; a.N = N; a.O = O; a.I = I; a.packed = packed; a.ktiles = ktiles; a.rotate = rotate;
+  a.group_tiles = group_tiles; a.ldw = ldw; a.ldx = ldx;
   static_assert(FT * NT <= WAVES && (FT == 1 || EPI == EPI_STORE || EPI == EPI_GLU), "several tiles: store and GLU only; a wave per tile of the result");
   // STAGE (more than a few rows of X): a wave brings its part of X in through LDS, 128 contiguous bytes or
   // more of a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory
@@ -525,6 +532,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(FusedAr
   }
 }
 
+#define FUSED_KERNEL_ARGS(a) (a).W, (a).X, (a).N, (a).O, (a).I, (a).packed, (a).ktiles, (a).rotate, (a).group_tiles, (a).ldw, (a).ldx, (a)
+
 template <int NT, bool ST, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
   constexpr int tiles2_from = 192;   // pairs of tiles from which a workgroup takes two (measured at 33 to 64 rows)
@@ -532,7 +541,7 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
     // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
     // (also where single tiles would need a second round of workgroups that pairs do not: 257 to 383 tiles)
     if (a.O / 32 >= tiles2_from || (ceil_div(a.O, 16) > 256 && a.O / 32 >= 128)) {
-      gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(a);
+      gemm_skinny_fused_kernel<NT, RG, 16, 2, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 32), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
       return;
     }
   }
@@ -540,19 +549,19 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
   if ((NT <= 2 || EPI == EPI_CONV) && pair_layout(a.O)) {
     if constexpr (NT == 1 && !ST) {
       if (a.N <= 8) {   // the rows of X fit half a tile: paired B operands
-        gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+        gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
         return;
       }
     }
-    gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
   } else {
     if constexpr (NT == 1 && !ST) {
       if (a.N <= 8) {
-        gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+        gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
         return;
       }
     }
-    gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(a);
+    gemm_skinny_fused_kernel<NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
   }
 }
 
