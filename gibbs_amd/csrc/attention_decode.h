@@ -117,7 +117,13 @@ __device__ __forceinline__ void fold(float& ma, float& la, float* aa, float mb, 
 template <int LPK, int GT, bool RAW, int NW, bool MM>
 __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void attention_decode_kernel(const bf16* __restrict__ qkv, bf16* __restrict__ kpages,
                                                                bf16* __restrict__ vpages, float* __restrict__ partial,
-                                                               bf16* __restrict__ out, DecodeArgs a) {
+                                                               bf16* __restrict__ out, const int* __restrict__ pos_,
+                                                               const int* __restrict__ table_, DecodeArgs rest) {
+  // (the pointers that the first loads hang on are scalar arguments: those arrive in registers with the wave,
+  // the struct's fields by loads)
+  DecodeArgs a = rest;
+  a.pos = pos_;
+  a.table = table_;
   constexpr int KPW = WAVE / LPK;
   constexpr int MAX_HD = LPK * EPL;
   __shared__ float s_ml[NW][GT][2];
@@ -512,10 +518,10 @@ template <int LPK, bool RAW, int NW, bool MM>
 void launch_decode(int gt, dim3 grid, hipStream_t stream, const bf16* q, bf16* k, bf16* v, float* partial, bf16* out,
                    const DecodeArgs& a) {
   switch (gt) {
-    case 1: attention_decode_kernel<LPK, 1, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 2: attention_decode_kernel<LPK, 2, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
-    case 4: attention_decode_kernel<LPK, 4, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
-    default: attention_decode_kernel<LPK, 8, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a); break;
+    case 1: attention_decode_kernel<LPK, 1, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a.pos, a.table, a); break;
+    case 2: attention_decode_kernel<LPK, 2, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a.pos, a.table, a); break;
+    case 4: attention_decode_kernel<LPK, 4, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a.pos, a.table, a); break;
+    default: attention_decode_kernel<LPK, 8, RAW, NW, MM><<<grid, NW * WAVE, 0, stream>>>(q, k, v, partial, out, a.pos, a.table, a); break;
   }
 }
 
