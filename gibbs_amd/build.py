@@ -24,11 +24,13 @@ LIB_NAME = "libgibbs_hip.so"
 ARCH = "gfx950"
 # packed-fp32 instructions are kept off for every kernel (the host pass warns that it does
 # not know the feature; that is harmless).
-# A kernel's first 16 dwords of scalar arguments arrive in registers with the wave (gfx950 preloads them) instead
-# of by a load that everything else in the kernel waits for; arguments passed as a struct are not preloaded.
 HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fvisibility=hidden",
-               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result",
-               "-mllvm", "-amdgpu-kernarg-preload-count=16"]
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
+# In these files a kernel's first dwords of scalar arguments arrive in registers with the wave (gfx950 preloads
+# them) instead of by a load that everything else in the kernel waits for; arguments passed as a struct are not
+# preloaded.  It pays for the kernels of a decode step, which are short and many.
+PRELOAD_FLAGS = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
+PRELOAD_FILES = {"gemm_skinny_fused.hip", "attention_decode.hip", "attention_decode_fused.hip"}
 
 
 HOST_SRC = os.path.join(CSRC, "host")
@@ -54,7 +56,7 @@ def _stamp() -> str:
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + PRELOAD_FLAGS + sorted(PRELOAD_FILES)).encode())
     return h.hexdigest()
 
 
@@ -93,7 +95,8 @@ def _writable(path: str) -> bool:
 
 def _compile_one(cc: str, src: str, obj: str, env: dict) -> tuple[str, float]:
     t0 = time.time()
-    proc = subprocess.run([cc, *HIPCC_FLAGS, "-c", src, "-o", obj], capture_output=True, text=True, env=env)
+    flags = HIPCC_FLAGS + (PRELOAD_FLAGS if os.path.basename(src) in PRELOAD_FILES else [])
+    proc = subprocess.run([cc, *flags, "-c", src, "-o", obj], capture_output=True, text=True, env=env)
     if proc.returncode != 0:
         raise BuildError(f"hipcc failed on {os.path.basename(src)}:\n{proc.stderr[-4000:]}")
     return os.path.basename(src), time.time() - t0
