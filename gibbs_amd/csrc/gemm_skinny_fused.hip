@@ -92,10 +92,11 @@ struct FusedArgs {
 // and runs its epilogue.
 template <int NT, int RG, int ROWS, int FT, int WAVES, bool RMS, int EPI, int KC, bool STAGE, bool BP = false>
 __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const bf16* W, const bf16* X, int N, int O, int I, int packed,
-                                                                         int ktiles, int rotate, long group_tiles, long ldw,
-                                                                         long ldx, FusedArgs rest) {
-  // What the first loads need comes as 16 dwords of scalar arguments, which arrive in registers with the wave;
-  // the rest of the arguments is a struct, which the kernel loads as it needs it.
+                                                                         int ktiles, int rotate, long group_tiles, long ldx,
+                                                                         long ldw, FusedArgs rest) {
+  // What the first loads need comes as scalar arguments, the first 14 dwords of which arrive in registers with
+  // the wave (all but ldw, the row stride of a matrix that is not in tile order); the rest of the arguments is a
+  // struct, which the kernel loads as it needs it.
   FusedArgs a = rest;
   a.W = W; a.X = X; a.N = N; a.O = O; a.I = I; a.packed = packed; a.ktiles = ktiles; a.rotate = rotate;
   a.group_tiles = group_tiles; a.ldw = ldw; a.ldx = ldx;
@@ -532,7 +533,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
   }
 }
 
-#define FUSED_KERNEL_ARGS(a) (a).W, (a).X, (a).N, (a).O, (a).I, (a).packed, (a).ktiles, (a).rotate, (a).group_tiles, (a).ldw, (a).ldx, (a)
+#define FUSED_KERNEL_ARGS(a) (a).W, (a).X, (a).N, (a).O, (a).I, (a).packed, (a).ktiles, (a).rotate, (a).group_tiles, (a).ldx, (a).ldw, (a)
 
 template <int NT, bool ST, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
