@@ -30,7 +30,7 @@ HIPCC_FLAGS = ["-O3", f"--offload-arch={ARCH}", "-fPIC", "-std=c++17", "-fvisibi
 # them) instead of by a load that everything else in the kernel waits for; arguments passed as a struct are not
 # preloaded.  It pays for the kernels of a decode step, which are short and many.
 PRELOAD_FLAGS = ["-mllvm", "-amdgpu-kernarg-preload-count=16"]
-PRELOAD_FILES = {"gemm_skinny_fused.hip", "attention_decode.hip", "attention_decode_fused.hip"}
+PRELOAD_FILES = {"gemm_skinny_fused.hip", "gemm_skinny_fused_rows.hip", "attention_decode.hip", "attention_decode_fused.hip"}
 
 
 HOST_SRC = os.path.join(CSRC, "host")
