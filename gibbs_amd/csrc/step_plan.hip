@@ -197,7 +197,7 @@ void decode_splits(int n_rows, int nkv, int group, int max_seq, int hd, int page
     return;
   }
   const long want = ceil_div_l(512, per_split);
-  *n_splits = (int)std::max<long>(least, std::min<long>(std::min<long>(want, max_seq / (matrix ? 128 : 64)), 256));
+  *n_splits = (int)std::max<long>(least, std::min<long>(std::min<long>(want, max_seq / (matrix ? 256 : 64)), 256));
   *waves = 4;
 }
 

@@ -534,7 +534,7 @@ def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, 
     if per_split >= 256:
         return least, (4 if matrix else 8)
     want = -(-512 // per_split)
-    return max(least, min(want, max_seq // (128 if matrix else 64), 256)), 4
+    return max(least, min(want, max_seq // (256 if matrix else 64), 256)), 4
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
