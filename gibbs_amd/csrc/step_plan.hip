@@ -184,7 +184,7 @@ int skinny_splits(int n_out, int inner, int want_blocks = 512, int features = 16
 constexpr int MATRIX_SLICE_PAGES = 510;   // page ids of a key slice that the decode attention's matrix-core walk keeps in LDS
 
 // (key slices per (row, kv head), waves per workgroup) of the decode attention: few rows get enough
-// slices to give every compute unit two workgroups, but at least 128 keys to a slice on the matrix cores
+// slices to give every compute unit two workgroups, but at least 256 keys to a slice on the matrix cores
 // (64 on the vector units); rows and heads that fill the chip by themselves get none.
 void decode_splits(int n_rows, int nkv, int group, int max_seq, int hd, int page_size, int* n_splits, int* waves) {
   const bool matrix = hd > 0 && hd % 16 == 0 && hd <= 128;

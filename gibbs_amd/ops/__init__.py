@@ -522,7 +522,8 @@ def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, 
                   page_size: int = 16) -> tuple:
     """(key slices per (row, kv head), waves per workgroup) for the decode attention.  Few rows:
     enough slices to give each of the 256 compute units two workgroups of 4 waves, but at least 64
-    keys to a slice (128 on the matrix cores: a tile of 32 for every wave).  Rows and heads that fill
+    keys to a slice (256 on the matrix cores: two tiles of 32 for every wave, and few enough slices for the merge
+    to take them at once).  Rows and heads that fill
     the chip by themselves: no slices (a slice costs every wave its own prologue and final fold), 8
     waves on the vector units, 4 on the matrix cores (measured at batch 1 to 64, 2,048 to 8,192 keys).
     The matrix-core walk keeps the page ids of a whole slice in LDS: caches longer than that are cut
