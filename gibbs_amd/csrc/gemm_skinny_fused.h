@@ -515,7 +515,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
 template <bool TILED, int NT, bool ST, int RG, bool RMS, int EPI, int KC>
 void launch_rows(const FusedArgs& a, hipStream_t s) {
   constexpr int tiles2_from = 192;   // pairs of tiles from which a workgroup takes two (measured at 33 to 64 rows)
-  if constexpr (NT >= 3 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
+  if constexpr (NT >= 2 && (EPI == EPI_STORE || EPI == EPI_GLU)) {
     // many rows of X: two tiles of 16 features per workgroup where that still leaves enough workgroups
     // (also where single tiles would need a second round of workgroups that pairs do not: 257 to 383 tiles)
     if (a.O / 32 >= tiles2_from || (ceil_div(a.O, 16) > 256 && a.O / 32 >= 128)) {
