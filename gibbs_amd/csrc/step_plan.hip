@@ -478,7 +478,7 @@ struct Exec {
         RUN(gibbs_gemm_f32((const float*)h, (const float*)p.head.w, a.logits, M, V, H, H, H, V, a.stream));
       } else if (H % 8 || ((uintptr_t)h % 16) || ((uintptr_t)p.head.w % 16)) {
         RUN(gibbs_gemm_bf16_plain(h, p.head.w, a.logits, GIBBS_F32, M, V, H, H, H, V, a.stream));
-      } else if (M <= 32) {
+      } else if (M <= 48) {   // (see ops/linear.py)
         RUN(gibbs_gemm_skinny(h, p.head.packed ? p.head.packed : p.head.w, a.logits, GIBBS_F32, M, V, H, H,
                               p.head.packed ? 0 : H, V, 1, a.stream));
       } else {

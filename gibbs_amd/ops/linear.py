@@ -21,6 +21,8 @@ from .lib import KernelError, require_cuda
 # rows up to which the weight-streaming kernels are used (they re-read the activations once per 16
 # output features, which stops paying beyond one or two MFMA tiles of rows)
 SKINNY_ROWS = 32
+# float32 logits: the few-row kernel streams the head matrix faster than the tiled product up to here
+SKINNY_ROWS_F32_OUT = 48
 USE_LIBRARY_GEMM = os.environ.get("GIBBS_GEMM", "library") != "own"
 # the library product is hipBLASLt called directly (its heuristic's choice kept per shape: a call costs
 # the host 12 us instead of the 20 us of torch.matmul); "torch" goes through PyTorch
@@ -45,7 +47,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out_dtype: Optional[torch.dtype] = 
         n, i = x.shape
         if i % 8 or w.stride(0) % 8 or (n > 1 and x.stride(0) % 8) or x.data_ptr() % 16 or w.data_ptr() % 16:
             return gemm_bf16_plain(x, w, out_dtype)             # what the matrix-core kernels refuse
-        if 1 <= x.shape[0] <= SKINNY_ROWS:
+        if 1 <= x.shape[0] <= (SKINNY_ROWS_F32_OUT if out_dtype == torch.float32 and not partial_ok else SKINNY_ROWS):
             splits = skinny_splits(w.shape[0], w.shape[1]) if partial_ok else 1
             return gemm_skinny(x, w if packed is None else packed, out_dtype, splits)
         if USE_LIBRARY_GEMM and out_dtype == torch.bfloat16:
