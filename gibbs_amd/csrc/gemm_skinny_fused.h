@@ -545,10 +545,10 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
 
 template <bool TILED, int RG, bool RMS, int EPI, int KC = 0>
 void launch_nt(const FusedArgs& a, hipStream_t s) {
-  // Up to 8 rows of X come straight into paired B operands, 12 and more through LDS.  Between them neither is
-  // clearly better (measured at 9, 12 and 16 rows: staged products are 8 to 16 % faster at 16 rows, the same at
-  // 12, and up to 13 % slower at 9 for the widest matrices).
-  constexpr int stage_from = 12;
+  // Up to 8 rows of X come straight into paired B operands, 13 and more through LDS.  Between them neither is
+  // clearly better (staged products are 8 to 16 % faster at 16 rows and up to 13 % slower at 9 for the widest
+  // matrices; a whole step is 2 % slower staged at 9 rows, 0.4 % slower at 12 and 1 % faster at 13).
+  constexpr int stage_from = 13;
   const int nt = ceil_div(a.N, 16);
   if (nt == 1 && a.N < stage_from) launch_rows<TILED, 1, false, RG, RMS, EPI, KC>(a, s);
   else if (nt == 1) launch_rows<TILED, 1, true, RG, RMS, EPI, KC>(a, s);
