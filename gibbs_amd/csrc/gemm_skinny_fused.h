@@ -82,9 +82,9 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
   // more of a row per request instead of the 64 that a lane group of an MFMA operand covers (the memory
   // pipe of a compute unit is bound by requests in flight, and from 8 rows on X is as many requests as W
   // for a workgroup of 8 features).  The wave's region is its own: no barrier.
-  static_assert(STAGE || NT == 1, "more than 16 rows of X are staged");
+  static_assert(STAGE || NT == 1 || BP, "more than 16 rows of X are staged");
   // MFMA steps per iteration (8 features and one tile of rows: an A operand serves two steps, so 8 steps are 4 loads a row group)
-  constexpr int U = (ROWS == 8 && NT == 1) ? 8 : (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);
+  constexpr int U = (ROWS == 8 && (NT == 1 || BP)) ? 8 : (FT * RG * NT >= 6) ? 2 : (FT * RG * NT == 1 ? 8 : 4);
   constexpr int CH = 4 * U;                    // 16-byte chunks of a row per iteration
   constexpr int RED_BYTES = WAVES * FT * RG * NT * WAVE * 16;
   constexpr int STAGE_BYTES = STAGE ? WAVES * NT * 16 * CH * 16 : 0;
@@ -99,13 +99,15 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
   constexpr bool PAIR = ROWS == 8;
   constexpr int KU = PAIR ? 64 : 32;
   static_assert(!PAIR || FT == 1, "8 features: one tile per workgroup");
-  // BP (8 features and at most 8 rows of X): the B operands are pairs as well, rows 8..15 holding the same 8 rows
-  // of X at the next 32 values of k.  One MFMA then does two steps: the upper left 8 x 8 block of its result is
-  // the product at k, the lower right one the product at k + 32 (the other two blocks mix the two and are
-  // dropped).  A load of X is 8 requests of 128 bytes instead of two loads of 8 requests of 64.
+  // BP (at most 16 rows of X, not staged): the B operands are pairs as well, rows 8..15 holding the same 8 rows
+  // of X at the next 32 values of k, and a tile of rows is 8 rows of X (NT of them).  One MFMA then does two
+  // steps: the upper left 8 x 8 block of its result is the product at k, the lower right one the product at
+  // k + 32 (the other two blocks mix the two and are dropped).  A load of X is 8 requests of 128 bytes instead
+  // of two loads of 8 requests of 64.
   // With 16 features the A operands are single steps: the step at k takes the pair as it is (columns 0..7 of the
   // result are the rows of X), the step at k + 32 takes it with the halves of every 16 lanes exchanged.
-  static_assert(!BP || (NT == 1 && !STAGE && FT == 1), "paired B operands: one tile of rows and of features, not staged");
+  static_assert(!BP || (NT <= 2 && !STAGE && FT == 1), "paired B operands: two tiles of 8 rows at most, one of features, not staged");
+  constexpr int TILE_ROWS = BP ? 8 : 16;   // rows of X in a tile of rows
   const int steps = (a.I + KU - 1) / KU;
   const int per_wave = (steps + WAVES - 1) / WAVES;
   const int k_begin = wave * per_wave * KU;
@@ -156,8 +158,9 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
   bool x_ok[NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    x_ok[t] = BP ? r8 < a.N : t * 16 + r < a.N;
-    xrow[t] = a.X + (size_t)(x_ok[t] ? (BP ? r8 : t * 16 + r) : 0) * a.ldx + (BP ? half * 32 : 0) + g * 8;
+    const int n = BP ? t * 8 + r8 : t * 16 + r;
+    x_ok[t] = n < a.N;
+    xrow[t] = a.X + (size_t)(x_ok[t] ? n : 0) * a.ldx + (BP ? half * 32 : 0) + g * 8;
   }
   // What the epilogue reads besides the product is asked for behind the first loads of the operands: the
   // product hides the latency (the state row hangs on a slot index, two dependent loads, and wave 0 would
@@ -167,8 +170,8 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
   constexpr int KH = KC > 1 ? KC - 1 : 1;
   const int f_epi = wave / NT, t_epi = wave % NT;
   const int o_epi = o0 + f_epi * ROWS + g * 4;
-  const int n_epi = t_epi * 16 + r;
-  const bool epi_lane = wave < FT * NT && g * 4 < ROWS && o_epi < a.O && n_epi < a.N;
+  const int n_epi = t_epi * TILE_ROWS + r;
+  const bool epi_lane = wave < FT * NT && g * 4 < ROWS && r < TILE_ROWS && o_epi < a.O && n_epi < a.N;
   float pre_x[4];          // RESIDUAL: the stream; CONV: unused
   float pre_hist[KH][4];   // CONV: the state rows
   float pre_taps[KC > 1 ? KC : 1][4], pre_bias[4];
@@ -271,20 +274,31 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
     if constexpr (BP) {
 #pragma unroll
       for (int u = 0; u < UB; ++u) {
-        bf16x8 b = bv[u][0];
-        if (ragged && !(k + u * 64 + xoff < k_end)) b = zero;
-        if (RMS) gram[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b, b, gram[0], 0, 0, 0);
+        bf16x8 b[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+          b[t] = bv[u][t];
+          if (ragged && !(k + u * 64 + xoff < k_end)) b[t] = zero;
+          if (RMS) gram[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[t], b[t], gram[t], 0, 0, 0);
+        }
         if constexpr (PAIR) {
 #pragma unroll
-          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][0][q], b, acc[0][q][0], 0, 0, 0);
+          for (int t = 0; t < NT; ++t)
+#pragma unroll
+            for (int q = 0; q < RG; ++q) acc[0][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[u][0][q], b[t], acc[0][q][t], 0, 0, 0);
           if (more) load_a(k_next, u);
         } else {
 #pragma unroll
-          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u][0][q], b, acc[0][q][0], 0, 0, 0);
-          if (more) load_a(k_next, 2 * u);
-          const bf16x8 b2 = swap_halves16(b);
+          for (int t = 0; t < NT; ++t)
 #pragma unroll
-          for (int q = 0; q < RG; ++q) acc[0][q][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u + 1][0][q], b2, acc[0][q][0], 0, 0, 0);
+            for (int q = 0; q < RG; ++q) acc[0][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u][0][q], b[t], acc[0][q][t], 0, 0, 0);
+          if (more) load_a(k_next, 2 * u);
+#pragma unroll
+          for (int t = 0; t < NT; ++t) {
+            const bf16x8 b2 = swap_halves16(b[t]);
+#pragma unroll
+            for (int q = 0; q < RG; ++q) acc[0][q][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[2 * u + 1][0][q], b2, acc[0][q][t], 0, 0, 0);
+          }
           if (more) load_a(k_next, 2 * u + 1);
         }
         if (more) load_b(k_next, u);
@@ -401,7 +415,7 @@ __global__ __launch_bounds__(WAVES * WAVE) void gemm_skinny_fused_kernel(const b
     const int t = t_epi;
     const int n = n_epi;
     const int o = o_epi;
-    if (n >= a.N || g * 4 >= ROWS || o >= a.O) return;
+    if (n >= a.N || r >= TILE_ROWS || g * 4 >= ROWS || o >= a.O) return;
     float scale = 1.f;
     if (RMS) {
       float tot = 0.f;
@@ -525,32 +539,34 @@ void launch_rows(const FusedArgs& a, hipStream_t s) {
   }
   // few features: halve the rows per workgroup so that every compute unit gets one
   if ((NT <= 2 || EPI == EPI_CONV) && pair_layout(a.O)) {
-    if constexpr (NT == 1 && !ST) {
-      if (a.N <= 8) {   // the rows of X fit half a tile: paired B operands
-        gemm_skinny_fused_kernel<TILED, NT, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
-        return;
-      }
+    if constexpr (NT == 1 && !ST) {   // paired B operands: one tile of 8 rows of X, or two
+      if (a.N <= 8) gemm_skinny_fused_kernel<TILED, 1, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
+      else gemm_skinny_fused_kernel<TILED, 2, RG, 8, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
+    } else {
+      gemm_skinny_fused_kernel<TILED, NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
     }
-    gemm_skinny_fused_kernel<TILED, NT, RG, 8, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 8), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
   } else {
     if constexpr (NT == 1 && !ST) {
-      if (a.N <= 8) {
-        gemm_skinny_fused_kernel<TILED, NT, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
-        return;
-      }
+      if (a.N <= 8) gemm_skinny_fused_kernel<TILED, 1, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
+      else gemm_skinny_fused_kernel<TILED, 2, RG, 16, 1, 8, RMS, EPI, KC, ST, true><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
+    } else {
+      gemm_skinny_fused_kernel<TILED, NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
     }
-    gemm_skinny_fused_kernel<TILED, NT, RG, 16, 1, 8, RMS, EPI, KC, ST><<<ceil_div(a.O, 16), 8 * WAVE, 0, s>>>(FUSED_KERNEL_ARGS(a));
   }
 }
 
 template <bool TILED, int RG, bool RMS, int EPI, int KC = 0>
 void launch_nt(const FusedArgs& a, hipStream_t s) {
-  // Up to 8 rows of X come straight into paired B operands, 13 and more through LDS.  Between them neither is
-  // clearly better (staged products are 8 to 16 % faster at 16 rows and up to 13 % slower at 9 for the widest
-  // matrices; a whole step is 2 % slower staged at 9 rows, 0.4 % slower at 12 and 1 % faster at 13).
-  constexpr int stage_from = 13;
+  // Up to 16 rows of X come straight into paired B operands, except 9 to 16 rows where the product has no more
+  // workgroups than the chip has compute units: those come through LDS.  Measured over whole decode steps of
+  // three model shapes (hidden sizes 1024, 2048 and 2048 with wider feed-forwards): products of up to 2048
+  // features (256 workgroups of 8) are 1 to 5 % of a step faster staged from 9 rows on and slower staged at 8
+  // and below; products of 3072 features and more are faster unstaged through 16 rows (2 to 3 % of a step at 13
+  // to 16 rows, the gate and up products most of all).
+  constexpr int one_round = 256;   // workgroups of 8 features that get a compute unit each
+  const bool staged = a.N > 8 && ceil_div(a.O, 8) <= one_round;
   const int nt = ceil_div(a.N, 16);
-  if (nt == 1 && a.N < stage_from) launch_rows<TILED, 1, false, RG, RMS, EPI, KC>(a, s);
+  if (nt == 1 && !staged) launch_rows<TILED, 1, false, RG, RMS, EPI, KC>(a, s);
   else if (nt == 1) launch_rows<TILED, 1, true, RG, RMS, EPI, KC>(a, s);
   else if (nt == 2) launch_rows<TILED, 2, true, RG, RMS, EPI, KC>(a, s);
   else if (nt == 3) launch_rows<TILED, 3, true, RG, RMS, EPI, KC>(a, s);

@@ -590,7 +590,8 @@ def rms_scale(x, eps):
 @pytest.mark.parametrize("n,o,i", [(1, 64, 128), (8, 3072, 2048), (16, 331 * 8, 1000), (17, 200, 512), (64, 96, 4096), (5, 40, 72),
                                    (48, 8200, 512), (64, 3072, 2048),      # two tiles a workgroup; many rows, one tile
                                    (3, 20, 104), (8, 1001, 1000), (7, 4100, 104), (8, 4099, 2048), (9, 4100, 72),
-                                   (12, 36, 200)])                          # paired operands with ragged ends, both layouts
+                                   (12, 36, 200),                           # paired operands with ragged ends, both layouts
+                                   (13, 2100, 264), (10, 40, 520)])         # 9 to 16 rows: two tiles of 8 rows in pairs; few features: staged
 def test_skinny_store_with_rms_prologue(n, o, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=3.0), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -603,7 +604,8 @@ def test_skinny_store_with_rms_prologue(n, o, i):
 
 @pytest.mark.parametrize("n,o,i", [(1, 2048, 2048), (8, 2048, 8192), (33, 200, 512), (64, 72, 96), (64, 2048, 2048),
                                    (40, 1000, 4096),                        # many rows: partial sums over k, then the add
-                                   (7, 36, 200), (8, 4100, 136), (2, 12, 8)])
+                                   (7, 36, 200), (8, 4100, 136), (2, 12, 8),
+                                   (12, 2056, 200), (15, 4100, 136), (10, 36, 200)])   # 9 to 16 rows: pairs (8 and 16 features), staged
 def test_skinny_residual(n, o, i):
     from gibbs_amd import ops
     y, w = rnd(n, i, dtype=torch.bfloat16), rnd(o, i, dtype=torch.bfloat16, seed=1)
@@ -620,7 +622,7 @@ def test_skinny_residual(n, o, i):
 
 @pytest.mark.parametrize("n,f,i", [(1, 8192, 2048), (8, 200, 512), (40, 128, 72), (64, 256, 1024), (64, 6200, 256),
                                    (36, 8192, 2048),                        # two tiles a workgroup
-                                   (5, 4100, 104), (8, 52, 40), (11, 4090, 72)])
+                                   (5, 4100, 104), (8, 52, 40), (11, 4090, 72), (14, 2200, 104), (9, 60, 136)])
 def test_skinny_glu(n, f, i):
     from gibbs_amd import ops
     x, w = rnd(n, i, dtype=torch.bfloat16, scale=2.0), rnd(2 * f, i, dtype=torch.bfloat16, scale=0.05, seed=1)
@@ -633,7 +635,8 @@ def test_skinny_glu(n, f, i):
         ops.skinny_glu(x, ops.PackedWeight(w), rms_eps=1e-6)
 
 
-@pytest.mark.parametrize("n,c,i,k,bias", [(1, 2048, 2048, 3, False), (8, 72, 96, 4, True), (20, 40, 64, 2, True), (64, 96, 128, 3, False)])
+@pytest.mark.parametrize("n,c,i,k,bias", [(1, 2048, 2048, 3, False), (8, 72, 96, 4, True), (20, 40, 64, 2, True), (64, 96, 128, 3, False),
+                                          (13, 2056, 96, 3, True), (16, 2104, 64, 4, False), (11, 40, 64, 2, True)])   # 9 to 16 rows
 def test_skinny_conv(n, c, i, k, bias):
     """In-projection + convolution of decoded tokens against the unfused kernels and the reference."""
     from gibbs_amd import ops
