@@ -69,16 +69,25 @@ struct PrefillArgs {
 
 // DT: head size = 16 * DT.  POW2: the page size is a power of two (shifts instead of divisions: an
 // integer division costs dozens of instructions, several times per thread and tile).
+// Five waves a SIMD are asked for: the walk over the keys is a chain of short waits (two barriers a tile, LDS, the
+// next tile's loads) that other waves have to fill; head sizes up to 64 fit the 96 registers that leaves without
+// spilling (at 8,192 rows 10 % faster than with four waves; six waves spill and are no faster), larger heads
+// cannot follow the hint and keep the registers they need.
 template <int DT, bool POW2>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __restrict__ q,
+__global__ __launch_bounds__(256, 5) void attention_prefill_kernel(const bf16* __restrict__ q,
                                                                 const bf16* __restrict__ kpages,
                                                                 const bf16* __restrict__ vpages, bf16* __restrict__ out,
                                                                 float* __restrict__ partial, PrefillArgs a) {
   constexpr int HD = 16 * DT;
   constexpr int DS = (DT + 1) / 2;  // steps of 32 over d
+  // Rows of the tiles in LDS are padded against bank conflicts, K and V differently: a read of K operands has 16
+  // lanes on 16 rows with 16 bytes each (row stride of 4 banks modulo 8), a transposing read of V has 32 lanes on
+  // 8 rows with 32 bytes each (row stride of 8 banks modulo 16: with the stride of K the eighth row wraps onto
+  // the first one's banks, and the read takes two turns).
   constexpr int LDK = HD + 8;
+  constexpr int LDV = HD % 32 == 16 ? HD + 32 : HD + 16;
   __shared__ bf16 sK[BN][LDK];
-  __shared__ bf16 sV[BN][LDK];
+  __shared__ __attribute__((aligned(16))) bf16 sV[BN][LDV];
   __shared__ int s_pages[SEG_PAGES];
 
   // which request and which 64 rows of it
@@ -142,6 +151,11 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
   // matrix cores work on the current tile, and go to LDS once everyone is done with it.
   constexpr int KCH = (BN * (HD / 8) + 255) / 256;        // 16-byte chunks of K (and of V) per thread and tile
   uint4 kreg[KCH], vreg[KCH];
+  // (a key's and its value's chunk lie at the same offset of their pools; with a page size that is a power of two
+  // the offset is a page's stride times the page id plus a few shifts: an address costs a handful of instructions,
+  // and the walk over the keys is bound by the vector instructions it issues)
+  const size_t page_stride = (size_t)a.nkv * a.page_size * HD;
+  const unsigned head_off = (unsigned)kvh * a.page_size * HD;
   auto load_tile = [&](int key0) {
 #pragma unroll
     for (int i = 0; i < KCH; ++i) {
@@ -149,8 +163,16 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
       const int key = c / (HD / 8), d = (c % (HD / 8)) * 8;
       kreg[i] = vreg[i] = make_uint4(0, 0, 0, 0);
       if (c < BN * (HD / 8) && key0 + key <= last_pos) {
-        kreg[i] = *(const uint4*)(page_row(kpages, key0 + key) + d);
-        vreg[i] = *(const uint4*)(page_row(vpages, key0 + key) + d);
+        if constexpr (POW2) {
+          const int ak = key0 + key;
+          const unsigned page = (unsigned)s_pages[(ak >> a.page_shift) - seg_first_page];
+          const size_t off = page * page_stride + (head_off + (unsigned)(ak & (a.page_size - 1)) * HD + d);
+          kreg[i] = *(const uint4*)(kpages + off);
+          vreg[i] = *(const uint4*)(vpages + off);
+        } else {
+          kreg[i] = *(const uint4*)(page_row(kpages, key0 + key) + d);
+          vreg[i] = *(const uint4*)(page_row(vpages, key0 + key) + d);
+        }
       }
     }
   };
@@ -247,10 +269,13 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(const bf16* __re
         l += p;
         pf[c / 2][(c % 2) * 4 + i] = (bf16)p;
       }
+    // (most tiles leave every row's maximum as it was: a factor of exactly 1, and nothing to do)
+    if (__builtin_amdgcn_ballot_w64(keep != 1.f) != 0) {
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+      for (int t = 0; t < DT; ++t)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[t][i] *= keep;
+        for (int i = 0; i < 4; ++i) o[t][i] *= keep;
+    }
     // O^T += V^T P^T: k runs over the 64 keys in 2 steps of 32
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
