@@ -71,10 +71,10 @@ struct PrefillArgs {
 // integer division costs dozens of instructions, several times per thread and tile).
 // Five waves a SIMD are asked for: the walk over the keys is a chain of short waits (two barriers a tile, LDS, the
 // next tile's loads) that other waves have to fill; head sizes up to 64 fit the 96 registers that leaves without
-// spilling (at 8,192 rows 10 % faster than with four waves; six waves spill and are no faster), larger heads
-// cannot follow the hint and keep the registers they need.
+// spilling (at 8,192 rows 10 % faster than with four waves; six waves spill and are no faster).  Larger heads are
+// left to the compiler: asked for five waves, head sizes 80 and 96 spill.
 template <int DT, bool POW2>
-__global__ __launch_bounds__(256, 5) void attention_prefill_kernel(const bf16* __restrict__ q,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(DT <= 4 ? 5 : 1))) void attention_prefill_kernel(const bf16* __restrict__ q,
                                                                 const bf16* __restrict__ kpages,
                                                                 const bf16* __restrict__ vpages, bf16* __restrict__ out,
                                                                 float* __restrict__ partial, PrefillArgs a) {
