@@ -307,11 +307,12 @@ def decode_batch_steps(seqs, prompt_len, ends_early):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,live", [("W", 7), ("M", 9), ("W", 12), ("M", 17), ("W", 33), ("M", 48), ("W", 64)])
+@pytest.mark.parametrize("name,live", [("W", 7), ("M", 9), ("W", 12), ("W", 16), ("M", 17), ("W", 20), ("W", 33), ("M", 48), ("W", 64)])
 def test_many_requests_decoding_side_by_side(tmp_path_factory, name, live, dtype):
     """7 to 64 live requests that decode together (in bfloat16 the fused decode kernels: up to 8 rows in
-    paired operands, 9 to 11 straight into the operands, from 12 on staged through LDS, from 33 on with
-    two tiles of features per workgroup and the down projection cut along k), with
+    paired operands; 9 to 16 rows in two tiles of 8 paired rows for products of more than 2,048 features (W's
+    feed-forward and head) and staged through LDS for the others; from 17 on staged, with the loads of rows beyond
+    the batch left out, from 33 on with two tiles of features per workgroup and the down projection cut along k), with
     prompts of different lengths so that sequences cross page edges at different steps, one request
     ending mid-way: every decoded place against the plain implementation, and the bfloat16 fused
     path against the same engine on its general path without folded gains."""
