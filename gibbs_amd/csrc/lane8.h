@@ -83,18 +83,20 @@ __device__ __forceinline__ Rot8 rotation8(int e0, const float* inv_freq, int rot
 
 // Norm (optional) and rotation of one head held 8 elements per lane by LPK neighbouring lanes.
 // `v` are this lane's elements e0 .. e0+7 of the head; returns them normed and rotated.
+// `gain8`: the norm's gain for this lane's elements, already in registers (a caller that norms several heads
+// reads it once); `normed` false: no norm.
 template <int LPK>
-__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
-                                           const Rot8& rt, int rot, int variant, int lane) {
+__device__ __forceinline__ void norm_rope8_with(float* v, int e0, int hd, bool normed, const float* gain8, float eps,
+                                                bool rotate, const Rot8& rt, int rot, int variant, int lane) {
   const bool active = e0 < hd;
-  if (gain) {
+  if (normed) {
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < EPL; ++i) ss += v[i] * v[i];
     ss = group_sum<LPK>(ss);
     const float sc = 1.0f / sqrtf(ss / (float)hd + eps);
 #pragma unroll
-    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain[e0 + i] : 0.f;
+    for (int i = 0; i < EPL; ++i) v[i] = active ? v[i] * sc * gain8[i] : 0.f;
   }
   if (!rotate) return;
   const int half = rot / 2;
@@ -121,4 +123,14 @@ __device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float
     const float other = __shfl(v[i], src, WAVE);
     if (e0 + i < rot) v[i] = low ? v[i] * rt.c[i] - other * rt.s[i] : other * rt.s[i] + v[i] * rt.c[i];
   }
+}
+
+// The same with the gain read here (null: no norm).
+template <int LPK>
+__device__ __forceinline__ void norm_rope8(float* v, int e0, int hd, const float* gain, float eps, bool rotate,
+                                           const Rot8& rt, int rot, int variant, int lane) {
+  float gain8[EPL];
+#pragma unroll
+  for (int i = 0; i < EPL; ++i) gain8[i] = (gain && e0 < hd) ? gain[e0 + i] : 1.f;
+  norm_rope8_with<LPK>(v, e0, hd, gain != nullptr, gain8, eps, rotate, rt, rot, variant, lane);
 }
