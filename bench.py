@@ -184,6 +184,30 @@ def suite_rows(path: str) -> list:
 
 
 PARITY_PROMPT, PARITY_DECODE = 64, 8
+# bfloat16 against the 32-bit path at these layer sizes: the largest difference of a logit measured is
+# 0.9 % of the largest logit (3 layers); a place whose best logit leads by more than twice the bound
+# must keep its choice
+PARITY_BF16_MAX_ERR = 0.02
+
+
+def greedy_through_loop(engine, prompt, n: int) -> list:
+    """`n` greedy tokens after `prompt` through the captured decode loop (the path that the speed
+    figures time: the rows' embeddings written by the end of the step before, argmax on the device)."""
+    from gibbs_amd.engine.decode import DecodeLoop
+    first = int(engine.step([("g", prompt, [len(prompt) - 1])]).argmax(-1).item())
+    loop = DecodeLoop(engine, ["g"], [first])
+    loop.run(n - 1)
+    out = [first] + loop.tokens()[0]
+    engine.release("g")
+    return out
+
+
+def greedy_through_steps(engine, prompt, n: int) -> list:
+    out = [int(engine.step([("s", prompt, [len(prompt) - 1])]).argmax(-1).item())]
+    for _ in range(n - 1):
+        out.append(int(engine.step([("s", [out[-1]], [0])]).argmax(-1).item()))
+    engine.release("s")
+    return out
 
 
 def parity(layers: int = 3) -> dict:
@@ -192,7 +216,11 @@ def parity(layers: int = 3) -> dict:
     an attention and a convolution layer): a model folder with random weights is written, 64 prompt
     tokens run as one step and 8 given tokens one by one; the logits of those 9 places from the
     32-bit path are held against the plain implementation's (at most 1e-5 of the scale, same
-    argmax), and the bfloat16 path's against the 32-bit path's (cosine >= 0.999)."""
+    argmax), and the bfloat16 path's against the 32-bit path's (cosine >= 0.999, no logit further off
+    than `PARITY_BF16_MAX_ERR` of the scale, the same argmax wherever the 32-bit lead is more than
+    twice that).  Then 8 greedy tokens through the captured decode loop, the path that is timed: in
+    32-bit they are the plain implementation's, in bfloat16 those of the same engine stepped from
+    the host."""
     import tempfile
 
     import numpy as np
@@ -205,28 +233,45 @@ def parity(layers: int = 3) -> dict:
     shape = dict(SHAPE, num_hidden_layers=layers, full_attn_idxs=[1])
     cfg = config_from_dict(shape)
     ids = seeded_prompt(77, PARITY_PROMPT + PARITY_DECODE, cfg.vocab_size)
+    prompt = ids[:PARITY_PROMPT]
     with tempfile.TemporaryDirectory() as tmp:
         write_random_model(tmp, cfg, DecoderModel(cfg.model_spec()).tensor_decls(), seed=5, gain_std=0.1)
-        got = {}
+        got, loop_tokens, step_tokens = {}, {}, {}
         for dtype in ("float32", "bfloat16"):
-            engine = Engine(tmp, dtype=dtype, max_tokens=256, max_requests=1, ctx=256)
-            rows = [engine.step([("p", ids[:PARITY_PROMPT], [PARITY_PROMPT - 1])])[0]]
+            engine = Engine(tmp, dtype=dtype, max_tokens=512, max_requests=2, ctx=256)
+            rows = [engine.step([("p", prompt, [PARITY_PROMPT - 1])])[0]]
             rows += [engine.step([("p", [t], [0])])[0] for t in ids[PARITY_PROMPT:]]
             got[dtype] = np.stack([r.float().cpu().numpy() for r in rows]).astype(np.float64)
+            engine.release("p")
+            loop_tokens[dtype] = greedy_through_loop(engine, prompt, PARITY_DECODE)
+            step_tokens[dtype] = greedy_through_steps(engine, prompt, PARITY_DECODE)
             del engine
         weights, raw = P.load_model_dir(tmp)
         want = P.forward(weights, raw, ids)[PARITY_PROMPT - 1:]
+        seq, plain_tokens = list(prompt), []
+        for _ in range(PARITY_DECODE):
+            plain_tokens.append(P.argmax_first(P.forward(weights, raw, seq)[-1]))
+            seq.append(plain_tokens[-1])
     f32, b16 = got["float32"], got["bfloat16"]
-    err = float(np.abs(f32 - want).max() / np.abs(want).max())
+    scale = np.abs(want).max()
+    err = float(np.abs(f32 - want).max() / scale)
     cos = (f32 * b16).sum(-1) / np.sqrt((f32 * f32).sum(-1) * (b16 * b16).sum(-1))
     rel = float(np.sqrt(((b16 - f32) ** 2).sum(-1) / (f32 ** 2).sum(-1)).max())
+    b16_err = float(np.abs(b16 - f32).max() / scale)
     same_f32 = int((f32.argmax(-1) == want.argmax(-1)).sum())
-    same_b16 = int((b16.argmax(-1) == f32.argmax(-1)).sum())
+    top2 = np.sort(f32, axis=-1)[:, -2:]
+    decided = (top2[:, 1] - top2[:, 0]) > 2 * PARITY_BF16_MAX_ERR * scale
+    same_b16 = int((b16.argmax(-1) == f32.argmax(-1))[decided].sum())
     n = len(want)
-    ok = err <= 1e-5 and same_f32 == n and float(cos.min()) >= 0.999
+    loop_ok = loop_tokens["float32"] == plain_tokens and loop_tokens["bfloat16"] == step_tokens["bfloat16"]
+    ok = (err <= 1e-5 and same_f32 == n and float(cos.min()) >= 0.999 and b16_err <= PARITY_BF16_MAX_ERR
+          and same_b16 == int(decided.sum()) and loop_ok)
     return {"layers": layers, "places": n, "fp32_vs_plain_max_err_of_scale": float(f"{err:.3e}"),
             "fp32_same_argmax": same_f32, "bf16_vs_fp32_min_cosine": round(float(cos.min()), 6),
-            "bf16_vs_fp32_max_rel_l2": round(rel, 5), "bf16_same_argmax": same_b16, "pass": bool(ok)}
+            "bf16_vs_fp32_max_rel_l2": round(rel, 5), "bf16_vs_fp32_max_err_of_scale": round(b16_err, 5),
+            "bf16_same_argmax": same_b16, "bf16_places_with_a_clear_lead": int(decided.sum()),
+            "fp32_loop_tokens_are_plain": loop_tokens["float32"] == plain_tokens,
+            "bf16_loop_tokens_are_stepped": loop_tokens["bfloat16"] == step_tokens["bfloat16"], "pass": bool(ok)}
 
 
 def main() -> int:
@@ -261,6 +306,7 @@ def main() -> int:
     engine = build_engine(args.dtype, args.layers, max_requests=args.batch if args.no_points else max(64, args.batch),
                           context=context)
 
+    ceiling = R.measured_hbm_bytes_per_s()
     prefill_s = time_prefill(engine)
     prefill_flops = R.prefill_flops(engine, PROMPT_LEN)
     peak = R.PEAK_FLOPS[args.dtype]
@@ -296,13 +342,22 @@ def main() -> int:
         },
         "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / peak, 4)},
+        # `peak` is the published figure; `measured_peak` is what a kernel that only reads reaches on this GPU
+        # (the reference's rows divide by a measured ceiling, src/bench.rs:438-442)
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": R.HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / (R.HBM_BYTES_PER_S / 1e9), 4)},
+                     "frac": round(achieved / (R.HBM_BYTES_PER_S / 1e9), 4), "measured_peak": round(ceiling / 1e9, 1),
+                     "frac_of_measured": round(achieved / (ceiling / 1e9), 4)},
         "points": points, "parity": gate, "top_kernels": top,
     }
     if args.suite:
         del engine
         line["rows"] = suite_rows(args.suite)
+    if gate is not None and not gate["pass"]:
+        # speed of an engine that fails its correctness gate is no measurement: the figures stay in the
+        # line for the reader, under another key, and the run fails
+        line["value_with_failed_parity"], line["value"] = line["value"], None
+        print(json.dumps(line))
+        return 3
     print(json.dumps(line))
     return 0
 

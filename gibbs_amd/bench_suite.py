@@ -137,10 +137,15 @@ def measure(entry: Dict, base: str) -> Dict:
         engine.release(rid)
     tok_s = batch * n_decode / decode_s
     roof = batch * roofline.HBM_BYTES_PER_S / step_bytes
+    measured = roofline.measured_hbm_bytes_per_s()
     return {"model": entry["name"], "batch": batch, "dtype": entry["dtype"],
             "bytes_per_token": int(step_bytes // batch), "ceiling_gbps": roofline.HBM_BYTES_PER_S / 1e9,
             "decode_tok_s": round(tok_s, 1), "roofline_tok_s": round(roof, 1),
-            "roofline_pct": round(100.0 * tok_s / roof, 2), "wall_ms": round(1e3 * decode_s, 3),
+            "roofline_pct": round(100.0 * tok_s / roof, 2),
+            # the same against what a kernel that only reads reaches on this GPU (src/bench.rs:438-442)
+            "measured_ceiling_gbps": round(measured / 1e9, 1),
+            "measured_roofline_pct": round(100.0 * tok_s * step_bytes / batch / measured, 2),
+            "wall_ms": round(1e3 * decode_s, 3),
             "ms_per_step": round(1e3 * decode_s / n_decode, 4),
             # per decode step, as the reference's rows have them (src/bench.rs:92-106): the time between the
             # first and the last of the run's launches on the device, what is left of the wall time, and

@@ -63,3 +63,7 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   for (int i = 0; i < n_waves; ++i) total += scratch[i];
   return total;
 }
+
+// Every file of the library sees the entry points' prototypes, so that a definition whose signature has
+// drifted from what the native step (step_plan.hip) calls does not compile.
+#include "kernels.h"

@@ -71,8 +71,11 @@ class DecodeLoop:
         engine, b = self.engine, self.n
         cm, dev = engine.cache, engine.device
         self.greedy = params is None or all(p.greedy for p in params)
-        # a request holds at most the pages of the context limit, and never more than its group's pool has
-        self.width = [min(cm.pages_for(engine.ctx_limit), cm.pools[g].num_pages) for g in range(cm.n_groups)]
+        # A block table has one entry per logical page (entries of pages that a window has passed stay, as
+        # NO_PAGE), so its width follows the context limit; only a group without a window can never name
+        # more logical pages than its pool has.
+        self.width = [cm.pages_for(engine.ctx_limit) if cm.group_needs[g].window
+                      else min(cm.pages_for(engine.ctx_limit), cm.pools[g].num_pages) for g in range(cm.n_groups)]
         # static metadata: ids pos row_req cu ctx slot logit_rows tables...
         sizes = [b, b, b, b + 1, b, b, b] + [b * w for w in self.width]
         offs = np.concatenate([[0], np.cumsum([(s + 3) // 4 * 4 for s in sizes])])

@@ -10,6 +10,37 @@ HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bfloat16": 2.5e15, "float16": 2.5e15, "float8": 5.0e15, "float32": 157.3e12}
 
 
+_measured_ceiling = None
+
+
+def measured_hbm_bytes_per_s(mib: int = 512, pool_mib: int = 2048, repeats: int = 5) -> float:
+    """What a kernel that only reads reaches on this GPU: `mib` MiB read by a plain sum kernel, the read
+    window moving through a pool of `pool_mib` MiB so that nothing is found in a cache, the best of
+    `repeats` timed by device events.  The reference divides by a measured streaming ceiling rather
+    than the spec-sheet figure (src/bench.rs:438-442); the rows report both.  Measured once per process."""
+    global _measured_ceiling
+    if _measured_ceiling is None:
+        import torch
+
+        from . import ops
+        pool = torch.empty(pool_mib << 19, dtype=torch.bfloat16, device="cuda").normal_()
+        sums = torch.zeros(4096, device="cuda")
+        nbytes, pool_bytes = mib << 20, pool_mib << 20
+        best = 0.0
+        for r in range(repeats + 1):                           # the first is the warm-up
+            offset = (r * nbytes) % (pool_bytes - nbytes + 1) // 256 * 256
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            ops.probe_read(pool, offset, nbytes, sums, grid=4096, block=256)
+            end.record()
+            torch.cuda.synchronize()
+            if r:
+                best = max(best, nbytes / (begin.elapsed_time(end) * 1e-3))
+        del pool
+        _measured_ceiling = best
+    return _measured_ceiling
+
+
 def torch_element_size(dtype) -> int:
     import torch
     return torch.empty((), dtype=dtype).element_size()

@@ -122,20 +122,24 @@ def plain_logits(model_dir: str, ids) -> np.ndarray:
 
 
 def tolerance(dtype: str) -> float:
-    """Largest allowed max|engine - plain| as a fraction of max|plain|.
+    """Largest allowed max|engine - plain| as a fraction of max|plain| in 32-bit: the reference's own
+    CPU tolerance of 1e-5 x scale (src/runtime/lm.rs:1497-1511); the engine measures about 2e-6.
+    bfloat16 runs are held to per-model bounds instead (`assert_close`, `BF16_REL_L2`, `max_logit_error`)."""
+    return {"float32": 1e-5}[dtype]
 
-    32-bit: the reference's own CPU tolerance of 1e-5 x scale
-    (src/runtime/lm.rs:1497-1511); the engine measures about 2e-6.
 
-    bfloat16: every activation that a matrix product reads or writes is rounded to 8 bits of
-    mantissa (relative error up to 2^-9 = 2e-3 each), about five such roundings lie on the path
-    through each half of a layer, and the error a layer inherits through the residual stream adds
-    to its own.  For these 3 to 6 layer models that gives a mean error of 1 to 2 % of the logits'
-    size and, over the 10^5 logits of a test, a maximum of about 3 % (measured: A 1.5 %, B 3.2 %,
-    C 1.7 %, the same in every execution mode).  This figure is what the smoke test and the
-    sampling tests use; the engine tests hold every row's relative L2 error and cosine against
-    per-model bounds instead (`assert_close`, `BF16_REL_L2`)."""
-    return {"float32": 1e-5, "bfloat16": 6e-2}[dtype]
+# Largest error of a single bfloat16 logit against the plain implementation, as a fraction of the
+# largest plain logit: 1.3 x the worst measured over every test of that model.  Every activation that a
+# matrix product reads or writes is rounded to 8 bits of mantissa (relative error up to 2^-9 each), about
+# five such roundings lie on the path through each half of a layer, and what a layer inherits through the
+# residual stream adds to its own: 1.5 to 3.2 % for these 3 to 6 layer models.
+BF16_MAX_ERR = {"A": 0.020, "B": 0.042, "C": 0.022}
+
+
+def max_logit_error(dtype: str, model: str) -> float:
+    """How far one logit of the engine may lie from the plain implementation's, as a fraction of the
+    largest plain logit."""
+    return 1e-5 if dtype == "float32" else BF16_MAX_ERR[model]
 
 
 def consistency(dtype: str) -> float:
@@ -190,8 +194,6 @@ def assert_close(got: np.ndarray, want: np.ndarray, dtype: str, what: str = "", 
     _record(what, model, dtype, float(rel.max()), float((g2 * w2).sum() / np.sqrt((g2 * g2).sum() * (w2 * w2).sum() + 1e-300)),
             float(err.max() / scale))
     if dtype == "bfloat16" and tol is None:
-        if os.environ.get("GIBBS_TEST_MEASURE"):        # a run that only records the errors (to set the bounds from)
-            return
         bound = BF16_REL_L2.get(model, BF16_REL_L2_OTHER)
         worst = int(np.argmax(rel))
         all_cos = (g2 * w2).sum() / np.sqrt((g2 * g2).sum() * (w2 * w2).sum() + 1e-300)

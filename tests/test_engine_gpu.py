@@ -335,8 +335,8 @@ def test_many_requests_decoding_side_by_side(tmp_path_factory, name, live, dtype
         general = run_steps(make_engine(d, dtype, max_tokens=live * 64, max_requests=live, fold_gains=False,
                                         fused_decode_rows=0), steps)
         for key in got:
-            # (measured: up to 3.4 % of the scale)
-            H.assert_close(got[key], general[key], dtype, f"{live} decoding {name}: fused vs general path {key}", tol=5.5e-2)
+            # (measured: up to 3.4 % of the scale; the bound is 1.3 x that)
+            H.assert_close(got[key], general[key], dtype, f"{live} decoding {name}: fused vs general path {key}", tol=4.4e-2)
 
 
 @pytest.mark.parametrize("live", [33, 64])
@@ -366,13 +366,19 @@ def test_captured_decode_loop_with_many_requests(tmp_path_factory, live):
     assert tokens["loop"] == tokens["steps"]
 
 
+@pytest.fixture(scope="module")
+def big_dir(tmp_path_factory):
+    """Three layers of the LFM2-1.2B layer sizes, written once for the tests below."""
+    return H.make_model_dir(str(tmp_path_factory.mktemp("big")), "L", seed=3, std=0.02)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_benchmark_layer_sizes(tmp_path_factory, dtype):
+def test_benchmark_layer_sizes(big_dir, dtype):
     """Three layers of the LFM2-1.2B layer sizes (hidden 2,048, 32 heads in 8 groups, feed-forward 8,192,
     vocabulary 65,536): a sequence whole, in portions of changing size, and with its last tokens one by
     one beside a second request, against the plain implementation (every place of the portions run,
     the decoded places, and a few of the whole run)."""
-    d = H.make_model_dir(str(tmp_path_factory.mktemp("big")), "L", seed=3, std=0.02)
+    d = big_dir
     vocab = H.TINY["L"]["vocab_size"]
     seqs = {"a": H.tokens(61, 150, vocab), "b": H.tokens(62, 40, vocab)}
     eng = make_engine(d, dtype, max_tokens=512, max_requests=2)
@@ -394,6 +400,67 @@ def test_benchmark_layer_sizes(tmp_path_factory, dtype):
     got = run_steps(eng, steps)
     assert ("a", 149) in got and ("b", 39) in got
     check(d, seqs, got, dtype, f"1.2B layer sizes, portions and decoding {dtype}", against_whole=False)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_benchmark_layer_sizes_many_requests_decoding(big_dir, dtype):
+    """17, 33, 48 and 64 live requests decoding side by side at the LFM2-1.2B layer sizes (what the
+    batch-64 figure of the benchmark runs): in bfloat16 the staged products of two to four tiles of rows,
+    two tiles of features per workgroup, the down projection cut along k with its partial sums added by a
+    second kernel, and the head through the few-row kernel (up to 48 rows) and the tiled product with
+    float32 output (above).  Prompts of different lengths, one request ends mid-way; every decoded
+    place against the plain implementation, and the bfloat16 fused path against the same engine on its
+    general path without folded gains."""
+    d = big_dir
+    vocab = H.TINY["L"]["vocab_size"]
+    rng = np.random.default_rng(64)
+    n_decode = 12
+    prompt_len = {f"r{i}": int(rng.integers(3, 22)) for i in range(64)}
+    seqs = {r: H.tokens(900 + i, n + (5 if i == 2 else n_decode), vocab) for i, (r, n) in enumerate(prompt_len.items())}
+    eng = make_engine(d, dtype, max_tokens=64 * 64, max_requests=64)
+    general = make_engine(d, dtype, max_tokens=64 * 64, max_requests=64, fold_gains=False, fused_decode_rows=0) if dtype == "bfloat16" else None
+    for live in (17, 33, 48, 64):
+        some = {r: seqs[r] for r in list(seqs)[:live]}
+        steps = decode_batch_steps(some, {r: prompt_len[r] for r in some}, "r2")
+        assert max(len(e) for e, _ in steps) == live and any(len(e) == live - 1 for e, _ in steps)
+        got = run_steps(eng, steps)
+        check(d, some, got, dtype, f"{live} decoding at the 1.2B layer sizes {dtype}", against_whole=False)
+        eng.cache.check()
+        assert eng.cache.free_pages() == eng.cache.pools[0].num_pages
+        if general is not None:
+            other = run_steps(general, steps)
+            for key in got:
+                # (measured: up to MEASURED_L % of the scale; the bound is 1.3 x that)
+                H.assert_close(got[key], other[key], dtype, f"{live} decoding at the 1.2B layer sizes: fused vs general path {key}", tol=3.0e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sequence_of_9000_tokens_in_pages_of_16(tmp_path_factory, dtype):
+    """9,000 tokens at the default page size: 563 pages, more page ids than a key slice of the decode
+    attention's matrix-core walk keeps in LDS (so the cache is cut into slices whatever the batch), and
+    prompt portions late in the sequence walk a second segment of the block table; the last 24 tokens one
+    by one, a short request beside them."""
+    d = H.make_model_dir(str(tmp_path_factory.mktemp("medium")), "M", seed=7, std=0.05)
+    total = 9000
+    seqs = {"long": H.tokens(51, total, 4096), "other": H.tokens(52, 60, 4096)}
+    at = {"long": 0, "other": 0}
+    cuts = [2048, 2048, 2048, 2048, 700, 64, 18, 2]
+    steps = []
+    while at["long"] < total:
+        left = total - at["long"]
+        n = min(cuts.pop(0), left - 24) if cuts and left > 24 else 1
+        want = sorted({0, n // 2} | set(range(max(0, n - 3), n)))
+        entries = [("long", seqs["long"][at["long"]:at["long"] + n], want)]
+        at["long"] += n
+        if at["other"] < 60:
+            m = 1 if at["other"] >= 40 else 20
+            entries.insert(0 if m == 1 else 1, ("other", seqs["other"][at["other"]:at["other"] + m], [m - 1]))
+            at["other"] += m
+        steps.append((entries, []))
+    eng = make_engine(d, dtype, max_tokens=9216 + 64, max_requests=2, page_size=16, ctx=9216)
+    got = run_steps(eng, steps)
+    assert ("long", total - 1) in got and sum(1 for r, p in got if r == "long" and p > 8192) >= 24
+    check(d, seqs, got, dtype, f"9,000 tokens {dtype}", against_whole=False)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -478,6 +478,88 @@ def test_qk_rope_kv(dtype, variant, nh, nkv, hd, rot, table_len):
     assert kp.float().abs().sum(dim=(1, 3)).count_nonzero().item() == n, "exactly one page slot per row was written"
 
 
+def plain_qk(x, gain, positions, inv, eps):
+    """Per-head RMSNorm then the half-split rotation of x [n, heads, hd], by the plain implementation
+    (float32 angle = float32(pos) * inv_freq, src/graph/cpu.rs:673)."""
+    from tests.plain import lfm2_plain as P
+    return torch.tensor(P.rope_half_split(P.rms_norm(x.double().cpu().numpy(), gain.double().cpu().numpy(), eps), positions, inv))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("table_len", [0, 4096])
+def test_qk_rope_kv_at_far_positions(dtype, table_len):
+    """theta 1e6, heads of 64, rows at positions 32,767 and 99,999 (and beside them, and near the start):
+    there the float32 product float32(pos) * inv_freq has lost its low bits, and an angle computed any
+    other way (in float64, from a recurrence, as pos * a rounded inverse) is off by up to 4e-3 rad.  Against
+    the plain implementation's rotation, which takes the reference's float32 steps."""
+    from gibbs_amd import ops
+    from tests.plain import lfm2_plain as P
+    nh, nkv, hd, page = 4, 2, 64, 16
+    positions = [99999, 32767, 99998, 5, 65536, 32768]
+    n = len(positions)
+    inv_np = P.rope_inv_freq(hd, 1e6)
+    inv = torch.from_numpy(inv_np).to(DEV)
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=3)
+    qkv0 = qkv.clone()
+    qg, kg = rnd(hd, seed=1) * 0.1 + 1, rnd(hd, seed=2) * 0.1 + 1
+    width = 100000 // page
+    table = np.full((n, width), -1, dtype=np.int32)
+    for r, p in enumerate(positions):                       # one request per row, one real page each
+        table[r, p // page] = n - 1 - r
+    kp = torch.zeros(n, nkv, page, hd, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    ops.qk_rope_kv(qkv, n, nh, nkv, hd, q_gain=qg, k_gain=kg, eps=1e-5, inv_freq=inv, rotary_dim=hd, variant="half_split",
+                   pos=i32(positions), row_req=i32(list(range(n))), kpages=kp, vpages=vp, table=i32(table), n_req=n,
+                   cos_sin=ops.rope_table(inv, table_len) if table_len else None)
+    q0 = qkv0[:, :nh * hd].view(n, nh, hd)
+    k0 = qkv0[:, nh * hd:(nh + nkv) * hd].view(n, nkv, hd)
+    close(qkv[:, :nh * hd].view(n, nh, hd), plain_qk(q0, qg, positions, inv_np, 1e-5), dtype, "q at far positions", f32=2e-6, bf16=8e-3)
+    kr = plain_qk(k0, kg, positions, inv_np, 1e-5)
+    for r, p in enumerate(positions):
+        close(kp[n - 1 - r, :, p % page], kr[r], dtype, f"k at position {p}", f32=2e-6, bf16=8e-3)
+    # the same angles in float64 would fail this bound: the test can tell the difference
+    ang32 = (np.float32(99999) * inv_np).astype(np.float64)
+    ang64 = 99999.0 * inv_np.astype(np.float64)
+    assert np.abs(np.cos(ang32) - np.cos(ang64)).max() > 1e-4
+
+
+@pytest.mark.parametrize("kind", ["valu", "mfma"])
+@pytest.mark.parametrize("window", [None, 48])
+def test_attention_decode_fused_at_far_positions(kind, window):
+    """Decoded tokens at positions 99,999 and 32,767 (theta 1e6, pages of 16: 6,250 page ids, so the
+    matrix-core walk must cut the cache into slices whatever the batch) beside a short request: q/k norm and
+    rotation against the plain implementation's, attention against float64 over all 100,000 keys.  The
+    query gain is large, so that the softmax stands on a few hundred keys spread over the whole cache (a
+    slice or a page lost shows), and with a window of 48 keys every score depends on the rotation."""
+    from gibbs_amd import ops
+    from tests.plain import lfm2_plain as P
+    dtype, nh, nkv, hd, page = torch.bfloat16, 8, 2, 64, 16
+    seq_lens = [100000, 32768, 40]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, sum(-(-l // page) for l in seq_lens) + 3, seed=11)
+    n = len(seq_lens)
+    positions = [l - 1 for l in seq_lens]
+    pos, row_req = i32(positions), i32(list(range(n)))
+    qkv = rnd(n, (nh + 2 * nkv) * hd, dtype=dtype, seed=9)
+    qg, kg = rnd(hd, seed=1) * 0.1 + 3.0, rnd(hd, seed=2) * 0.1 + 1
+    inv_np = P.rope_inv_freq(hd, 1e6)
+    inv = torch.from_numpy(inv_np).to(DEV)
+    scale = 1 / math.sqrt(hd)
+    got = ops.attention_decode_fused(qkv, n, nh, nkv, hd, kp, vp, table, n, pos, row_req, scale, q_gain=qg, k_gain=kg,
+                                     eps=1e-5, inv_freq=inv, rotary_dim=hd, variant="half_split", window=window,
+                                     max_seq=max(seq_lens), kind=kind, cos_sin=ops.rope_table(inv, 4096))
+    q = plain_qk(qkv[:, :nh * hd].view(n, nh, hd), qg, positions, inv_np, 1e-5).to(DEV)
+    k_new = plain_qk(qkv[:, nh * hd:(nh + nkv) * hd].view(n, nkv, hd), kg, positions, inv_np, 1e-5).to(DEV)
+    v_new = qkv[:, (nh + nkv) * hd:].view(n, nkv, hd)
+    for r, p in enumerate(positions):
+        pg = table[r, p // page].item()
+        close(kp[pg, :, p % page], k_new[r], dtype, f"new key at position {p}", bf16=8e-3)
+        assert torch.equal(vp[pg, :, p % page], v_new[r])
+        k_all = torch.cat([ks[r][:p].double(), k_new[r:r + 1]])
+        v_all = torch.cat([vs[r][:p].double(), v_new[r:r + 1].double()])
+        want = attention_reference(q[r:r + 1], k_all, v_all, [p], scale, window)
+        close(got[r].view(1, nh, hd), want, dtype, f"row at position {p}", bf16=1e-2)
+
+
 def test_rope_table():
     from gibbs_amd import ops
     from gibbs_amd.parts.rope import rope_inv_freq

@@ -436,6 +436,48 @@ def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
         H.assert_close(np.concatenate(got[r]), plain[r], name, f"windowed model request {r}")
 
 
+@pytest.mark.parametrize("name,dtype", DTYPES)
+def test_captured_decode_loop_past_the_pages_of_a_window_group(name, dtype):
+    """The captured decode loop on the model with a window's cache group whose pool (12 pages of 8 tokens) is
+    smaller than a request's count of logical pages: the request decodes to 150 tokens (19 logical pages, of
+    which the window's group holds 4 at a time), so the loop's block tables must be as wide as the context,
+    not as the pool.  Same greedy tokens as stepping the same engine from the host."""
+    from gibbs_amd import Engine
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.engine.decode import DecodeLoop
+    from gibbs_amd.parts import DecoderModel
+    from gibbs_amd.weights import random_tensor
+    spec = window_spec()
+    decls = DecoderModel(spec).tensor_decls()
+    tensors = {d.name: random_tensor(d, 9, torch.bfloat16, std=0.15, gain_std=0.1) for d in decls}
+
+    class Windowed(ArchConfig):
+        def model_spec(self):
+            return spec
+    prompt = H.tokens(5, 21, spec.vocab)
+    tokens = {}
+    for mode in ("loop", "steps"):
+        ws = store({k: v.float().numpy() for k, v in tensors.items()}, decls, dtype)
+        eng = Engine(config=Windowed(), weights=ws, dtype=name, max_tokens=24 * 8, max_requests=2, page_size=8,
+                     group_pages=[24, 12], ctx=192)
+        first = int(eng.step([("r", prompt, [len(prompt) - 1])]).argmax(-1).item())
+        if mode == "loop":
+            loop = DecodeLoop(eng, ["r"], [first])
+            assert loop.width == [24, 24], "one table entry per logical page of the context"
+            for n in (9, 40, 40, 39):                      # past 12 logical pages during the third run
+                loop.run(n)
+            tokens[mode] = [first] + loop.tokens()[0]
+            assert eng.cache.tokens("r") == 21 + 128
+            assert (eng.cache.block_table(["r"], 1)[0] >= 0).sum() <= 20 // 8 + 2
+        else:
+            out = [first]
+            for _ in range(128):
+                out.append(int(eng.step([("r", [out[-1]], [0])]).argmax(-1).item()))
+            tokens[mode] = out
+        eng.cache.check()
+    assert tokens["loop"] == tokens["steps"]
+
+
 # --------------------------------------------------------------------------- a toy mixer with its own state
 def register_toy():
     """An exponential moving average over time of a projection of the input: state [hidden] per
