@@ -430,8 +430,8 @@ def test_benchmark_layer_sizes_many_requests_decoding(big_dir, dtype):
         if general is not None:
             other = run_steps(general, steps)
             for key in got:
-                # (measured: up to MEASURED_L % of the scale; the bound is 1.3 x that)
-                H.assert_close(got[key], other[key], dtype, f"{live} decoding at the 1.2B layer sizes: fused vs general path {key}", tol=3.0e-2)
+                # (measured: up to 2.1 % of the scale; the bound is 1.3 x that)
+                H.assert_close(got[key], other[key], dtype, f"{live} decoding at the 1.2B layer sizes: fused vs general path {key}", tol=2.7e-2)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

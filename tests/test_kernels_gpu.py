@@ -547,8 +547,10 @@ def test_attention_decode_fused_at_far_positions(kind, window):
     got = ops.attention_decode_fused(qkv, n, nh, nkv, hd, kp, vp, table, n, pos, row_req, scale, q_gain=qg, k_gain=kg,
                                      eps=1e-5, inv_freq=inv, rotary_dim=hd, variant="half_split", window=window,
                                      max_seq=max(seq_lens), kind=kind, cos_sin=ops.rope_table(inv, 4096))
-    q = plain_qk(qkv[:, :nh * hd].view(n, nh, hd), qg, positions, inv_np, 1e-5).to(DEV)
-    k_new = plain_qk(qkv[:, nh * hd:(nh + nkv) * hd].view(n, nkv, hd), kg, positions, inv_np, 1e-5).to(DEV)
+    # (the kernel rounds the prepared q and the new key to bfloat16, as the separate kernels store them; with
+    # scores this large that rounding alone moves the output by 1 %, so the reference takes the same values)
+    q = plain_qk(qkv[:, :nh * hd].view(n, nh, hd), qg, positions, inv_np, 1e-5).to(DEV).to(dtype).double()
+    k_new = plain_qk(qkv[:, nh * hd:(nh + nkv) * hd].view(n, nkv, hd), kg, positions, inv_np, 1e-5).to(DEV).to(dtype).double()
     v_new = qkv[:, (nh + nkv) * hd:].view(n, nkv, hd)
     for r, p in enumerate(positions):
         pg = table[r, p // page].item()
@@ -718,7 +720,8 @@ def test_skinny_glu(n, f, i):
 
 
 @pytest.mark.parametrize("n,c,i,k,bias", [(1, 2048, 2048, 3, False), (8, 72, 96, 4, True), (20, 40, 64, 2, True), (64, 96, 128, 3, False),
-                                          (13, 2056, 96, 3, True), (16, 2104, 64, 4, False), (11, 40, 64, 2, True)])   # 9 to 16 rows
+                                          (13, 2056, 96, 3, True), (16, 2104, 64, 4, False), (11, 40, 64, 2, True),   # 9 to 16 rows
+                                          (31, 1, 512, 3, False), (2, 1, 520, 4, True)])   # one channel: sums that cancel
 def test_skinny_conv(n, c, i, k, bias):
     """In-projection + convolution of decoded tokens against the unfused kernels and the reference."""
     from gibbs_amd import ops
@@ -735,6 +738,7 @@ def test_skinny_conv(n, c, i, k, bias):
     bcx = (x.double() @ w.double().t()) * rms_scale(x, 1e-5)
     B, C, X = bcx[:, :c], bcx[:, c:2 * c], bcx[:, 2 * c:]
     bx = B * X
+    want_state = state2.double().clone()
     for r in range(n):
         hist = state2[slots[r]].double().clone()
         for j in range(k - 1):
@@ -743,7 +747,12 @@ def test_skinny_conv(n, c, i, k, bias):
         window = torch.cat([hist, bx[r:r + 1]])
         cv = (window * taps.double().t()).sum(0) + (b.double() if bias else 0)
         close(y[r], C[r] * cv, torch.bfloat16, f"skinny_conv row {r}", bf16=8e-3)
-        close(state[slots[r]], window[1:], torch.float32, "state", f32=2e-5)
+        want_state[slots[r]] = window[1:]
+    # All rows' states against one scale.  The new entry B * x is a product of two float32 sums over k, whose
+    # rounding error follows the size of their terms, not of the sums: with one channel, a row whose B or x
+    # cancels to almost nothing has a tiny state of its own and misses a bound taken from that row alone
+    # (random shapes found such rows), though every value is as exact as float32 sums get.
+    close(state, want_state, torch.float32, "state", f32=2e-5)
     untouched = [s for s in range(n + 3) if s not in slots.tolist()]
     assert torch.equal(state[untouched], state2[untouched])
 
