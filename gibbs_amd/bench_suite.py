@@ -12,7 +12,6 @@ model entry inherits the defaults; the keys that mean something here:
     batch           requests decoded side by side (default 1)
     dtype           "bfloat16" (default) or "float32"
     min_tok_s       the run fails (exit status 3) if decode is slower
-    native_step     false: step through the parts in Python instead of the one native call
     workload        "decode" (default: the protocol below) or "serve": `requests` prompts of
                     `prefill_tokens` seeded ids each are submitted at once to the continuous-batching
                     scheduler and generate `decode_tokens` tokens each (greedy, no EOS), with
@@ -80,11 +79,9 @@ def _load(entry: Dict, base: str, batch: int = 0, ctx: int = 0):
         decls = DecoderModel(cfg.model_spec()).tensor_decls()
         compute = torch.bfloat16 if entry["dtype"] == "bfloat16" else torch.float32
         weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0")
-        return Engine(config=cfg, weights=weights, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx,
-                      native_step=bool(entry.get("native_step", True)))
+        return Engine(config=cfg, weights=weights, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
     path = ident if os.path.isabs(ident) else os.path.join(base, ident)
-    return Engine(path, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx,
-                      native_step=bool(entry.get("native_step", True)))
+    return Engine(path, dtype=entry["dtype"], max_tokens=batch * ctx, max_requests=batch, ctx=ctx)
 
 
 def measure(entry: Dict, base: str) -> Dict:
@@ -218,7 +215,7 @@ def products(entry: Dict, base: str) -> Dict:
     rows, iters, only = int(entry.get("rows", 2048)), int(entry.get("iters", 24)), entry.get("only")
     shapes: List[tuple] = []
     for block in model.blocks:
-        for part in (block.mixer, block.ffn):
+        for part in block.parts():
             for shape in part.product_shapes():
                 if shape not in shapes:
                     shapes.append(shape)
@@ -304,7 +301,7 @@ def streams(entry: Dict, base: str) -> Dict:
         model = DecoderModel(cfg.model_spec())
         shapes: List[tuple] = []
         for block in model.blocks:
-            for part in (block.mixer, block.ffn):
+            for part in block.parts():
                 for shape in part.product_shapes():
                     if shape not in shapes:
                         shapes.append(shape)
@@ -350,7 +347,7 @@ def mixed(entry: Dict, base: str) -> Dict:
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     return {"model": entry["name"], "workload": "mixed", "dtype": entry["dtype"], "decoding": n_dec, "portion": portion,
-            "rows": n_dec + portion, "cached_tokens": cached, "native_step": engine.plan is not None,
+            "rows": n_dec + portion, "cached_tokens": cached,
             "ms_per_step": round(1e3 * wall / steps, 4), "host_ms_per_step": round(1e3 * host / steps, 4)}
 
 

@@ -10,7 +10,7 @@ a field; none is written into the code of a part.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Mapping, Optional, Tuple
+from typing import Any, Mapping, Optional, Sequence, Tuple, Union
 
 
 @dataclass(frozen=True)
@@ -51,24 +51,57 @@ class FeedForwardSpec:
     tensors: Mapping[str, str]
 
 
-@dataclass(frozen=True)
+PartSpec = Union[NormSpec, MixerSpec, FeedForwardSpec]
+
+
 class LayerSpec:
-    """One block: how norm, mixer and feed-forward are arranged (`"pre_norm"`:
-    x += mixer(norm(x)); x += ffn(norm(x)))."""
-    name: str                       # checkpoint prefix, e.g. "model.layers.3"
-    arrangement: str
-    mixer_norm: NormSpec
-    mixer: MixerSpec
-    ffn_norm: NormSpec
-    ffn: FeedForwardSpec
+    """One block: its parts by role, in the order the arrangement names them, and how they are arranged.
+    `"pre_norm"` (x += mixer(mixer_norm(x)); x += ffn(ffn_norm(x))) takes the four roles `mixer_norm`,
+    `mixer`, `ffn_norm`, `ffn`, which may be given in that order as positional arguments; another
+    arrangement names whatever roles it wants through `parts` (one norm and two bodies, a block
+    without a feed-forward, two mixers, norms after the bodies), and any number of them may be
+    mixers with caches or state of their own."""
+    PRE_NORM_ROLES = ("mixer_norm", "mixer", "ffn_norm", "ffn")
+
+    def __init__(self, name: str, arrangement: str, mixer_norm: Optional[NormSpec] = None, mixer: Optional[MixerSpec] = None,
+                 ffn_norm: Optional[NormSpec] = None, ffn: Optional[FeedForwardSpec] = None,
+                 parts: Optional[Sequence[Tuple[str, PartSpec]]] = None):
+        self.name = name                    # checkpoint prefix, e.g. "model.layers.3"
+        self.arrangement = arrangement
+        if parts is None:
+            parts = [(r, p) for r, p in zip(self.PRE_NORM_ROLES, (mixer_norm, mixer, ffn_norm, ffn)) if p is not None]
+        elif any(p is not None for p in (mixer_norm, mixer, ffn_norm, ffn)):
+            raise ValueError("a layer's parts are given either by role (`parts`) or as the four of a pre-norm block")
+        self.parts: Tuple[Tuple[str, PartSpec], ...] = tuple((str(r), p) for r, p in parts)
+        roles = [r for r, _ in self.parts]
+        if len(set(roles)) != len(roles):
+            raise ValueError(f"layer {name!r} names a role twice: {roles}")
+
+    def part(self, role: str) -> PartSpec:
+        for r, p in self.parts:
+            if r == role:
+                return p
+        raise KeyError(f"layer {self.name!r} has no part {role!r}; it has {[r for r, _ in self.parts]}")
+
+    # the four roles of a pre-norm block, by name
+    mixer_norm = property(lambda self: self.part("mixer_norm"))
+    mixer = property(lambda self: self.part("mixer"))
+    ffn_norm = property(lambda self: self.part("ffn_norm"))
+    ffn = property(lambda self: self.part("ffn"))
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, LayerSpec) and (self.name, self.arrangement, self.parts) == (other.name, other.arrangement, other.parts)
+
+    def __repr__(self) -> str:
+        return f"LayerSpec({self.name!r}, {self.arrangement!r}, parts={self.parts!r})"
 
 
 @dataclass(frozen=True)
 class ModelSpec:
     """A whole decoder.  `layers` are the distinct layers (each owns weights and, if its
-    mixer needs one, a cache); `order` is the list of layer indices in the order they run:
+    mixers need them, caches); `order` is the list of layer indices in the order they run:
     it may name a layer twice.  A mixer whose params carry `kv_source` reads the cache of
-    that layer instead of owning one."""
+    that layer (of its first mixer that owns one) instead of owning one."""
     architecture: str
     hidden: int
     vocab: int

@@ -92,12 +92,9 @@ class DecodeLoop:
         self.counter = torch.zeros(b, dtype=torch.int32, device=dev)          # steps done, per row
         # native step: the rows of the residual stream (and their bfloat16 mirror) live here from one step to
         # the next; the end of a step writes the next tokens' embeddings into them
-        self.x = self.mirror = None
-        if engine.plan is not None:
-            hidden = engine.spec.hidden
-            self.x = torch.zeros((b, hidden), dtype=torch.float32, device=dev)
-            if engine.dtype == torch.bfloat16:
-                self.mirror = torch.zeros((b, hidden), dtype=torch.bfloat16, device=dev)
+        hidden = engine.spec.hidden
+        self.x = torch.zeros((b, hidden), dtype=torch.float32, device=dev)
+        self.mirror = torch.zeros((b, hidden), dtype=torch.bfloat16, device=dev) if engine.dtype == torch.bfloat16 else None
         if not self.greedy:
             self.temperature = torch.zeros(b, dtype=torch.float32, device=dev)
             self.top_p = torch.zeros(b, dtype=torch.float32, device=dev)
@@ -156,8 +153,7 @@ class DecodeLoop:
     def _embed(self) -> None:
         """The embeddings of the tokens in `ids` into the loop's residual rows (the first step after binding;
         every later step finds what the end of the step before it wrote)."""
-        if self.x is not None:
-            ops.embed(self.engine.model.table, self.batch.ids, self.n, out=self.x, mirror=self.mirror)
+        ops.embed(self.engine.model.table, self.batch.ids, self.n, out=self.x, mirror=self.mirror)
 
     # ------------------------------------------------------------------ host side
     def _fill_tables(self) -> None:
@@ -192,7 +188,7 @@ class DecodeLoop:
     def _step(self) -> None:
         b = self.batch
         logits = self.engine.forward(b, self._workspace, self.x, self.mirror)
-        table = self.engine.model.table if self.x is not None else None
+        table = self.engine.model.table
         if self.greedy:
             ops.decode_tail(logits, b.ids, b.pos, b.ctx, self.log, self.counter, None, None, self.n, table, self.x, self.mirror)
         else:
@@ -224,7 +220,7 @@ class DecodeLoop:
         self.u.copy_(self.u_all[self.steps_done])
 
     def _capture(self, many: bool) -> None:
-        if self.graph is None and self.engine.plan is not None:
+        if self.graph is None:
             # the native step's activations: a buffer of the loop's own, which the captured graphs replay
             # over (the engine's own may be replaced by a larger one when another step needs more)
             need = self.engine.plan.workspace_bytes(self.batch, self.x, self.mirror)

@@ -22,7 +22,7 @@ from ..config import config_from_dict, read_config_json
 from ..config.base import ArchConfig
 from ..ops.lib import KernelError, library
 from ..parts import DecoderModel, Runtime
-from ..parts.native import MAX_GROUPS, NativePlan
+from ..parts.native import NativePlan
 from ..weights import WeightStore, load_weights, table_of
 from .batch import BatchStager, Entry, StepBatch
 
@@ -44,7 +44,7 @@ class Engine:
                  max_requests: int = 8, page_size: int = DEFAULT_PAGE_SIZE, device: str = "cuda:0", arch: Optional[str] = None,
                  ctx: Optional[int] = None, config: Optional[ArchConfig] = None,
                  weights: Optional[WeightStore] = None, fold_gains: bool = True, fused_decode_rows: int = 64,
-                 group_pages: Optional[Sequence[int]] = None, native_step: bool = True):
+                 group_pages: Optional[Sequence[int]] = None):
         """`model_dir`: a folder with config.json and model.safetensors (the model class is chosen
         by config.json).  `max_tokens`: tokens the cache pool holds (each request's count rounded
         up to whole pages).  `ctx`: context limit, default config.json's max_position_embeddings or 4,096,
@@ -54,9 +54,7 @@ class Engine:
         keeps steps of decoded tokens off the fused decode kernels: the same model on the general path,
         for comparisons.  `group_pages`: pages of every cache group's pool, one count per group in
         the order the groups first appear in the layer order (default: `max_tokens` worth for each; a
-        group with a window can do with about max_requests x (window + longest portion) tokens).
-        `native_step=False` steps through the parts in Python instead of the one native call (the
-        same kernels; a model with a part from outside the package always does)."""
+        group with a window can do with about max_requests x (window + longest portion) tokens)."""
         if not torch.cuda.is_available():
             raise KernelError("no GPU: this engine has no CPU path")
         if dtype not in DTYPES:
@@ -86,10 +84,12 @@ class Engine:
         self.cache = CacheManager(self.model.cache_needs(), self.model.state_needs(), page_size,
                                   num_pages if group_pages is None else list(group_pages), max_requests)
         self.device_cache = DeviceCache(self.cache, self.dtype, self.device)
-        self._views = [self.device_cache.layer_view(run, src)
-                       for run, src in enumerate(self.model.kv_source_runs())]
+        # the cache views of every run's mixers, by role (a cache owner is a mixer of a run)
+        self._views: List[Dict[str, object]] = [{} for _ in self.spec.order]
+        for owner, ((run, role), src) in enumerate(zip(self.model.cache_owners(), self.model.kv_sources())):
+            self._views[run][role] = self.device_cache.layer_view(owner, src)
         self._stager = BatchStager(self.device)
-        self.plan = NativePlan.build(self.model, self._views, self.rt) if native_step and self.cache.n_groups <= MAX_GROUPS else None
+        self.plan = NativePlan.build(self.model, self._views, self.rt)
 
     # ------------------------------------------------------------------ requests
     def admit(self, rid: Hashable) -> bool:
@@ -152,12 +152,9 @@ class Engine:
 
     def forward(self, batch: StepBatch, workspace: Optional[torch.Tensor] = None, x_in: Optional[torch.Tensor] = None,
                 mirror_in: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-        """The model's forward pass over a staged batch: one native call when the model has a plan
-        (`workspace`, `x_in`, `mirror_in`: see `NativePlan.step`), else through the parts."""
-        if self.plan is not None:
-            return self.plan.step(batch, workspace, x_in, mirror_in)
-        assert x_in is None, "only the native step takes the rows' embeddings from its caller"
-        return self.model.forward(batch, self._views)
+        """The model's forward pass over a staged batch: one native call (`workspace`, `x_in`,
+        `mirror_in`: see `NativePlan.step`)."""
+        return self.plan.step(batch, workspace, x_in, mirror_in)
 
     def step(self, entries: Sequence[Entry]) -> Optional[torch.Tensor]:
         """Runs one batch; returns float32 logits [wanted places, vocab] in the order of the

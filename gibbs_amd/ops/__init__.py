@@ -219,11 +219,9 @@ def _w(w) -> torch.Tensor:
 
 def skinny_splits(n_out: int, inner: int, want_blocks: int = 512, features: int = 16, min_k: int = 1024) -> int:
     """How many ranges of k `gemm_skinny` should cut a product into so that at least `want_blocks`
-    workgroups run (a workgroup owns `features` output features), each with at least `min_k` of k."""
-    blocks = -(-n_out // features)
-    s = max(1, min(-(-want_blocks // blocks), inner // min_k))
-    per = -(-(-(-inner // s)) // 128) * 128
-    return -(-inner // per)
+    workgroups run (a workgroup owns `features` output features), each with at least `min_k` of k
+    (the rule is the native step's)."""
+    return int(library().gibbs_rule_skinny_splits(n_out, inner, want_blocks, features, min_k))
 
 
 def gemm_skinny(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype = torch.bfloat16, k_splits: int = 1,
@@ -291,14 +289,11 @@ def skinny_residual(x_in: torch.Tensor, w: torch.Tensor, stream_x: torch.Tensor,
     o = w.shape[0]
     assert stream_x.dtype == torch.float32 and stream_x.shape == (n, o) and stream_x.is_contiguous()
     assert mirror.dtype == torch.bfloat16 and mirror.shape == (n, o) and mirror.is_contiguous()
-    if n > 32 and i >= 4096:
-        # many rows and a long inner size: every workgroup re-reads x_in, so workgroups take 64 features
-        # each and the chip is filled by cutting k instead; the partial sums are added to the stream by
-        # a second kernel (measured at 33 to 64 rows: 17 against 24 us at k = 8192, 12 against 9 at 2048)
-        parts = gemm_skinny(x_in, w, torch.float32, skinny_splits(o, i, want_blocks=256, features=64, min_k=256))
-        residual_add(stream_x, parts if parts.dim() == 3 else parts[None], mirror)
-        return
-    call("gibbs_skinny_residual", ptr(x_in), ptr(_w(w)), ptr(stream_x), ptr(mirror), n, o, i, ldx, w.stride(0), stream())
+    # (many rows and a long inner size: k is cut over workgroups and the float32 partial sums are added to the
+    # stream by a second kernel; whether, and into how many, is the native step's rule)
+    floats = int(library().gibbs_skinny_residual_workspace(n, o, i))
+    parts = torch.empty(floats, dtype=torch.float32, device=x_in.device) if floats else None
+    call("gibbs_skinny_residual_routed", ptr(x_in), ptr(_w(w)), w.stride(0), ptr(stream_x), ptr(mirror), n, o, i, ptr(parts), stream())
 
 
 def skinny_glu(x: torch.Tensor, w_gate_up: torch.Tensor, rms_eps: Optional[float] = None,
@@ -515,27 +510,15 @@ def slices_workspace(n_rows: int, nh: int, hd: int, n_splits: int) -> int:
     return int(library().gibbs_attention_decode_workspace(n_rows, nh, hd, n_splits))
 
 
-MATRIX_SLICE_PAGES = 510   # page ids of a key slice that the matrix-core walk keeps in LDS
-
-
 def decode_splits(n_rows: int, nkv: int, group: int, max_seq: int, hd: int = 0, kind: str = "auto",
                   page_size: int = 16) -> tuple:
-    """(key slices per (row, kv head), waves per workgroup) for the decode attention.  Few rows:
-    enough slices to give each of the 256 compute units two workgroups of 4 waves, but at least 64
-    keys to a slice (256 on the matrix cores: two tiles of 32 for every wave, and few enough slices for the merge
-    to take them at once).  Rows and heads that fill
-    the chip by themselves: no slices (a slice costs every wave its own prologue and final fold), 8
-    waves on the vector units, 4 on the matrix cores (measured at batch 1 to 64, 2,048 to 8,192 keys).
-    The matrix-core walk keeps the page ids of a whole slice in LDS: caches longer than that are cut
-    into as many slices as it takes."""
-    matrix = kind != "valu" and hd > 0 and hd % 16 == 0 and hd <= 128
-    gt = 8 if group >= 8 else (4 if group > 2 else group)
-    per_split = n_rows * nkv * -(-group // gt)
-    least = max(1, -(-max_seq // (MATRIX_SLICE_PAGES * page_size - 256))) if matrix else 1
-    if per_split >= 256:
-        return least, (4 if matrix else 8)
-    want = -(-512 // per_split)
-    return max(least, min(want, max_seq // (256 if matrix else 64), 256)), 4
+    """(key slices per (row, kv head), waves per workgroup) that the native step would choose for the
+    decode attention (csrc/step_plan.hip)."""
+    import ctypes
+    n_splits, waves = ctypes.c_int(0), ctypes.c_int(0)
+    library().gibbs_rule_decode_splits(n_rows, nkv, group, max_seq, hd, page_size, DECODE_KINDS[kind], ctypes.byref(n_splits),
+                                       ctypes.byref(waves))
+    return n_splits.value, waves.value
 
 
 def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
@@ -578,15 +561,8 @@ def attention_decode(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, k
 
 
 def prefill_splits(n_tiles: int, nh: int, max_seq: int, window: Optional[int] = None) -> int:
-    """Slices of the key tiles for the prompt attention: none while the query tiles and heads fill the
-    chip by themselves (about three workgroups per compute unit); else enough for eight workgroups per
-    compute unit, with at least four tiles of 64 keys to a slice (measured: 512 rows over 7,680 cached
-    keys take 203 us whole, 113 us in 4 slices, 94 us in 8)."""
-    blocks = max(1, n_tiles * nh)
-    keys = max_seq if not window else min(max_seq, int(window) + 64)
-    if blocks >= 768 or keys < 8 * 64:
-        return 1
-    return max(1, min(-(-2048 // blocks), keys // 256, 16))
+    """Slices of the key tiles that the native step would choose for the prompt attention (csrc/step_plan.hip)."""
+    return int(library().gibbs_rule_prefill_splits(n_tiles, nh, max_seq, int(window or 0)))
 
 
 def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kpages: torch.Tensor,
@@ -615,7 +591,7 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
     assert out.shape == (n_rows, nh * hd) and out.dtype == q.dtype and out.is_contiguous()
     rows, reqs = n_rows - first_row, n_req - first_req
     if n_splits is None:
-        n_splits = prefill_splits(-(-rows // 64) + reqs // 2, nh, max_seq, window) if max_seq > 0 else 1
+        n_splits = prefill_splits(int(library().gibbs_rule_prefill_tiles(rows, reqs)), nh, max_seq, window) if max_seq > 0 else 1
     partial = None
     if n_splits > 1:
         partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=q.device)

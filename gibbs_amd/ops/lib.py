@@ -67,22 +67,20 @@ _SIGNATURES = {
     "gibbs_probe_read": [c_void_p, c_long, c_void_p, c_int, c_int, c_void_p],
     "gibbs_repetition_penalty": [c_void_p, c_int, c_int, c_long, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     "gibbs_sample": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    "gibbs_linear": [c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
+    "gibbs_skinny_residual_routed": [c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p],
 }
 
 
 _VALUE_SIGNATURES = {
-    "gibbs_plan_create": ([c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_float, c_int, c_int], c_void_p),
-    "gibbs_plan_destroy": ([c_void_p], None),
-    "gibbs_plan_add_block": ([c_void_p, c_void_p, c_float, c_void_p, c_float], c_int),
-    "gibbs_plan_set_conv": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p,
-                             c_long, c_int], c_int),
-    "gibbs_plan_set_attention": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int,
-                                  c_void_p, c_void_p, c_float, c_void_p, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p,
-                                  c_int, c_int, c_int, c_int, c_int], c_int),
-    "gibbs_plan_set_glu": ([c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
-    "gibbs_plan_workspace": ([c_void_p, c_void_p], c_long),
-    "gibbs_plan_step": ([c_void_p, c_void_p], c_int),
     "gibbs_pair_layout_below_tiles": ([], c_int),
+    "gibbs_rule_skinny_splits": ([c_int, c_int, c_int, c_int, c_int], c_int),
+    "gibbs_rule_decode_splits": ([c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p], None),
+    "gibbs_rule_prefill_splits": ([c_long, c_int, c_int, c_int], c_int),
+    "gibbs_rule_prefill_tiles": ([c_int, c_int], c_long),
+    "gibbs_rule_fused_rows": ([], c_int),
+    "gibbs_linear_splits": ([c_int, c_int, c_int, c_int, c_long, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
+    "gibbs_skinny_residual_workspace": ([c_int, c_int, c_int], c_long),
 }
 
 
@@ -104,6 +102,8 @@ def library() -> ctypes.CDLL:
                     fn.restype = c_int
                 for name, (argtypes, restype) in _VALUE_SIGNATURES.items():
                     getattr(lib, name).argtypes, getattr(lib, name).restype = argtypes, restype
+                from ..parts import native
+                native.declare(lib)
                 for name in ("gibbs_gemm_library_timings", "gibbs_gemm_library_plans"):
                     getattr(lib, name).argtypes, getattr(lib, name).restype = [], c_long
                 lib.gibbs_attention_decode_workspace.argtypes = [c_int, c_int, c_int, c_int]

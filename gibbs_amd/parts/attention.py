@@ -9,9 +9,10 @@ kv head h // (heads / kv_heads) with scale `scale`; output projection.  A mixer 
 name `kv_source` projects no k, v and reads that layer's pages (the reference's `write: false`).
 
 The position encoding is asked how it works (`PositionEncoding`): a rotation goes to the kernels
-as tables and every fast path stays open; an encoding that changes q and k itself (`apply`) or
-biases the scores by distance (`score_slopes`) sends the mixer down its general path (norm, the
-hook, cache write; the plain attention kernel takes the slopes).
+as tables and every fast path stays open; an encoding that changes q and k itself (`apply`) is
+called back between the q/k norm and the cache write, and one that biases the scores by distance
+(`score_slopes`) takes the plain attention kernel, which knows such a bias.  Which kernels a step
+takes is decided where the step runs (csrc/step_plan.hip).
 """
 from __future__ import annotations
 
@@ -21,12 +22,8 @@ import torch
 
 from .. import ops
 from ..cache.needs import CacheNeed
-from ..ops.linear import linear
 from ..weights.loader import FLOAT32, TensorDecl, WeightStore
 from .base import Mixer, Runtime, build_position, register_mixer
-
-
-MIN_LEADING_DECODED = 2      # decoded tokens at the head of a mixed step that are worth a kernel of their own
 
 
 @register_mixer("attention")
@@ -95,8 +92,6 @@ class AttentionMixer(Mixer):
             self.pos_hook = self.rot is None and self.position.transforms_rows()
         if self.slopes is not None and (self.slopes.dtype != torch.float32 or tuple(self.slopes.shape) != (self.heads,)):
             raise ValueError(f"score slopes must be float32 [{self.heads}]")
-        # the fast kernels know rotations only (or no encoding at all)
-        self.fast_ok = self.slopes is None and not self.pos_hook
 
     def matrices(self):
         return [self.w_qkv, self.w_out]
@@ -117,98 +112,12 @@ class AttentionMixer(Mixer):
         self.p_qkv = ops.PackedWeight(self.w_qkv)
         self.p_out = ops.PackedWeight(self.w_out)
 
-    def _rotation_args(self) -> dict:
-        """The rotation as the kernels take it (no rotation: nulls)."""
-        r = self.rot
-        if r is None:
-            return dict(inv_freq=None, rotary_dim=0, variant="half_split", cos_sin=None)
-        return dict(inv_freq=r.inv_freq, rotary_dim=r.rotary_dim, variant=r.variant, cos_sin=r.cos_sin)
-
-    def can_decode_fused(self, batch) -> bool:
-        rot_ok = self.fast_ok and (self.rot is None or self.rot.rotary_dim % 16 == 0)
-        return (self.source is None and self.hidden % 8 == 0 and self.head_dim % 16 == 0 and self.head_dim <= 256
-                and rot_ok and (self.heads * self.head_dim) % 8 == 0)
-
-    def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
-        """norm -> q, k, v in one kernel; q/k norm, rotation, the write of the new key and value and
-        attention over split keys in a second (and the merge of the slices); out_proj + residual
-        add in a third."""
-        qkv = ops.skinny_store(stream.mirror, self.p_qkv or self.w_qkv, rms_eps=norm_eps)
-        ops.skinny_residual(self._attend_decoded(qkv, batch, cache), self.p_out or self.w_out, stream.x, stream.mirror)
-
-    def _attend_decoded(self, qkv, batch, cache) -> torch.Tensor:
-        """A step of single decoded tokens, from the raw projection: one kernel norms and rotates q and
-        the new key, writes key and value to their pages and attends."""
-        return ops.attention_decode_fused(
-            qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages, cache.vpages,
-            batch.tables[cache.group], batch.n_req, batch.pos, batch.row_req, self.scale, q_gain=self.q_gain,
-            k_gain=self.k_gain, eps=self.qk_norm_eps, window=self.window, max_seq=batch.max_seq,
-            **self._rotation_args())
-
-    def emit_native(self, builder, cache, folded: bool) -> bool:
-        if not self.fast_ok or cache.kpages is None or cache.kpages.shape != cache.vpages.shape:
-            return False                # (an encoding with a hook or score slopes steps through `forward`)
-        builder.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
-                          kv_heads=self.kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
-                          q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
-                          kpages=cache.kpages, vpages=cache.vpages, group=cache.group, owns=self.source is None,
-                          fusable=folded and self.can_decode_fused(None))
-        return True
-
-    # ------------------------------------------------------------------ one step
-    def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
-        n = batch.n_rows
-        qkv = linear(h, self.w_qkv)
-        table = batch.tables[cache.group]
-        owns = self.source is None
-        rot_ok = self.fast_ok and (self.rot is None or self.rot.rotary_dim % 16 == 0)
-        if (owns and self.rt.act_dtype == torch.bfloat16 and batch.max_q == 1 and self.head_dim % 16 == 0
-                and self.head_dim <= 256 and rot_ok):
-            return linear(self._attend_decoded(qkv, batch, cache), self.w_out, partial_ok=True, packed=self.p_out)
-        nkv = self.kv_heads if owns else 0
-        where = dict(pos=batch.pos, row_req=batch.row_req, table=table, n_req=batch.n_req)
-        pages = dict(kpages=cache.kpages if owns else None, vpages=cache.vpages if owns else None)
-        if self.pos_hook:
-            # q/k norm, then the encoding's own doing on the rows, then k and v into their pages
-            hd = self.head_dim
-            plain = dict(k_gain=None, eps=self.qk_norm_eps, **self._rotation_args(), **where)
-            k_rows = qkv[:, self.heads * hd:(self.heads + nkv) * hd]
-            if self.q_gain is not None:          # the kernel norms heads in place when it is given no pages
-                ops.qk_rope_kv(qkv, n, self.heads, 0, hd, q_gain=self.q_gain, kpages=None, vpages=None, **plain)
-            if owns and self.k_gain is not None:
-                ops.qk_rope_kv(k_rows, n, nkv, 0, hd, q_gain=self.k_gain, kpages=None, vpages=None, **plain)
-            self.position.apply(qkv[:, :self.heads * hd].unflatten(1, (self.heads, hd)),
-                                k_rows.unflatten(1, (nkv, hd)) if owns else None, batch)
-            if owns:
-                ops.qk_rope_kv(qkv, n, self.heads, nkv, hd, q_gain=None, **pages, **plain)
-        else:
-            ops.qk_rope_kv(qkv, n, self.heads, nkv, self.head_dim, q_gain=self.q_gain, k_gain=self.k_gain,
-                           eps=self.qk_norm_eps, **self._rotation_args(), **pages, **where)
-        a = self.attend(qkv, batch, cache, table)
-        return linear(a, self.w_out, partial_ok=True, packed=self.p_out)
-
-    def attend(self, qkv, batch, cache, table) -> torch.Tensor:
-        """Attention of the step's rows over the cache.  bfloat16: rows that are all single decoded
-        tokens take the kernel that splits the keys, steps with prompt portions the matrix-core
-        kernel (head sizes up to 128).  float32, and whatever the fast kernels do not take: the
-        plain kernel."""
-        bf16 = self.rt.act_dtype == torch.bfloat16 and self.slopes is None   # (the fast kernels take no score bias)
-        if bf16 and batch.max_q > 1 and self.head_dim % 16 == 0 and self.head_dim <= 128:
-            # decoded tokens at the head of the batch (where the scheduler puts them) take the kernel that
-            # splits their keys; a row of its own in the matrix-core kernel would walk its cache alone
-            lead = batch.lead_single if batch.lead_single >= MIN_LEADING_DECODED else 0
-            out = torch.empty((batch.n_rows, self.heads * self.head_dim), dtype=qkv.dtype, device=qkv.device)
-            if lead:
-                ops.attention_decode(qkv[:lead], lead, self.heads, self.kv_heads, self.head_dim, cache.kpages,
-                                     cache.vpages, table, batch.n_req, batch.pos[:lead], batch.row_req[:lead],
-                                     self.scale, self.window, max_seq=batch.max_seq, out=out[:lead])
-            return ops.attention_prefill(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
-                                         cache.vpages, table, batch.n_req, batch.cu, batch.ctx, self.scale, self.window,
-                                         out=out, max_seq=batch.max_seq, first_req=lead, first_row=lead)
-        if bf16 and batch.max_q == 1 and self.head_dim % 8 == 0:
-            return ops.attention_decode(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
-                                        cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
-                                        self.window, max_seq=batch.max_seq)
-        return ops.attention_plain(qkv, batch.n_rows, self.heads, self.kv_heads, self.head_dim, cache.kpages,
-                                   cache.vpages, table, batch.n_req, batch.pos, batch.row_req, self.scale,
-                                   self.window, slopes=self.slopes)
+    def emit(self, plan, cache) -> int:
+        if cache.kpages is None or cache.kpages.shape != cache.vpages.shape:
+            raise ValueError("the attention mixer's kernels want keys and values of one head size")
+        hook = self.position.apply if self.pos_hook else None
+        return plan.attention(w_qkv=self.w_qkv, p_qkv=self.p_qkv, w_out=self.w_out, p_out=self.p_out, heads=self.heads,
+                              kv_heads=self.kv_heads, head_dim=self.head_dim, scale=self.scale, window=self.window,
+                              q_gain=self.q_gain, k_gain=self.k_gain, qk_eps=self.qk_norm_eps, rotation=self.rot,
+                              kpages=cache.kpages, vpages=cache.vpages, group=cache.group, owns=self.source is None,
+                              slopes=self.slopes, rows_hook=hook)

@@ -2,27 +2,31 @@
 spec's `kind` to the class that implements it.
 
 A part is built from its spec alone (sizes and constants are the spec's parameters), declares
-the checkpoint tensors it reads, and is later bound to loaded weights.  No part knows which
-model it is in.  To add a part: subclass the interface, decorate the class with the matching
-`register_*`, and name its kind in a spec; nothing else in the framework changes.
+the checkpoint tensors it reads, is bound to loaded weights, and lays itself down in the native
+plan of the model's step (`emit`, parts/native.py).  No part knows which model it is in.  To add
+a part: subclass the interface, decorate the class with the matching `register_*`, and name its
+kind in a spec; nothing else in the framework changes.
 
   Norm            forward(x, delta, rows) -> normed rows in the activation dtype (adds delta first)
   PositionEncoding  tables and parameters that a mixer hands to its kernels
   Mixer           forward(h, batch, cache) -> delta [N, hidden] (or float32 parts [S, N, hidden]
-                  that the next norm adds in order); may ask for cache pages
-                  (`cache_need`) and per-request state of fixed size (`state_needs`)
+                  that are added in order); may ask for cache pages (`cache_need`) and
+                  per-request state of fixed size (`state_needs`)
   FeedForward     forward(h, batch) -> delta [N, hidden]
-  Block           forward(stream, batch, cache) -> stream (arrangement of the above)
+  Block           emit(plan, caches): the arrangement of a layer's parts, as operations of the plan
 
-Optional fast-path hooks (a part without them simply takes the general path): a norm may offer
-`fold_gain()` (hand its gain over to be multiplied into the following matrices), a mixer or
-feed-forward `fold_input_gain(gain)` and `decode_fused(stream, norm_eps, batch[, cache])`, which
-runs norm + part + residual add for a step of single decoded tokens in a few fused kernels.
+A part written with tensor operations implements `forward` and nothing else: the base class's
+`emit` lays it down as a callback of the native step.  A part with kernels of its own in the
+library overrides `emit` (the built-in ones do); its `forward` then runs the part alone through a
+small plan of its own, the same native code that a whole step takes.
+
+Optional fast-path hooks: a norm may offer `fold_gain()` (hand its gain over to be multiplied into
+the following matrices), a mixer or feed-forward `fold_input_gain(gain)` and `pack_matrices()`.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Callable, Dict, List, Optional, Sequence, Type
+from typing import Callable, Dict, List, Mapping, Optional, Sequence, Type
 
 import torch
 
@@ -42,47 +46,6 @@ class Runtime:
     # up to `fused_decode_rows` single decoded tokens take the parts' fused decode kernels (0: never)
     fold_gains: bool = True
     fused_decode_rows: int = 64
-
-
-@dataclass
-class Stream:
-    """The residual stream between blocks.  `x` is float32 [N, hidden].  `pending` is a delta that
-    has not been added yet (the next norm adds it as it reads x).  `mirror`, when kept, is
-    bfloat16(x) with nothing pending: what the fused decode products read as their input."""
-    x: torch.Tensor
-    pending: Optional[torch.Tensor] = None
-    mirror: Optional[torch.Tensor] = None
-
-    # What every arrangement does with the stream, so that none has to know how deltas travel:
-    def normed(self, norm: "Norm", rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None) -> torch.Tensor:
-        """norm(x + what is pending) in the activation type.  All rows: the pending delta is added
-        into x on the way (one kernel).  With `rows`, only those rows are normed and x stays as it is."""
-        h = norm.forward(self.x, self.pending, rows, n_rows)
-        if rows is None and self.pending is not None:
-            self.pending, self.mirror = None, None
-        return h
-
-    def add(self, delta: torch.Tensor) -> None:
-        """x += delta, lazily: the delta stays pending until the next `normed` or `add` (a delta is
-        [N, hidden] in the activation type, or float32 partial sums [S, N, hidden])."""
-        self.settle()
-        self.pending, self.mirror = delta, None
-
-    def settle(self) -> None:
-        """Adds what is pending into x now."""
-        if self.pending is not None:
-            from .. import ops
-            ops.residual_add(self.x, self.pending)
-            self.pending, self.mirror = None, None
-
-    def with_mirror(self) -> "Stream":
-        """Settles the stream and makes sure that `mirror` = bfloat16(x) exists (one kernel for both)."""
-        if self.pending is not None or self.mirror is None:
-            from .. import ops
-            mirror = torch.empty(self.x.shape, dtype=torch.bfloat16, device=self.x.device)
-            ops.residual_add(self.x, self.pending, mirror)
-            self.pending, self.mirror = None, mirror
-        return self
 
 
 class Part:
@@ -112,17 +75,36 @@ class Part:
         copies in the order its few-row kernels read fastest (`ops.PackedWeight`)."""
 
 
+def _solo_plan(rt: Runtime, hidden: int):
+    """A plan of one part's own, for running it alone."""
+    from .native import NativePlan
+    return NativePlan(rt, hidden)
+
+
 class Norm(Part):
     def __init__(self, spec: NormSpec, width: int):
         self.spec, self.width = spec, width
+
+    def emit(self, plan) -> int:
+        """Lays the norm down in `plan`; returns its number there.  Default: a callback to `forward`."""
+        if type(self).forward is Norm.forward:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        return plan.host_norm(self.forward)
 
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], rows: Optional[torch.Tensor] = None,
                 n_rows: Optional[int] = None) -> torch.Tensor:
         """x (float32 residual stream) += delta (if given and all rows are normed); returns norm(x)
         in the activation dtype.  With `rows` only those rows (of x + delta) are normed.  `delta` is
         [N, width] in the activation dtype, or float32 [S, N, width]: parts that are added in
-        ascending s (a product that was split over its inner dimension)."""
-        raise NotImplementedError
+        ascending s (a product that was split over its inner dimension).  (A norm with `emit` of its
+        own runs alone through a plan of one part.)"""
+        if type(self).emit is Norm.emit:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        solo = getattr(self, "_solo", None)
+        if solo is None:
+            plan = _solo_plan(self.rt, self.width)
+            solo = self._solo = (plan, self.emit(plan))
+        return solo[0].norm_forward(solo[1], x, delta, rows, n_rows)
 
 
 @dataclass
@@ -185,30 +167,78 @@ class Mixer(Part):
         the matrix products: scores and weighted values of an attention; 0 for a mixer without."""
         return 0.0
 
+    def emit(self, plan, cache) -> int:
+        """Lays the mixer down in `plan` over the cache view `cache`; returns its number there.
+        Default: a callback to `forward`."""
+        if type(self).forward is Mixer.forward:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        return plan.host_body(lambda h, batch: self.forward(h, batch, cache), None if cache.kpages is None else cache.group)
+
     def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
-        raise NotImplementedError
+        """The delta of the normed rows h [N, hidden] (a mixer with `emit` of its own runs alone
+        through a plan of one part, kept per cache view)."""
+        if type(self).emit is Mixer.emit:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        solos = self.__dict__.setdefault("_solos", {})
+        solo = solos.get(id(cache))
+        if solo is None:
+            plan = _solo_plan(self.rt, self.hidden)
+            solo = solos[id(cache)] = (plan, self.emit(plan, cache), cache)
+        return solo[0].body_forward(solo[1], h.contiguous(), batch)
 
 
 class FeedForward(Part):
     def __init__(self, spec: FeedForwardSpec, hidden: int):
         self.spec, self.hidden = spec, hidden
 
+    def emit(self, plan) -> int:
+        """Lays the feed-forward down in `plan`; returns its number there.  Default: a callback to `forward`."""
+        if type(self).forward is FeedForward.forward:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        return plan.host_body(lambda h, batch: self.forward(h, batch))
+
     def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
-        raise NotImplementedError
+        if type(self).emit is FeedForward.emit:
+            raise NotImplementedError(f"{type(self).__name__} has neither `forward` nor `emit`")
+        solo = getattr(self, "_solo", None)
+        if solo is None:
+            plan = _solo_plan(self.rt, self.hidden)
+            solo = self._solo = (plan, self.emit(plan))
+        return solo[0].body_forward(solo[1], h.contiguous(), batch)
+
+
+def build_part(spec, hidden: int, layer_index: int) -> Part:
+    """The part that a spec of any of the layer's kinds describes."""
+    if isinstance(spec, NormSpec):
+        return build_norm(spec, hidden)
+    if isinstance(spec, MixerSpec):
+        return build_mixer(spec, hidden, layer_index)
+    if isinstance(spec, FeedForwardSpec):
+        return build_feed_forward(spec, hidden)
+    raise TypeError(f"a layer's parts are norms, mixers and feed-forwards, not {type(spec).__name__}")
 
 
 class Block(Part):
-    """One layer: an arrangement of two norms, a mixer and a feed-forward."""
+    """One layer: its parts by role, as the layer's spec names them (any number of norms, mixers and
+    feed-forwards), and their arrangement, which a subclass lays down in `emit`."""
 
     def __init__(self, spec: LayerSpec, hidden: int, layer_index: int):
-        self.spec = spec
-        self.mixer_norm = build_norm(spec.mixer_norm, hidden)
-        self.mixer = build_mixer(spec.mixer, hidden, layer_index)
-        self.ffn_norm = build_norm(spec.ffn_norm, hidden)
-        self.ffn = build_feed_forward(spec.ffn, hidden)
+        self.spec, self.hidden = spec, hidden
+        self.named: Dict[str, Part] = {role: build_part(ps, hidden, layer_index) for role, ps in spec.parts}
+
+    def __getattr__(self, role: str) -> Part:
+        """`block.mixer`, `block.ffn_norm`, ...: the part of that role."""
+        named = self.__dict__.get("named", {})
+        if role in named:
+            return named[role]
+        raise AttributeError(f"{type(self).__name__} has no attribute or part {role!r}")
 
     def parts(self) -> List[Part]:
-        return [self.mixer_norm, self.mixer, self.ffn_norm, self.ffn]
+        return list(self.named.values())
+
+    def mixers(self) -> Dict[str, Mixer]:
+        """The parts that may own a cache or state, by role, in the spec's order."""
+        return {role: p for role, p in self.named.items() if isinstance(p, Mixer)}
 
     def tensor_decls(self) -> List[TensorDecl]:
         return [d for p in self.parts() for d in p.tensor_decls()]
@@ -221,13 +251,34 @@ class Block(Part):
     def matrices(self) -> List[torch.Tensor]:
         return [m for p in self.parts() for m in p.matrices()]
 
+    def product_shapes(self) -> List[tuple]:
+        return [m for p in self.parts() for m in p.product_shapes()]
+
     def small_tensors(self) -> List[torch.Tensor]:
         return [m for p in self.parts() for m in p.small_tensors()]
 
-    def forward(self, stream: Stream, batch, cache) -> Stream:
-        """Runs the block on the residual stream (updated in place) and returns it, with the
-        block's last delta either added or left pending for the next norm."""
+    def attention_flops(self, keys: float) -> float:
+        return sum(m.attention_flops(keys) for m in self.mixers().values())
+
+    def emit(self, plan, caches: Mapping[str, object]) -> None:
+        """Lays the block down in `plan`: its parts (`part.emit`) and the operations that arrange them
+        (`plan.half`, or `plan.normed` / `plan.apply` / `plan.add` / `plan.drop` in any order).
+        `caches[role]`: the cache view of the mixer of that role."""
         raise NotImplementedError
+
+    def forward(self, x: torch.Tensor, batch, caches: Mapping[str, object]) -> torch.Tensor:
+        """The block alone on the residual rows x [N, hidden] (float32, changed in place): through a plan
+        that holds this block only (kept per set of cache views).  Returns x."""
+        solos = self.__dict__.setdefault("_solos", {})
+        key = tuple(id(c) for c in caches.values())
+        solo = solos.get(key)
+        if solo is None:
+            from .native import NativePlan
+            plan = NativePlan(self.rt, self.hidden)
+            self.emit(plan, caches)
+            solo = solos[key] = (plan, dict(caches))
+        solo[0].step(batch, x_in=x, first_op=0, n_ops=solo[0].op_count(), settle=True)
+        return x
 
 
 # --------------------------------------------------------------------------- registries

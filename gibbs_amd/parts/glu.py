@@ -8,7 +8,6 @@ from typing import List
 import torch
 
 from .. import ops
-from ..ops.linear import linear
 from ..weights.loader import TensorDecl, WeightStore
 from .base import FeedForward, Runtime, register_feed_forward
 
@@ -48,20 +47,6 @@ class GluFeedForward(FeedForward):
         self.p_gate_up = ops.PackedWeight(self.w_gate_up, groups=2)
         self.p_down = ops.PackedWeight(self.w_down)
 
-    def can_decode_fused(self, batch) -> bool:
-        return self.hidden % 8 == 0 and self.inter % 8 == 0
-
-    def decode_fused(self, stream, norm_eps: float, batch) -> None:
-        """norm -> gate/up -> activation in one kernel, down + residual add in another."""
-        act = ops.skinny_glu(stream.mirror, self.p_gate_up or self.w_gate_up, rms_eps=norm_eps, activation=self.activation)
-        ops.skinny_residual(act, self.p_down or self.w_down, stream.x, stream.mirror)
-
-    def emit_native(self, builder, folded: bool) -> bool:
-        builder.glu(w_gate_up=self.w_gate_up, p_gate_up=self.p_gate_up, w_down=self.w_down, p_down=self.p_down,
-                    inter=self.inter, activation=ops.ACTIVATIONS[self.activation],
-                    fusable=folded and self.can_decode_fused(None))
-        return True
-
-    def forward(self, h: torch.Tensor, batch) -> torch.Tensor:
-        gu = linear(h, self.w_gate_up)
-        return linear(ops.glu(gu, self.activation), self.w_down, partial_ok=True, packed=self.p_down)
+    def emit(self, plan) -> int:
+        return plan.glu(w_gate_up=self.w_gate_up, p_gate_up=self.p_gate_up, w_down=self.w_down, p_down=self.p_down,
+                        inter=self.inter, activation=ops.ACTIVATIONS[self.activation])

@@ -2,22 +2,21 @@
 norm and head (arch/families/lfm2.json5:66-95,
 arch/lib/transformer.json5:170-198).
 
-Only the rows whose logits are wanted go through the final norm and the head: the gather comes
-before the norm, as in the reference's `last_row` (transformer.json5:177-192).
+The model owns structure and weights; its step is the native plan that its blocks lay down
+(parts/native.py).  Only the rows whose logits are wanted go through the final norm and the head:
+the gather comes before the norm, as in the reference's `last_row` (transformer.json5:177-192).
 """
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
 from .. import ops
 from ..cache.needs import CacheNeed, StateNeed
 from ..config.spec import ModelSpec
-from ..ops.linear import linear
 from ..weights.loader import TensorDecl, WeightStore
-from .base import Block, Part, Runtime, Stream, build_block, build_norm
-from .block import fused_decode_step
+from .base import Block, Part, Runtime, build_block, build_norm
 
 
 class DecoderModel(Part):
@@ -29,13 +28,19 @@ class DecoderModel(Part):
             if not 0 <= i < len(self.blocks):
                 raise ValueError(f"layer order names layer {i}; the model has {len(self.blocks)}")
         for i, b in enumerate(self.blocks):
-            src = b.mixer.kv_source()
-            if src is not None:
-                if not 0 <= src < len(self.blocks) or self.blocks[src].mixer.cache_need() is None:
+            for mixer in b.mixers().values():
+                src = mixer.kv_source()
+                if src is None:
+                    continue
+                if not 0 <= src < len(self.blocks) or self._cache_owner_role(src) is None:
                     raise ValueError(f"layer {i} reads the cache of layer {src}, which owns none")
                 first_use = spec.order.index(i) if i in spec.order else -1
                 if first_use >= 0 and src not in spec.order[:first_use]:
                     raise ValueError(f"layer {i} runs before layer {src}, whose cache it reads")
+
+    def _cache_owner_role(self, layer: int) -> Optional[str]:
+        """The role of the first mixer of `layer` that owns cache pages."""
+        return next((role for role, m in self.blocks[layer].mixers().items() if m.cache_need() is not None), None)
 
     # ------------------------------------------------------------------ what the model asks for
     def tensor_decls(self) -> List[TensorDecl]:
@@ -48,22 +53,34 @@ class DecoderModel(Part):
             decls.append(TensorDecl(s.head, (s.vocab, s.hidden)))
         return decls
 
-    # Caches belong to runs (entries of the run order), not to layers: a layer that the order
-    # names twice shares its weights between both runs, but each run caches its own keys,
-    # values and state.
+    # Caches belong to the mixers of runs (entries of the run order), not to layers: a layer that the
+    # order names twice shares its weights between both runs, but each run caches its own keys,
+    # values and state.  `cache_owners` lists them, (run, role) in the order they run; what the cache
+    # manager calls a layer is an entry of this list.
+    def cache_owners(self) -> List[Tuple[int, str]]:
+        return [(run, role) for run, i in enumerate(self.spec.order) for role in self.blocks[i].mixers()]
+
+    def _mixer(self, owner: Tuple[int, str]):
+        return self.blocks[self.spec.order[owner[0]]].mixers()[owner[1]]
+
     def cache_needs(self) -> List[Optional[CacheNeed]]:
-        return [self.blocks[i].mixer.cache_need() for i in self.spec.order]
+        return [self._mixer(o).cache_need() for o in self.cache_owners()]
 
     def state_needs(self) -> List[Sequence[StateNeed]]:
-        return [tuple(self.blocks[i].mixer.state_needs()) for i in self.spec.order]
+        return [tuple(self._mixer(o).state_needs()) for o in self.cache_owners()]
 
-    def kv_source_runs(self) -> List[Optional[int]]:
-        """For each run, the earlier run whose pages it reads (the latest run of the layer that
-        its mixer names as `kv_source`), or None."""
+    def kv_sources(self) -> List[Optional[int]]:
+        """For each cache owner, the earlier owner whose pages it reads (the page-owning mixer of the
+        latest run of the layer that its mixer names as `kv_source`), or None."""
+        owners = self.cache_owners()
         out: List[Optional[int]] = []
-        for run, i in enumerate(self.spec.order):
-            src = self.blocks[i].mixer.kv_source()
-            out.append(None if src is None else max(j for j in range(run) if self.spec.order[j] == src))
+        for run, role in owners:
+            src = self._mixer((run, role)).kv_source()
+            if src is None:
+                out.append(None)
+                continue
+            src_run = max(j for j in range(run) if self.spec.order[j] == src)
+            out.append(owners.index((src_run, self._cache_owner_role(src))))
         return out
 
     def bind(self, weights: WeightStore, rt: Runtime) -> None:
@@ -74,20 +91,3 @@ class DecoderModel(Part):
         self.final_norm.bind(weights, rt)
         for b in self.blocks:
             b.bind(weights, rt)
-
-    # ------------------------------------------------------------------ one step
-    def forward(self, batch, caches) -> Optional[torch.Tensor]:
-        """Runs the batch's rows through every layer from the cache (`caches[run]` is the view of
-        run number `run` of the layer order); returns float32 logits [len(logit_rows), vocab]
-        (None if no logits are wanted)."""
-        mirror = None
-        if fused_decode_step(self.rt, batch):
-            # a step of decoded tokens: the fused kernels read the stream's bfloat16 mirror
-            mirror = torch.empty((batch.n_rows, self.spec.hidden), dtype=torch.bfloat16, device=self.rt.device)
-        stream = Stream(ops.embed(self.table, batch.ids, batch.n_rows, mirror=mirror), None, mirror)
-        for run, i in enumerate(self.spec.order):
-            stream = self.blocks[i].forward(stream, batch, caches[run])
-        if batch.n_logits == 0:
-            return None
-        h = stream.normed(self.final_norm, batch.logit_rows, batch.n_logits)
-        return linear(h, self.head, out_dtype=torch.float32, packed=self.head_packed)

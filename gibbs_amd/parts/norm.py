@@ -7,7 +7,6 @@ from typing import List, Optional
 
 import torch
 
-from .. import ops
 from ..weights.loader import FLOAT32, TensorDecl, WeightStore
 from .base import Norm, Runtime, register_norm
 
@@ -27,12 +26,8 @@ class RMSNorm(Norm):
         gain, self.gain = self.gain, None
         return gain
 
-    def forward(self, x, delta, rows=None, n_rows=None):
-        return ops.add_rmsnorm(x, delta, self.gain, self.spec.eps, self.rt.act_dtype, rows, n_rows)
-
     def small_tensors(self):
         return [] if self.gain is None else [self.gain]
 
-    def native_norm(self):
-        """(gain or None, eps) for the native step."""
-        return self.gain, self.spec.eps
+    def emit(self, plan) -> int:
+        return plan.rms_norm(self.gain, self.spec.eps)

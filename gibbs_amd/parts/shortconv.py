@@ -14,7 +14,6 @@ import torch
 
 from .. import ops
 from ..cache.needs import StateNeed
-from ..ops.linear import linear
 from ..weights.loader import FLOAT32, TensorDecl, WeightStore
 from .base import Mixer, Runtime, register_mixer
 
@@ -65,28 +64,10 @@ class ShortConvMixer(Mixer):
         """The preceding norm's gain, multiplied into the columns of the in-projection."""
         self.w_in = (self.w_in.float() * gain[None, :]).to(self.w_in.dtype)
 
-    def can_decode_fused(self, batch) -> bool:
-        return self.hidden % 8 == 0 and self.width % 8 == 0 and self.kernel <= 8
-
     def pack_matrices(self) -> None:
         self.p_in = ops.PackedWeight(self.w_in, groups=3)
         self.p_out = ops.PackedWeight(self.w_out)
 
-    def decode_fused(self, stream, norm_eps: float, batch, cache) -> None:
-        """norm -> in_proj -> gated convolution with its state in one kernel, out_proj + residual
-        add in another."""
-        y = ops.skinny_conv(stream.mirror, self.p_in or self.w_in, self.taps, self.conv_bias, cache.states[STATE], batch.slot,
-                            batch.ctx, rms_eps=norm_eps)
-        ops.skinny_residual(y, self.p_out or self.w_out, stream.x, stream.mirror)
-
-    def emit_native(self, builder, cache, folded: bool) -> bool:
-        builder.short_conv(w_in=self.w_in, p_in=self.p_in, w_out=self.w_out, p_out=self.p_out, taps=self.taps,
-                           bias=self.conv_bias, width=self.width, kernel=self.kernel, state=cache.states[STATE],
-                           fusable=folded and self.can_decode_fused(None))
-        return True
-
-    def forward(self, h: torch.Tensor, batch, cache) -> torch.Tensor:
-        bcx = linear(h, self.w_in)
-        y = ops.shortconv(bcx, self.taps, self.conv_bias, cache.states[STATE], batch.cu, batch.ctx, batch.slot,
-                          batch.n_rows, batch.n_req)
-        return linear(y, self.w_out, partial_ok=True, packed=self.p_out)
+    def emit(self, plan, cache) -> int:
+        return plan.short_conv(w_in=self.w_in, p_in=self.p_in, w_out=self.w_out, p_out=self.p_out, taps=self.taps,
+                               bias=self.conv_bias, width=self.width, kernel=self.kernel, state=cache.states[STATE])

@@ -91,6 +91,6 @@ def prefill_flops(engine, n_tokens: int, n_logit_rows: int = 1, start: int = 0) 
     for i in m.spec.order:
         b = m.blocks[i]
         flops += 2.0 * n_tokens * sum(t.numel() for t in b.matrices())
-        flops += b.mixer.attention_flops(keys)
+        flops += b.attention_flops(keys)
     flops += 2.0 * n_logit_rows * m.head.numel()
     return flops

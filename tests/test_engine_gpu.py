@@ -463,12 +463,44 @@ def test_sequence_of_9000_tokens_in_pages_of_16(tmp_path_factory, dtype):
     check(d, seqs, got, dtype, f"9,000 tokens {dtype}", against_whole=False)
 
 
+def through_callbacks(config):
+    """The same model with every mixer and feed-forward laid down as a callback from the native step into
+    the part's own `forward` (which runs the part alone, through a plan of one part), instead of as a
+    native part of the step: the route that a part written outside the package takes."""
+    import dataclasses
+
+    from gibbs_amd.config import LayerSpec
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.parts import register_arrangement
+    from gibbs_amd.parts.block import PreNormBlock
+
+    @register_arrangement("pre_norm_through_callbacks")
+    class ThroughCallbacks(PreNormBlock):
+        def emit(self, plan, caches):
+            cache = caches["mixer"]
+            mixer = plan.host_body(lambda h, batch: self.mixer.forward(h, batch, cache), None if cache.kpages is None else cache.group)
+            ffn = plan.host_body(lambda h, batch: self.ffn.forward(h, batch))
+            plan.half(self.mixer_norm.emit(plan), mixer)
+            plan.half(self.ffn_norm.emit(plan), ffn)
+
+    spec = config.model_spec()
+    spec = dataclasses.replace(spec, layers=tuple(LayerSpec(l.name, "pre_norm_through_callbacks", parts=l.parts) for l in spec.layers))
+
+    class Wrapped(ArchConfig):
+        def model_spec(self):
+            return spec
+    return Wrapped()
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "B", "C", "D", "M"])
-def test_native_step_equals_stepping_through_the_parts(model_dirs, tmp_path_factory, name, dtype):
-    """The step as one native call queues the kernels that the parts' `forward` would queue, with the
-    same choices: the logits of a mixed schedule (portions, decoded tokens alone and at the head of a
-    step, many rows) are the same bit for bit."""
+def test_parts_as_callbacks_of_the_native_step(model_dirs, tmp_path_factory, name, dtype):
+    """Every kernel choice is made in one place, the native step; a part run alone goes through the
+    same code.  So a model whose mixers and feed-forwards are callbacks into the parts' own `forward`
+    gives, on the general path, the logits of the model laid down natively: in 32-bit bit for bit over
+    a mixed schedule (portions, decoded tokens alone and at the head of a step, many rows); in
+    bfloat16 up to the rounding of a delta that the native step hands on as float32 partial sums."""
+    from gibbs_amd.config import config_from_dict, read_config_json
     d = model_dirs[name] if name in model_dirs else H.make_model_dir(str(tmp_path_factory.mktemp("native")), name, seed=8, std=0.05)
     vocab = H.TINY[name]["vocab_size"]
     rng = np.random.default_rng(11)
@@ -479,10 +511,15 @@ def test_native_step_equals_stepping_through_the_parts(model_dirs, tmp_path_fact
     steps.append(([("long", long[200:203], [2]), ("q0", [1, 2], [1])], ["q0"]))
     steps += [([("long", [t], [0])], []) for t in long[203:240]]
     got = {}
-    for native in (True, False):
-        eng = make_engine(d, dtype, max_tokens=1024, max_requests=5, native_step=native)
-        assert (eng.plan is not None) == native
-        got[native] = run_steps(eng, steps)
+    for callbacks in (False, True):
+        kw = {}
+        if callbacks:
+            kw["config"] = through_callbacks(config_from_dict(read_config_json(d)))
+        eng = make_engine(d, dtype, max_tokens=1024, max_requests=5, fused_decode_rows=0, **kw)
+        got[callbacks] = run_steps(eng, steps)
     assert got[True].keys() == got[False].keys()
     for key in got[True]:
-        assert np.array_equal(got[True][key], got[False][key]), f"{name} {dtype}: place {key} differs between the two ways"
+        if dtype == "float32":
+            assert np.array_equal(got[True][key], got[False][key]), f"{name} {dtype}: place {key} differs between the two ways"
+        else:
+            H.assert_close(got[True][key], got[False][key], dtype, f"{name}: place {key}, callbacks vs native parts", tol=H.consistency(dtype))

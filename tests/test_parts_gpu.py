@@ -176,13 +176,13 @@ def test_glu_part(name, dtype):
 
 def run_block(block, xs, chunks, dtype, page_size=8):
     """Feeds residual rows xs (one [T_r, hidden] array per request) through a bound block in the given
-    chunks per step; returns the stream after the block (x with whatever was left pending added)."""
+    chunks per step; returns the stream after the block, and how many steps took the fused decode
+    kernels in both halves."""
     from gibbs_amd.cache import CacheManager, DeviceCache
     from gibbs_amd.engine.batch import BatchStager
-    from gibbs_amd.parts.base import Stream
     cm = CacheManager([block.mixer.cache_need()], [tuple(block.mixer.state_needs())], page_size, 64, 4)
     dc = DeviceCache(cm, dtype, torch.device(DEV))
-    view = dc.layer_view(0)
+    views = {"mixer": dc.layer_view(0)}
     stager = BatchStager(torch.device(DEV))
     outs = {r: [] for r in range(len(xs))}
     fused_steps = 0
@@ -202,13 +202,9 @@ def run_block(block, xs, chunks, dtype, page_size=8):
                              np.array([cm.slot(r) for r in rids], np.int32), np.zeros(0, np.int32),
                              [cm.block_table(rids, g) for g in range(cm.n_groups)])
         x = torch.tensor(np.concatenate([xs[r][a:b] for r, a, b in step]), dtype=torch.float32, device=DEV).contiguous()
-        out = block.forward(Stream(x=x), batch, view)
-        fused_steps += out.pending is None
-        y = out.x.clone()
-        if out.pending is not None:
-            pend = out.pending.sum(0) if out.pending.dim() == 3 else out.pending
-            y += pend.float()
-        y = y.cpu().numpy()
+        y = block.forward(x, batch, views).cpu().numpy()
+        plan = next(iter(block._solos.values()))[0]
+        fused_steps += plan.last_fused() == 2
         for i, (r, a, b) in enumerate(step):
             outs[r].append(y[cu[i]:cu[i + 1]])
             cm.commit(r, b - a)
@@ -594,6 +590,7 @@ def test_toy_mixer_with_state_registers_builds_and_steps(name, dtype, tmp_path):
     assert json.load(open(os.path.join(folder, "config.json")))["mixers"] == ["ema", "attn", "ema"]
     eng = Engine(folder, dtype=name, max_tokens=128, max_requests=2, page_size=8)     # the class is chosen by config.json
     assert [type(b.mixer).__name__ for b in eng.model.blocks] == ["ToyEma", "AttentionMixer", "ToyEma"]
+    assert eng.plan.op_count() == 6, "the toy mixer is a part of the native step's program like any other"
     assert set(eng.cache.state_layout) == {(0, "ema"), (2, "ema")}
     weights, _ = P.load_model_dir(folder)
     seqs = {"a": H.tokens(1, 30, 83), "b": H.tokens(2, 17, 83)}
@@ -975,12 +972,12 @@ def test_positions_that_are_no_rotation_and_values_wider_than_keys(name, dtype, 
         H.assert_close(np.concatenate(got[r]), wide_plain(cfg, weights, ids), name, f"toy positions / wide values request {r}")
 
 
-# --------------------------------------------------------------------------- another arrangement of a block's parts
-def test_an_arrangement_from_outside_uses_the_stream_protocol(tmp_path):
+# --------------------------------------------------------------------------- other arrangements of a block's parts
+def test_an_arrangement_from_outside_is_a_program_of_the_native_step(tmp_path):
     """A block in which mixer and feed-forward read the same normed rows and both add to the stream
-    (x += mixer(norm(x)) + ffn(norm(x))), registered from here: it hands its deltas to the residual
-    stream through `Stream.normed` / `Stream.add` and knows nothing of how they travel (pending
-    deltas, float32 partial sums, the bfloat16 mirror).  Both precisions, portions and single tokens."""
+    (x += mixer(norm(x)) + ffn(norm(x))), registered from here: one norm and two bodies by role, laid
+    down as norm, body, body, add, add, drop operations of the native step.  It knows nothing of how
+    deltas travel (pending deltas, float32 partial sums).  Both precisions, portions and single tokens."""
     from gibbs_amd import Engine, Entry
     from gibbs_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
                                   register_architecture)
@@ -990,14 +987,13 @@ def test_an_arrangement_from_outside_uses_the_stream_protocol(tmp_path):
 
     @register_arrangement("toy_parallel")
     class Parallel(Block):
-        def parts(self):
-            return [self.mixer_norm, self.mixer, self.ffn]          # (one norm: the second is not used)
-
-        def forward(self, stream, batch, cache):
-            h = stream.normed(self.mixer_norm)
-            stream.add(self.mixer.forward(h, batch, cache))
-            stream.add(self.ffn.forward(h, batch))
-            return stream
+        def emit(self, plan, caches):
+            h = plan.normed(self.norm.emit(plan))
+            a = plan.apply(self.mixer.emit(plan, caches["mixer"]), h)
+            m = plan.apply(self.ffn.emit(plan), h)
+            plan.add(a)
+            plan.add(m)
+            plan.drop(h)
 
     class ParallelConfig(ArchConfig):
         architecture = "ToyParallelForCausalLM"
@@ -1025,8 +1021,8 @@ def test_an_arrangement_from_outside_uses_the_stream_protocol(tmp_path):
                                       {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o"},
                                       PositionSpec("rope", {"theta": 1e4, "rotary_dim": 16, "precision": "f32"}))
                 ffn = FeedForwardSpec("glu", {"inter": c["ff"], "activation": "silu"}, {"gate": f"{p}.g", "up": f"{p}.u", "down": f"{p}.d"})
-                norm = NormSpec("rms", c["eps"], f"{p}.n")
-                layers.append(LayerSpec(p, "toy_parallel", norm, mixer, norm, ffn))
+                layers.append(LayerSpec(p, "toy_parallel", parts=[("norm", NormSpec("rms", c["eps"], f"{p}.n")), ("mixer", mixer),
+                                                                  ("ffn", ffn)]))
             return ModelSpec(self.architecture, c["width"], c["vocab"], tuple(layers), tuple(range(len(layers))), "tok",
                              NormSpec("rms", c["eps"], "out_norm"), None, 128)
     register_architecture("ToyParallelForCausalLM", ParallelConfig)
@@ -1053,7 +1049,112 @@ def test_an_arrangement_from_outside_uses_the_stream_protocol(tmp_path):
     want = P.linear(P.rms_norm(x, w["out_norm"], cfg["eps"]), w["tok"])
     for name in ("float32", "bfloat16"):
         eng = Engine(folder, dtype=name, max_tokens=128, max_requests=1, page_size=8)
-        assert eng.plan is None and [type(b).__name__ for b in eng.model.blocks] == ["Parallel"] * 3
+        assert [type(b).__name__ for b in eng.model.blocks] == ["Parallel"] * 3
+        assert eng.plan.op_count() == 3 * 6, "the step is the native program that the blocks laid down"
         got = [eng.step([Entry("r", ids[a:b], list(range(b - a)))]).cpu().numpy()
                for a, b in [(0, 21), (21, 23), (23, 24), (24, 25), (25, 49), (49, 50)]]
         H.assert_close(np.concatenate(got), want, name, f"parallel arrangement {name}")
+
+
+def test_layers_with_two_mixers_and_layers_without_a_feed_forward(tmp_path):
+    """A layer is whatever parts its spec names, by role: here layers of the kind "mix" hold a norm and
+    TWO mixers that read the same normed rows (a short convolution with its state and an attention with
+    its cache pages: two cache owners in one layer) and no feed-forward; layers of the kind "ff" hold a
+    norm and a feed-forward and no mixer.  The arrangement, registered from here, lays down whichever
+    parts a layer has.  Cache manager, step function and scheduler take the model as it is."""
+    from gibbs_amd import Engine, Entry, generate
+    from gibbs_amd.config import (FeedForwardSpec, LayerSpec, MixerSpec, ModelSpec, NormSpec, PositionSpec,
+                                  register_architecture)
+    from gibbs_amd.config.base import ArchConfig
+    from gibbs_amd.parts import Block, DecoderModel, register_arrangement
+    from gibbs_amd.weights import write_random_model
+
+    @register_arrangement("toy_all_of_them")
+    class AllOfThem(Block):
+        """x += sum of every body's delta of norm(x)."""
+        def emit(self, plan, caches):
+            h = plan.normed(self.norm.emit(plan))
+            deltas = [plan.apply(part.emit(plan, caches[role]) if role in caches else part.emit(plan), h)
+                      for role, part in self.named.items() if role != "norm"]
+            for d in deltas:
+                plan.add(d)
+            plan.drop(h)
+
+    class MixConfig(ArchConfig):
+        architecture = "ToyTwoMixersForCausalLM"
+
+        def __init__(self, cfg):
+            self.cfg = dict(cfg)
+
+        @classmethod
+        def from_dict(cls, cfg, tensors=None):
+            return cls(cfg)
+
+        def to_dict(self):
+            return dict(self.cfg)
+
+        def model_spec(self):
+            c, layers = self.cfg, []
+            for i, kind in enumerate(c["layers"]):
+                p = f"l{i}"
+                parts = [("norm", NormSpec("rms", c["eps"], f"{p}.n"))]
+                if kind == "mix":
+                    parts.append(("local", MixerSpec("short_conv", {"width": c["width"], "kernel": 4, "bias": True},
+                                                     {"in_proj": f"{p}.in", "conv": f"{p}.taps", "out_proj": f"{p}.out",
+                                                      "conv_bias": f"{p}.cb"})))
+                    parts.append(("global", MixerSpec("attention", {"heads": 4, "kv_heads": 2, "head_dim": 16, "scale": 0.25,
+                                                                     "qk_norm": None, "window": None},
+                                                      {"q_proj": f"{p}.q", "k_proj": f"{p}.k", "v_proj": f"{p}.v", "out_proj": f"{p}.o"},
+                                                      PositionSpec("rope", {"theta": 1e4, "rotary_dim": 16, "precision": "f32"}))))
+                else:
+                    parts.append(("ffn", FeedForwardSpec("glu", {"inter": c["ff"], "activation": "silu"},
+                                                         {"gate": f"{p}.g", "up": f"{p}.u", "down": f"{p}.d"})))
+                layers.append(LayerSpec(p, "toy_all_of_them", parts=parts))
+            return ModelSpec(self.architecture, c["width"], c["vocab"], tuple(layers), tuple(range(len(layers))), "tok",
+                             NormSpec("rms", c["eps"], "out_norm"), None, 128)
+    register_architecture("ToyTwoMixersForCausalLM", MixConfig)
+    cfg = {"architectures": ["ToyTwoMixersForCausalLM"], "width": 64, "ff": 96, "vocab": 67, "layers": ["mix", "ff", "mix"],
+           "eps": 1e-5}
+    config = MixConfig(cfg)
+    folder = str(tmp_path / "two_mixers")
+    write_random_model(folder, config, DecoderModel(config.model_spec()).tensor_decls(), seed=3, std=0.2, gain_std=0.2, bias_std=0.1)
+    w, _ = P.load_model_dir(folder)
+
+    def plain(ids):
+        T = len(ids)
+        x = P.embedding(w["tok"], ids)
+        for i, kind in enumerate(cfg["layers"]):
+            p = f"l{i}"
+            h = P.rms_norm(x, w[f"{p}.n"], cfg["eps"])
+            if kind == "mix":
+                inv = P.rope_inv_freq(16, 1e4)
+                q = P.rope_half_split(P.linear(h, w[f"{p}.q"]).reshape(T, 4, 16), range(T), inv)
+                k = P.rope_half_split(P.linear(h, w[f"{p}.k"]).reshape(T, 2, 16), range(T), inv)
+                att = P.linear(P.causal_attention(q, k, P.linear(h, w[f"{p}.v"]).reshape(T, 2, 16), 0.25).reshape(T, 64), w[f"{p}.o"])
+                x = x + P.short_conv_mixer(h, w[f"{p}.in"], w[f"{p}.taps"], w[f"{p}.out"], w[f"{p}.cb"]) + att
+            else:
+                x = x + P.swiglu_ffn(h, w[f"{p}.g"], w[f"{p}.u"], w[f"{p}.d"])
+        return P.linear(P.rms_norm(x, w["out_norm"], cfg["eps"]), w["tok"])
+    seqs = {"a": H.tokens(8, 45, 67), "b": H.tokens(9, 20, 67)}
+    steps = [[("a", 0, 17)], [("a", 17, 19), ("b", 0, 9)], [("a", 19, 20), ("b", 9, 10)], [("a", 20, 21), ("b", 10, 11)],
+             [("a", 21, 44), ("b", 11, 12)], [("a", 44, 45), ("b", 12, 20)]]
+    for name in ("float32", "bfloat16"):
+        eng = Engine(folder, dtype=name, max_tokens=128, max_requests=2, page_size=8)
+        # two cache owners in each "mix" layer: the convolution's state and the attention's pages
+        assert eng.model.cache_owners() == [(0, "local"), (0, "global"), (2, "local"), (2, "global")]
+        assert eng.cache.group_layers == [[1, 3]] and set(eng.cache.state_layout) == {(0, "conv"), (2, "conv")}
+        got = {}
+        for step in steps:
+            out = eng.step([Entry(r, seqs[r][a:b], list(range(b - a))) for r, a, b in step]).cpu().numpy()
+            at = 0
+            for r, a, b in step:
+                got.setdefault(r, []).append(out[at:at + b - a]); at += b - a
+        for r, ids in seqs.items():
+            H.assert_close(np.concatenate(got[r]), plain(ids), name, f"two mixers in a layer, request {r}, {name}")
+        eng.release("a"); eng.release("b")
+        if name == "float32":
+            out = generate(eng, [seqs["b"][:7]], max_tokens=6, temperature=0.0, ignore_eos=True)[0].tokens
+            seq = list(seqs["b"][:7])
+            for t in out:
+                assert t == P.argmax_first(plain(seq)[-1])
+                seq.append(t)
