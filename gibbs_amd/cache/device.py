@@ -23,7 +23,12 @@ class LayerCache:
 class DeviceCache:
     """Keys and values of a group are laid out [layer of group, page, kv head, slot in page, head_dim]
     (values with their own head size) in the cache dtype (the activation dtype of the run); every
-    group has as many pages as its pool; states are float32."""
+    group has as many pages as its pool; states are float32.
+
+    Behind the pool's pages every group holds one more page, and behind the requests' slots the arena
+    one more slot, that the cache manager never hands out (`scratch_page`, `scratch_slot`): rows of a
+    batch that stand for no request (the padding of a captured decode loop made for more rows than
+    are live) write their keys, values and state there, where no request reads."""
 
     def __init__(self, manager: CacheManager, cache_dtype: torch.dtype, device: torch.device):
         self.manager = manager
@@ -32,11 +37,13 @@ class DeviceCache:
         self.kpages: List[torch.Tensor] = []
         self.vpages: List[torch.Tensor] = []
         for g, need in enumerate(manager.group_needs):
-            lead = (len(manager.group_layers[g]), manager.pools[g].num_pages, need.kv_heads, manager.page_size)
+            lead = (len(manager.group_layers[g]), manager.pools[g].num_pages + 1, need.kv_heads, manager.page_size)
             self.kpages.append(torch.zeros(lead + (need.head_dim,), dtype=cache_dtype, device=device))
             self.vpages.append(torch.zeros(lead + (need.value_dim,), dtype=cache_dtype, device=device))
-        self.arena = torch.zeros((manager.max_requests, max(1, manager.slot_floats)),
+        self.arena = torch.zeros((manager.max_requests + 1, max(1, manager.slot_floats)),
                                  dtype=torch.float32, device=device)
+        self.scratch_slot = manager.max_requests
+        self.scratch_page = [manager.pools[g].num_pages for g in range(len(manager.group_needs))]
 
     def nbytes(self) -> int:
         return sum(p.numel() * p.element_size() for p in self.kpages + self.vpages) + self.arena.numel() * 4

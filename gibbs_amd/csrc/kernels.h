@@ -62,7 +62,7 @@ int gibbs_sample(const float* logits, int* out, int M, int V, long ld, const flo
                  const int* top_k, const float* u, hipStream_t stream);
 int gibbs_decode_tail(const float* logits, int V, long ld, int* ids, int* pos, int* ctx, int* log, int* steps, int n,
                       int capacity, float* u, const float* u_all, const void* table, int table_dtype, int vocab, int hidden,
-                      float* x, void* mirror, hipStream_t stream);
+                      float* x, void* mirror, const int* live, hipStream_t stream);
 }
 
 // Inside the library only: gibbs_skinny_store with the output's type given (bfloat16 or float32); what

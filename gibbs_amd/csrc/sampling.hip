@@ -295,19 +295,24 @@ GIBBS_EXPORT int gibbs_repetition_penalty(float* logits, int M, int V, long ld, 
 // loaded, and the token's embedding is written as the row of the next step's residual stream (and of its
 // bfloat16 mirror), so that the next step starts at its first layer.
 //   log[steps[i] * n + i] = ids[i];  pos[i] += 1;  ctx[i] += 1;  u[i] = u_all[(steps[i] + 1) * n + i];  steps[i] += 1
+// A row with live[i] == 0 stands for no request (the padding of a loop made for more rows than are live):
+// nothing of it is logged or moves on; it only gets the embedding of the token it holds again, so that its
+// residual row, which the step updated in place, starts the next step from the same finite values.
 template <typename T>
 __global__ __launch_bounds__(THREADS) void decode_tail_kernel(const float* __restrict__ logits, int V, long ld,
                                                               int* __restrict__ ids, int* __restrict__ pos, int* __restrict__ ctx,
                                                               int* __restrict__ log, int* __restrict__ steps, int n, int capacity,
                                                               float* __restrict__ u, const float* __restrict__ u_all,
                                                               const T* __restrict__ table, int vocab, int hidden,
-                                                              float* __restrict__ x, bf16* __restrict__ mirror) {
+                                                              float* __restrict__ x, bf16* __restrict__ mirror,
+                                                              const int* __restrict__ live) {
   __shared__ float sv[THREADS / WAVE];
   __shared__ int si[THREADS / WAVE];
   __shared__ int s_token;
   const int i = blockIdx.x;
+  const bool padding = live && live[i] == 0;
   int token = 0;
-  if (logits) {
+  if (logits && !padding) {
     const float* row = logits + (size_t)i * ld;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
@@ -318,14 +323,16 @@ __global__ __launch_bounds__(THREADS) void decode_tail_kernel(const float* __res
     token = (bi == 0x7fffffff) ? 0 : bi;
   }
   if (threadIdx.x == 0) {
-    if (logits) ids[i] = token;
+    if (logits && !padding) ids[i] = token;
     else token = ids[i];
-    const int step = steps[i];
-    if (step < capacity) log[(size_t)step * n + i] = token;
-    pos[i] += 1;
-    ctx[i] += 1;
-    if (u && step + 1 < capacity) u[i] = u_all[(size_t)(step + 1) * n + i];
-    steps[i] = step + 1;
+    if (!padding) {
+      const int step = steps[i];
+      if (step < capacity) log[(size_t)step * n + i] = token;
+      pos[i] += 1;
+      ctx[i] += 1;
+      if (u && step + 1 < capacity) u[i] = u_all[(size_t)(step + 1) * n + i];
+      steps[i] = step + 1;
+    }
     s_token = token;
   }
   if (!x) return;
@@ -342,20 +349,20 @@ __global__ __launch_bounds__(THREADS) void decode_tail_kernel(const float* __res
 
 // logits: [n, V] float32 (row stride ld) or null (ids hold the tokens); steps: [n] steps done per row; u, u_all:
 // draws (or null); table: [vocab, hidden] in table_dtype; x: [n, hidden] float32 and mirror: [n, hidden]
-// bfloat16 for the next step (or null: no embedding).
+// bfloat16 for the next step (or null: no embedding); live: [n], 0 for rows that stand for no request (or null: all do).
 GIBBS_EXPORT int gibbs_decode_tail(const float* logits, int V, long ld, int* ids, int* pos, int* ctx, int* log, int* steps,
                                    int n, int capacity, float* u, const float* u_all, const void* table, int table_dtype,
-                                   int vocab, int hidden, float* x, void* mirror, hipStream_t stream) {
+                                   int vocab, int hidden, float* x, void* mirror, const int* live, hipStream_t stream) {
   GIBBS_REQUIRE(n > 0 && capacity > 0, "decode_tail: batch %d, log of %d steps", n, capacity);
   GIBBS_REQUIRE(!logits || (V > 0 && ld >= V), "decode_tail: bad logits V=%d ld=%ld", V, ld);
   GIBBS_REQUIRE(!x || (table && hidden > 0 && vocab > 0), "decode_tail: an embedding needs the token table");
   GIBBS_REQUIRE(!u || u_all, "decode_tail: draws without their table");
   if (table_dtype == GIBBS_F32)
     decode_tail_kernel<float><<<n, THREADS, 0, stream>>>(logits, V, ld, ids, pos, ctx, log, steps, n, capacity, u, u_all,
-                                                         (const float*)table, vocab, hidden, x, (bf16*)mirror);
+                                                         (const float*)table, vocab, hidden, x, (bf16*)mirror, live);
   else if (table_dtype == GIBBS_BF16)
     decode_tail_kernel<bf16><<<n, THREADS, 0, stream>>>(logits, V, ld, ids, pos, ctx, log, steps, n, capacity, u, u_all,
-                                                        (const bf16*)table, vocab, hidden, x, (bf16*)mirror);
+                                                        (const bf16*)table, vocab, hidden, x, (bf16*)mirror, live);
   else
     return gibbs_fail("decode_tail: unknown table dtype %d", table_dtype);
   GIBBS_LAUNCH_STATUS("decode_tail");

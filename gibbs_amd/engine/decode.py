@@ -49,14 +49,20 @@ def capture(graph: "torch.cuda.CUDAGraph"):
 class DecodeLoop:
     def __init__(self, engine: Engine, rids: Sequence[Hashable], last_tokens: Sequence[int],
                  params: Optional[Sequence[SamplingParams]] = None, use_graph: bool = True,
-                 max_steps: int = 2048, first_index: Optional[Sequence[int]] = None):
+                 max_steps: int = 2048, first_index: Optional[Sequence[int]] = None, rows: Optional[int] = None):
         """`rids`: live requests whose prompts are cached; `last_tokens`: the token each one feeds
         next (sampled from its last logits).  `params`: per-request sampling (default greedy);
-        `first_index`: for sampled requests, the output index of their next token (for the draws)."""
+        `first_index`: for sampled requests, the output index of their next token (for the draws).
+        `rows`: make the loop (its static buffers and captured graphs) for this many rows, of which
+        the requests take the first: the others are padding that stands for no request (it reads and
+        writes the cache's scratch page and slot, and nothing of it is logged), so that one loop serves
+        every number of live requests up to `rows` (the reference's decode needs no set-up per batch
+        size either, src/scheduler/mod.rs:1376-1487)."""
         self.engine = engine
-        self.n = len(rids)
-        if self.n == 0:
+        if len(rids) == 0:
             raise StepError("a decode loop needs at least one request")
+        self.padded = rows is not None
+        self.n = max(int(rows or 0), len(rids))
         self.use_graph = use_graph
         self.capacity = max_steps
         self.graph: Optional[torch.cuda.CUDAGraph] = None          # one step
@@ -90,6 +96,7 @@ class DecodeLoop:
             q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True)
         self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
         self.counter = torch.zeros(b, dtype=torch.int32, device=dev)          # steps done, per row
+        self.live_mask = torch.zeros(b, dtype=torch.int32, device=dev) if self.padded else None   # 0: a row of padding
         # native step: the rows of the residual stream (and their bfloat16 mirror) live here from one step to
         # the next; the end of a step writes the next tokens' embeddings into them
         hidden = engine.spec.hidden
@@ -105,32 +112,38 @@ class DecodeLoop:
     def rebind(self, rids: Sequence[Hashable], last_tokens: Sequence[int],
                params: Optional[Sequence[SamplingParams]] = None, first_index: Optional[Sequence[int]] = None) -> None:
         """Points the loop (and its captured graph, which only knows the static buffers) at another
-        set of as many live requests; greedy loops take greedy requests only."""
+        set of live requests: as many as the loop was made for, or, for a padded loop, at most as many
+        (the rows behind them become padding); greedy loops take greedy requests only."""
         engine, b = self.engine, self.n
         cm = engine.cache
-        if len(rids) != b or len(last_tokens) != b:
-            raise StepError(f"this decode loop was made for {b} requests with one last token each")
+        k = len(rids)
+        if len(last_tokens) != k or k == 0 or k > b or (k != b and not self.padded):
+            raise StepError(f"this decode loop was made for {'up to ' if self.padded else ''}{b} requests with one last token each")
         for rid in rids:
             if rid not in cm:
                 raise StepError(f"request {rid!r} is not live")
         self.rids = list(rids)
-        self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * b
+        self.params = list(params) if params is not None else [SamplingParams(temperature=0.0)] * k
         if self.greedy != all(p.greedy for p in self.params):
             raise StepError("a decode loop is captured either for greedy or for sampled requests")
         if any(p.penalises for p in self.params):
             raise StepError("a repetition penalty reads the recent tokens on the host: such requests step through the scheduler")
-        self.index = list(first_index) if first_index is not None else [0] * b
+        self.index = list(first_index) if first_index is not None else [0] * k
         h = self._host
-        h[self._sec[0]] = np.asarray(last_tokens, dtype=np.int32)
-        lens = np.array([cm.tokens(r) for r in self.rids], dtype=np.int32)
+        # (rows of padding: token 0 at position 0 with nothing cached, in the scratch slot and page)
+        pad = lambda values, fill: np.concatenate([np.asarray(values, dtype=np.int32), np.full(b - k, fill, dtype=np.int32)])
+        h[self._sec[0]] = pad(last_tokens, 0)
+        lens = pad([cm.tokens(r) for r in self.rids], 0)
         h[self._sec[1]] = lens
         h[self._sec[2]] = np.arange(b)
         h[self._sec[3]] = np.arange(b + 1)
         h[self._sec[4]] = lens
-        h[self._sec[5]] = [cm.slot(r) for r in self.rids]
+        h[self._sec[5]] = pad([cm.slot(r) for r in self.rids], engine.device_cache.scratch_slot)
         h[self._sec[6]] = np.arange(b)
         self._fill_tables()
         self._dev.copy_(torch.from_numpy(h))
+        if self.padded:
+            self.live_mask.copy_(torch.from_numpy(pad([1] * k, 0)))
         self.batch.ctx_lens, self.batch.slots = lens.tolist(), h[self._sec[5]].tolist()
         # The longest sequence the loop can reach before it is bound again: kernels choose their key
         # slices by it, and a captured graph keeps that choice, so graphs captured for a shorter bound
@@ -145,10 +158,10 @@ class DecodeLoop:
         self._prepared = None
         self._embed()
         if not self.greedy:
-            dev = engine.device
-            self.temperature.copy_(torch.tensor([p.resolved_temperature for p in self.params], dtype=torch.float32))
-            self.top_p.copy_(torch.tensor([p.resolved_top_p for p in self.params], dtype=torch.float32))
-            self.top_k.copy_(torch.tensor([p.top_k for p in self.params], dtype=torch.int32))
+            fill = [1.0] * (b - k)
+            self.temperature.copy_(torch.tensor([p.resolved_temperature for p in self.params] + fill, dtype=torch.float32))
+            self.top_p.copy_(torch.tensor([p.resolved_top_p for p in self.params] + fill, dtype=torch.float32))
+            self.top_k.copy_(torch.tensor([p.top_k for p in self.params] + [1] * (b - k), dtype=torch.int32))
 
     def _embed(self) -> None:
         """The embeddings of the tokens in `ids` into the loop's residual rows (the first step after binding;
@@ -157,9 +170,11 @@ class DecodeLoop:
 
     # ------------------------------------------------------------------ host side
     def _fill_tables(self) -> None:
-        cm = self.engine.cache
+        cm, k = self.engine.cache, len(self.rids)
         for g, w in enumerate(self.width):
-            self._host[self._sec[7 + g]] = cm.block_table(self.rids, g, w).reshape(-1)
+            table = np.full((self.n, w), self.engine.device_cache.scratch_page[g], dtype=np.int32)   # (padding: every position there)
+            table[:k] = cm.block_table(self.rids, g, w)
+            self._host[self._sec[7 + g]] = table.reshape(-1)
 
     def _reserve(self, n_steps: int) -> None:
         cm = self.engine.cache
@@ -190,11 +205,12 @@ class DecodeLoop:
         logits = self.engine.forward(b, self._workspace, self.x, self.mirror)
         table = self.engine.model.table
         if self.greedy:
-            ops.decode_tail(logits, b.ids, b.pos, b.ctx, self.log, self.counter, None, None, self.n, table, self.x, self.mirror)
+            ops.decode_tail(logits, b.ids, b.pos, b.ctx, self.log, self.counter, None, None, self.n, table, self.x, self.mirror,
+                            self.live_mask)
         else:
             ops.sample(logits, self.temperature, self.top_p, self.top_k, self.u, out=b.ids)
             ops.decode_tail(None, b.ids, b.pos, b.ctx, self.log, self.counter, self.u, self.u_all, self.n, table, self.x,
-                            self.mirror)
+                            self.mirror, self.live_mask)
 
     def prepare(self, n_steps: int) -> None:
         """Everything a `run(n_steps)` needs before its first replay, so that a caller who times
@@ -214,7 +230,7 @@ class DecodeLoop:
         if self.greedy:
             return
         rows = np.array([[uniform(p.seed, request_key(r), self.index[i] + self.steps_done + s)
-                          for i, (r, p) in enumerate(zip(self.rids, self.params))]
+                          for i, (r, p) in enumerate(zip(self.rids, self.params))] + [0.5] * (self.n - len(self.rids))
                          for s in range(n_steps)], dtype=np.float32)
         self.u_all[self.steps_done:self.steps_done + n_steps].copy_(torch.from_numpy(rows))
         self.u.copy_(self.u_all[self.steps_done])
@@ -279,4 +295,4 @@ class DecodeLoop:
         """Tokens sampled since the loop was bound (or only by the last `last` steps), per request
         (row s of the log is what step s sampled)."""
         first = 0 if last is None else self.steps_done - last
-        return self.log[first:self.steps_done].cpu().numpy().T.tolist()
+        return self.log[first:self.steps_done, :len(self.rids)].cpu().numpy().T.tolist()

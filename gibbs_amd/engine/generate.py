@@ -49,9 +49,17 @@ class GenerationStats:
         return self.decode_tokens / max(self.decode_seconds, 1e-9)
 
 
-# a burst shorter than this does not get a decode loop (and captured graphs) of its own: requests
-# that finish one after another would otherwise have a loop made for every batch size on the way down
+# a burst shorter than this does not get a decode loop (and captured graphs) made for it
 MIN_STEPS_FOR_NEW_LOOP = 8
+# Rows that decode loops are made for: a burst of n requests runs in the loop of the next size up, its other
+# rows being padding, so that requests that finish one after another stay on captured graphs all the way down
+# instead of having a loop made for every batch size.  The sizes are where the decode step's time steps up
+# (its kernels change shape beyond 8, 16, 32 and 48 rows); beyond 64 rows, multiples of 32.
+LOOP_ROWS = (1, 2, 4, 8, 16, 32, 48, 64)
+
+
+def loop_rows(n: int) -> int:
+    return next((r for r in LOOP_ROWS if r >= n), -(-n // 32) * 32)
 
 
 class Generator:
@@ -98,13 +106,13 @@ class Generator:
             return None                                     # the penalty reads the recent tokens on the host
         last = [s.output_tokens[-1] for s in seqs]
         index = [len(s.output_tokens) for s in seqs]
-        key = (len(seqs), greedy)
+        key = (loop_rows(len(seqs)), greedy)
         try:
             loop = self._loops.get(key)
             if loop is None and n < MIN_STEPS_FOR_NEW_LOOP:
                 return None                                 # capturing graphs for so few steps costs more than it saves
             if loop is None:
-                loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index)
+                loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index, rows=key[0])
             elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:
                 loop.rebind(rids, last, params, index)
             else:

@@ -658,12 +658,16 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
 def decode_tail(logits: Optional[torch.Tensor], ids: torch.Tensor, pos: torch.Tensor, ctx: torch.Tensor, log: torch.Tensor,
                 steps: torch.Tensor, u: Optional[torch.Tensor], u_all: Optional[torch.Tensor], n: int,
                 table: Optional[torch.Tensor] = None, x: Optional[torch.Tensor] = None,
-                mirror: Optional[torch.Tensor] = None) -> None:
+                mirror: Optional[torch.Tensor] = None, live: Optional[torch.Tensor] = None) -> None:
     """End of a decode step on the device, one kernel: with `logits` the rows' next tokens are their first
     largest logits (else `ids` hold them already); the tokens are logged (log[steps[i], i]), pos and ctx move
     on by one, the next draws are loaded, steps[i] counts; with `table` and `x` the tokens' embeddings become
-    the rows of the next step's residual stream x [n, hidden] (float32) and of its bfloat16 `mirror`."""
-    require_cuda(logits, ids, pos, ctx, log, steps, u, u_all, table, x, mirror)
+    the rows of the next step's residual stream x [n, hidden] (float32) and of its bfloat16 `mirror`.  `live`
+    (int32 [n]): rows with 0 stand for no request: nothing of theirs is logged or moves on, they only get the
+    embedding of the token they hold again."""
+    require_cuda(logits, ids, pos, ctx, log, steps, u, u_all, table, x, mirror, live)
+    if live is not None:
+        _i32(live, n, "live")
     for t, what in ((pos, "pos"), (ctx, "ctx"), (ids, "ids"), (steps, "steps")):
         _i32(t, n, what)
     assert log.dtype == torch.int32 and log.is_contiguous() and log.numel() % n == 0
@@ -683,4 +687,4 @@ def decode_tail(logits: Optional[torch.Tensor], ids: torch.Tensor, pos: torch.Te
         assert mirror is None or (mirror.dtype == torch.bfloat16 and mirror.shape == (n, hidden) and mirror.is_contiguous())
     call("gibbs_decode_tail", ptr(logits), v, ld, ptr(ids), ptr(pos), ptr(ctx), ptr(log), ptr(steps), n, capacity, ptr(u),
          ptr(u_all), ptr(table), dtype_code(table.dtype) if table is not None else 0, vocab, hidden, ptr(x),
-         ptr(mirror) if x is not None else None, stream())
+         ptr(mirror) if x is not None else None, ptr(live), stream())

@@ -250,6 +250,51 @@ def test_continuous_batching_under_page_pressure(dirs):
     assert eng.cache.free_pages() == 17 and eng.cache.free_slots() == 4
 
 
+@pytest.mark.parametrize("sampled", [False, True])
+def test_requests_that_end_one_after_another_share_padded_decode_loops(dirs, sampled):
+    """Five requests of different lengths (one of them ended early by an end-of-sequence token in the
+    middle of a burst) decode in captured loops made for 8, 4, 2 and 1 rows: the rows that stand for no
+    request are padding in the scratch page and slot.  In 32-bit every request gets exactly the tokens it
+    gets alone without bursts; only loops of those row counts were made, and the bursts ran in them."""
+    from gibbs_amd import Engine, Generator, SamplingParams
+    import importlib
+    G_ = importlib.import_module("gibbs_amd.engine.generate")
+    d = dirs["B"]
+    prompts = [H.tokens(170 + i, n, 512) for i, n in enumerate([9, 21, 5, 14, 30])]
+    lengths = [70, 41, 23, 55, 12]
+    temperature = 0.9 if sampled else 0.0
+    def params(n):
+        return SamplingParams(temperature=temperature, max_new_tokens=n, seed=11)
+    alone = []
+    for i, (p, n) in enumerate(zip(prompts, lengths)):
+        eng = Engine(d, dtype="float32", max_tokens=512, max_requests=1)
+        g = Generator(eng, decode_burst=0, eos_token_ids=())
+        rid = g.submit(p, params(n), rid=f"r{i}")
+        alone.append(g.run()[rid].tokens)
+    stop = alone[1][17]                                         # request 1 ends here, inside a burst
+    cut = alone[1].index(stop)
+    eng = Engine(d, dtype="float32", max_tokens=2048, max_requests=5)
+    gen = Generator(eng, decode_burst=16, eos_token_ids=(stop,))
+    rids = [gen.submit(p, params(n), rid=f"r{i}") for i, (p, n) in enumerate(zip(prompts, lengths))]
+    bursts = 0
+    while gen.scheduler.has_work():
+        before = gen.scheduler.steps
+        out = gen.step()
+        bursts += gen.scheduler.steps - before > 1
+        eng.cache.check()
+    res = gen.results()
+    for i, r in enumerate(rids):
+        want = alone[i]
+        if stop in want:
+            want = want[:want.index(stop)]
+        assert res[r].tokens == want, f"request {i}"
+    assert res[rids[1]].finish_reason == "stop" and len(res[rids[1]].tokens) == cut
+    made = sorted(rows for rows, _ in gen._loops)
+    assert made and set(made) <= set(G_.LOOP_ROWS) and 8 in made, made
+    assert bursts >= 4
+    assert eng.cache.free_slots() == 5 and eng.cache.free_pages() == eng.cache.pools[0].num_pages
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_loop_graph_replays_match_eager(dirs, dtype):
     """The captured decode step, replayed several times with eager work and synchronisations in

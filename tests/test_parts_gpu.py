@@ -393,7 +393,7 @@ def test_window_group_gives_pages_back_and_they_are_used_again(name, dtype):
                  group_pages=[24, 12])
     cm = eng.cache
     assert cm.n_groups == 2 and cm.group_layers == [[0], [1]]
-    assert [t.shape[1] for t in eng.device_cache.kpages] == [24, 12], "every group has the pages of its own pool"
+    assert [t.shape[1] for t in eng.device_cache.kpages] == [24 + 1, 12 + 1], "every group has the pages of its own pool (and a scratch page)"
     win = 1                                                     # the window's group
     seqs = {"a": H.tokens(1, 150, spec.vocab), "b": H.tokens(2, 40, spec.vocab), "c": H.tokens(3, 40, spec.vocab)}
     plain = {r: plain_spec_forward(spec, {k: v.double().numpy() for k, v in tensors.items()}, ids) for r, ids in seqs.items()}
