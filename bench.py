@@ -5,8 +5,8 @@ decode at batch 1 and 64 beside it.
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--batch B] [--prompt-len P --context C] [--suite bench/SUITE.json]
 
-`--prompt-len` / `--context` move the same measurement to longer contexts (16k, 32k, 100k; the timed
-prefill stays at 2,048 tokens); `--suite` runs the rows of a suite file of `gibbs --bench` afterwards
+`--prompt-len` / `--context` move the same measurement to longer contexts (16k, 32k, 100k);
+`--prefill-tokens` times a prompt of another length than 2,048; `--suite` runs the rows of a suite file of `gibbs --bench` afterwards
 (the serving workloads of the 350M and 2.6B shapes in bench/lfm2.json) and puts them into the line
 under `rows`.
 
@@ -75,16 +75,16 @@ def seeded_prompt(seed: int, n: int, vocab: int):
     return np.random.default_rng(seed).integers(0, vocab, size=n).tolist()
 
 
-def time_prefill(engine, runs: int = 3):
-    """Median time of a whole 2,048-token prompt in one step (one warm-up first)."""
+def time_prefill(engine, runs: int = 3, n_tokens: int = PROMPT_LEN):
+    """Median time of a whole prompt of `n_tokens` (2,048 unless asked otherwise) in one step (one warm-up first)."""
     import torch
     vocab = engine.spec.vocab
     times = []
     for i in range(runs + 1):
-        ids = seeded_prompt(1000 + i, PROMPT_LEN, vocab)
+        ids = seeded_prompt(1000 + i, n_tokens, vocab)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        engine.step([("prefill", ids, [PROMPT_LEN - 1])])
+        engine.step([("prefill", ids, [n_tokens - 1])])
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         engine.release("prefill")
@@ -284,6 +284,7 @@ def main() -> int:
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens every request holds before decoding starts")
     ap.add_argument("--context", type=int, default=None, help="context limit (default 4096, or what --prompt-len needs)")
+    ap.add_argument("--prefill-tokens", type=int, default=PROMPT_LEN, help="length of the timed prompt (default 2,048)")
     ap.add_argument("--suite", help="a suite file of `gibbs --bench` whose rows are run afterwards and reported under `rows`")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate")
@@ -295,7 +296,7 @@ def main() -> int:
     if args.steps < 1 or args.warmup < 0:
         print("--steps must be at least 1 and --warmup at least 0")
         return 2
-    need = args.prompt_len + args.warmup + (RUNS + 1) * args.steps + 1
+    need = max(args.prompt_len + args.warmup + (RUNS + 1) * args.steps + 1, args.prefill_tokens)
     context = args.context or max(CONTEXT, -(-need // 1024) * 1024)
     if args.prompt_len < 1 or need > context:
         print(f"--prompt-len + --warmup + {RUNS + 1} x --steps must stay below the context ({context})")
@@ -307,8 +308,8 @@ def main() -> int:
                           context=context)
 
     ceiling = R.measured_hbm_bytes_per_s()
-    prefill_s = time_prefill(engine)
-    prefill_flops = R.prefill_flops(engine, PROMPT_LEN)
+    prefill_s = time_prefill(engine, n_tokens=args.prefill_tokens)
+    prefill_flops = R.prefill_flops(engine, args.prefill_tokens)
     peak = R.PEAK_FLOPS[args.dtype]
 
     dt, seq_lens, top = time_decode(engine, args.batch, args.steps, args.warmup, profile=not args.no_kernels,
@@ -340,7 +341,7 @@ def main() -> int:
             "conv_L_cache": cfg.conv_L_cache, "tied_head": cfg.tie_embedding, "page_size": engine.page_size,
             "sampling": "greedy on device", "timed_runs": RUNS,
         },
-        "prefill": {"value": round(PROMPT_LEN / prefill_s, 1), "tokens": PROMPT_LEN, "ms": round(prefill_s * 1e3, 3),
+        "prefill": {"value": round(args.prefill_tokens / prefill_s, 1), "tokens": args.prefill_tokens, "ms": round(prefill_s * 1e3, 3),
                     "frac": round(prefill_flops / prefill_s / peak, 4)},
         # `peak` is the published figure; `measured_peak` is what a kernel that only reads reaches on this GPU
         # (the reference's rows divide by a measured ceiling, src/bench.rs:438-442)

@@ -50,7 +50,7 @@ int gibbs_attention_plain(const void* q, const void* kpages, const void* vpages,
 int gibbs_attention_prefill(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
                             const int* cu, const int* ctx, const int* table, int n_req, int max_pages, int page_size,
                             int num_pages, int n_rows, int nh, int nkv, int hd, long ldq, long ldo, float scale, int window,
-                            int n_splits, int first_row, hipStream_t stream);
+                            int n_splits, int first_row, int heads_per_wg, hipStream_t stream);
 int gibbs_attention_decode_fused(const void* qkv, void* kpages, void* vpages, void* out, float* partial,
                                  const float* q_gain, const float* k_gain, float eps, const float* inv_freq, int rot,
                                  int variant, const float* cs_table, int table_len, const int* pos, const int* row_req,

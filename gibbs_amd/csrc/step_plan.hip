@@ -92,6 +92,20 @@ int prefill_splits(long n_tiles, int nh, int max_seq, int window) {
   return (int)std::max<long>(1, std::min<long>(std::min<long>(ceil_div_l(2048, blocks), keys / 256), 16));
 }
 
+// Query heads of a kv head's group that a workgroup of the prompt attention takes (they share its K and V
+// tiles).  With one head a workgroup re-reads all keys and values of its rows' past for 64 x 64 scores at a
+// time, and from about 4,000 keys a row that traffic, not the arithmetic, bounds the kernel (537 TFLOP/s at
+// 8.4 TB/s through L2 and the L1s); more heads a workgroup are fewer, longer workgroups.  Measured at 32 heads
+// in groups of 4, head size 64 (us, with 1 / 2 / 4 heads): 2,048 rows 68 / 63 / 63; 4,096 rows 196 / 209 / 203;
+// 8,192 rows 577 / 562 / 584; 32,768 rows 8,086 / 7,147 / 6,626; 2,048 rows behind 6,144 keys 281 / 220 / 205;
+// 512 rows behind 7,680 keys in 8 slices 80 / 84 / 92.
+int prefill_heads(int rows, int reqs, int nh, int nkv, int hd, int max_seq, int n_splits) {
+  const int group = nh / std::max(nkv, 1);
+  if (hd > 64 || group % 2 || n_splits > 1) return 1;
+  const long seen = (long)max_seq - rows / (2 * std::max(reqs, 1));   // keys a row sees on average, if one request has them all
+  return (group % 4 == 0 && seen >= 6000) ? 4 : 2;
+}
+
 // Which product runs y = x W^T, and in how many float32 partial sums it leaves its result.
 enum { LIN_F32, LIN_PLAIN, LIN_SKINNY, LIN_LIBRARY, LIN_TILED };
 struct LinearChoice {
@@ -485,7 +499,8 @@ struct AttnBody : Body {
         const int n_splits = a.max_seq > 0 ? prefill_splits(prefill_tiles(rows, reqs), nh, a.max_seq, window) : 1;
         float* partial = n_splits > 1 ? (float*)e.take(gibbs_attention_decode_workspace(N, nh, hd, n_splits) * 4) : nullptr;
         RUN(e, gibbs_attention_prefill(raw, kpages, vpages, att, partial, a.cu + lead, a.ctx + lead, table + (long)lead * width, reqs,
-                                       width, page_size, num_pages, rows, nh, nkv, hd, ldq, ldo, scale, window, n_splits, lead, a.stream));
+                                       width, page_size, num_pages, rows, nh, nkv, hd, ldq, ldo, scale, window, n_splits, lead,
+                                       prefill_heads(rows, reqs, nh, nkv, hd, a.max_seq, n_splits), a.stream));
         e.give(partial);
       } else if (fast_bf16 && a.max_q == 1 && hd % 8 == 0) {
         decode_attention(e, raw, ldq, N, a.pos, a.row_req, att);
@@ -853,6 +868,9 @@ GIBBS_EXPORT int gibbs_rule_prefill_splits(long n_tiles, int nh, int max_seq, in
   return prefill_splits(n_tiles, nh, max_seq, window);
 }
 GIBBS_EXPORT long gibbs_rule_prefill_tiles(int rows, int reqs) { return prefill_tiles(rows, reqs); }
+GIBBS_EXPORT int gibbs_rule_prefill_heads(int rows, int reqs, int nh, int nkv, int hd, int max_seq, int n_splits) {
+  return prefill_heads(rows, reqs, nh, nkv, hd, max_seq, n_splits);
+}
 GIBBS_EXPORT int gibbs_rule_fused_rows(void) { return FUSED_ROWS; }
 
 GIBBS_EXPORT int gibbs_linear_splits(int dtype, int n, int O, int I, long ldx, const void* x, const void* w, int out_f32,

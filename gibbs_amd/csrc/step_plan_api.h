@@ -98,6 +98,7 @@ void gibbs_rule_decode_splits(int n_rows, int nkv, int group, int max_seq, int h
                               int* waves);
 long gibbs_rule_prefill_tiles(int rows, int reqs);            // query tiles that the rows of a ragged batch make
 int gibbs_rule_prefill_splits(long n_tiles, int nh, int max_seq, int window);
+int gibbs_rule_prefill_heads(int rows, int reqs, int nh, int nkv, int hd, int max_seq, int n_splits);   // query heads a workgroup
 int gibbs_rule_fused_rows(void);                              // rows that the fused decode kernels take at most
 // y = x W^T the way a step would run it.  gibbs_linear_splits: the float32 partial sums it would leave (1: the
 // finished product [n, O]; s >= 2: [s, n, O] float32).  gibbs_linear: runs it into y (sized by that answer).

@@ -110,7 +110,12 @@ class Generator:
         try:
             loop = self._loops.get(key)
             if loop is None and n < MIN_STEPS_FOR_NEW_LOOP:
-                return None                                 # capturing graphs for so few steps costs more than it saves
+                # capturing graphs for so few steps costs more than it saves; a loop that was made for more rows
+                # serves as well, while its step costs less than a step through the host (up to twice the rows)
+                loop = next((l for (rows, g), l in sorted(self._loops.items(), key=lambda kv: kv[0][0])
+                             if g == greedy and key[0] < rows <= 2 * key[0]), None)
+                if loop is None:
+                    return None
             if loop is None:
                 loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index, rows=key[0])
             elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:

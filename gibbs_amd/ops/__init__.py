@@ -569,12 +569,13 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
                       vpages: torch.Tensor, table: torch.Tensor, n_req: int, cu: torch.Tensor, ctx: torch.Tensor,
                       scale: float, window: Optional[int] = None, out: Optional[torch.Tensor] = None,
                       max_seq: int = 0, n_splits: Optional[int] = None, first_req: int = 0,
-                      first_row: int = 0) -> torch.Tensor:
+                      first_row: int = 0, heads_per_wg: Optional[int] = None) -> torch.Tensor:
     """bfloat16 paged causal attention for prompt portions on the matrix cores: rows cu[r] .. cu[r+1]
     of request r sit at positions ctx[r] ..; same result as `attention_plain`.  Head sizes: multiples
     of 16 up to 128.  `max_seq`: a bound on the keys of any row, from which the number of key slices
     is chosen (or `n_splits`).  `first_req`, `first_row`: only the requests from `first_req` on are
-    attended to (their rows start at `first_row`); the rows before are left as they are in `out`."""
+    attended to (their rows start at `first_row`); the rows before are left as they are in `out`.
+    `heads_per_wg`: query heads of a kv head's group per workgroup (1, 2 or 4; default: the native step's rule)."""
     require_cuda(q, kpages, vpages, table, cu, ctx)
     if q.dtype != torch.bfloat16:
         raise KernelError("attention_prefill is the bfloat16 kernel; the float32 path uses attention_plain")
@@ -592,12 +593,15 @@ def attention_prefill(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, 
     rows, reqs = n_rows - first_row, n_req - first_req
     if n_splits is None:
         n_splits = prefill_splits(int(library().gibbs_rule_prefill_tiles(rows, reqs)), nh, max_seq, window) if max_seq > 0 else 1
+    if heads_per_wg is None:
+        heads_per_wg = int(library().gibbs_rule_prefill_heads(rows, reqs, nh, nkv, hd, int(max_seq), int(n_splits)))
     partial = None
     if n_splits > 1:
         partial = torch.empty(slices_workspace(n_rows, nh, hd, n_splits), dtype=torch.float32, device=q.device)
     call("gibbs_attention_prefill", ptr(q), ptr(kpages), ptr(vpages), ptr(out), ptr(partial), ptr(cu[first_req:]),
          ptr(ctx[first_req:]), ptr(table[first_req:]), reqs, table.shape[1], page_size, num_pages, rows, nh, nkv, hd,
-         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), int(n_splits), int(first_row), stream())
+         q.stride(0) if n_rows > 1 else q.shape[1], nh * hd, float(scale), int(window or 0), int(n_splits), int(first_row),
+         int(heads_per_wg), stream())
     return out
 
 

@@ -60,7 +60,7 @@ _SIGNATURES = {
                                c_int, c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int,
                                c_int, c_int, c_int, c_void_p],
     "gibbs_attention_prefill": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_void_p],
+                                c_int, c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_gemm_library_init": [],
     "gibbs_gemm_library": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_long, c_long, c_long, c_void_p],
     "gibbs_argmax": [c_void_p, c_void_p, c_int, c_int, c_long, c_void_p],
@@ -78,6 +78,7 @@ _VALUE_SIGNATURES = {
     "gibbs_rule_decode_splits": ([c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p], None),
     "gibbs_rule_prefill_splits": ([c_long, c_int, c_int, c_int], c_int),
     "gibbs_rule_prefill_tiles": ([c_int, c_int], c_long),
+    "gibbs_rule_prefill_heads": ([c_int, c_int, c_int, c_int, c_int, c_int, c_int], c_int),
     "gibbs_rule_fused_rows": ([], c_int),
     "gibbs_linear_splits": ([c_int, c_int, c_int, c_int, c_long, c_void_p, c_void_p, c_int, c_int, c_int], c_int),
     "gibbs_skinny_residual_workspace": ([c_int, c_int, c_int], c_long),

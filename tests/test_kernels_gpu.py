@@ -362,7 +362,7 @@ def test_attention_decode_rows_as_requests_and_rows_beyond_the_bound(bound, n_sp
 @pytest.mark.parametrize("n_splits", [1, 3, 7])
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
                                                    (32, 8, 64, 16, None), (4, 2, 128, 16, None), (2, 2, 96, 64, 100),
-                                                   (3, 1, 32, 16, 5)])
+                                                   (3, 1, 32, 16, 5), (8, 2, 48, 16, None), (12, 2, 32, 8, 90)])
 def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window, n_splits):
     """Prompt portions on the matrix cores: a long portion after a cached context that ends off a
     tile edge, a whole short prompt, a 2-token portion, a single decoded row and a 65-row portion
@@ -393,6 +393,15 @@ def test_attention_prefill_matrix_cores(nh, nkv, hd, page, window, n_splits):
     ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window, out=part,
                           n_splits=n_splits, first_req=first_req, first_row=first_row)
     assert torch.equal(part[first_row:], out[first_row:]) and (part[:first_row] == 7.0).all()
+    # several query heads of a kv head's group in one workgroup (one K and V tile for all of them): every row of
+    # every head goes through the same operations in the same order, so the result is the same to the bit
+    for heads in (2, 4):
+        if (nh // nkv) % heads == 0 and hd <= 64:
+            many = ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window,
+                                         n_splits=n_splits, heads_per_wg=heads)
+            assert torch.equal(many, out), f"{heads} heads a workgroup"
+    with pytest.raises(ops.KernelError, match="heads a workgroup"):
+        ops.attention_prefill(q, n, nh, nkv, hd, kp, vp, table, 5, i32(cu), i32(ctx), scale, window, heads_per_wg=3)
 
 
 def test_prefill_splits_choice():
