@@ -8,7 +8,7 @@
 // reads 1 KB of contiguous cache per instruction) and keep an online-softmax stream of their own
 // (max, sum, weighted values); the streams are merged at the end, first across the wave by
 // shuffles, then across the waves through LDS (wave g folds head g).  With more than one slice the workgroup writes a
-// partial (max, sum, values) and a second kernel merges the slices.  The slice's page ids are
+// partial (max, sum, values) and the slices are merged (see below).  The slice's page ids are
 // staged in LDS, and the loads of the next two keys are in flight while a key is worked on.
 //
 // Two ways to walk the keys of a slice.  On the vector units: every LPK neighbouring lanes own one key
@@ -28,9 +28,15 @@
 // chunk 0 whose key slice holds the row's position does) and uses them from LDS instead of
 // reading them back.
 //
-// The slices are merged by a separate kernel: letting the last workgroup to arrive merge them in
-// place needs device-scope fences, and on this chip (one L2 per XCD) each such fence writes back
-// and invalidates an L2, which cost 130 us a call when it was tried.
+// The slices of a (row, group of heads) are merged by the workgroup that finishes last: every workgroup writes its
+// partial result through to memory (agent-scope stores), waits until the stores have arrived, and counts itself
+// in with one relaxed agent-scope atomic; the one that counts last reads all the partial results with agent-scope
+// loads, which pass its own L2, and leaves the counter at zero.  No fence: on this chip (one L2 per XCD) an
+// agent-scope release or acquire fence writes back or invalidates a whole L2, which cost 130 us a call when every
+// workgroup did it; the accesses above are coherent by themselves.  The chain (stores arrive, the count, the loads)
+// takes about as long as the boundary to a second kernel: 0.8 us a call less than the merge kernel at 8 slices,
+// 2.3 us at 64.  The merge kernel remains for calls with more (rows x groups of heads) than there are counters,
+// and for callers that ask for it (kind + 4).
 //
 // Visibility is by position only: row n sees keys lo .. pos[n] of its request
 // (lo = max(0, pos - window + 1), window 0 = all).
@@ -74,6 +80,68 @@ __device__ __forceinline__ short4v lds_read_transposed(const bf16* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((short4v __attribute__((address_space(3)))*)p);
 }
 
+// Counters of the slices of a (row, group of heads) that have finished, for calls whose last slice merges.  Zero
+// when the module is loaded, and the merging workgroup leaves zero behind.  One array per device and translation
+// unit: calls that overlap on one device (two streams) would share it, as they would share a workspace.
+constexpr int MERGE_COUNTERS = 1 << 15;
+static __device__ int g_merge_counters[MERGE_COUNTERS];
+
+// Two floats (8-byte aligned) written through to where every compute unit of the device sees them.
+__device__ __forceinline__ void store_through2(float* p, float a, float b) {
+  const unsigned long long v = ((unsigned long long)__float_as_uint(b) << 32) | __float_as_uint(a);
+  __hip_atomic_store((unsigned long long*)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_through(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One wave merges the slices of a (row, head) that other workgroups of the same kernel wrote with store_through2:
+// out = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s, eight slices' loads in flight at a time.
+// C: elements of a head per lane.
+template <int C>
+__device__ __forceinline__ void merge_slices_through(const float* ps, int n_splits, int hd, bf16* o, int lane) {
+  const int stride = hd + 2;
+  float M = -INFINITY, L = 0.f, v[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) v[c] = 0.f;
+  for (int s0 = 0; s0 < n_splits; s0 += 8) {
+    float ms[8], ls[8], av[8][C];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int s = min(s0 + j, n_splits - 1);      // (beyond the last slice: the last one again, weighted 0 below)
+      ms[j] = load_through(ps + (size_t)s * stride);
+      ls[j] = load_through(ps + (size_t)s * stride + 1);
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const int e = lane + c * WAVE;
+        av[j][c] = load_through(ps + (size_t)s * stride + 2 + (e < hd ? e : 0));
+      }
+    }
+    float Mn = M;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s0 + j < n_splits) Mn = fmaxf(Mn, ms[j]);
+    const float keep = M == -INFINITY ? 0.f : __expf(M - Mn);
+    L *= keep;
+#pragma unroll
+    for (int c = 0; c < C; ++c) v[c] *= keep;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float w = (s0 + j < n_splits && ms[j] != -INFINITY) ? __expf(ms[j] - Mn) : 0.f;
+      L = fmaf(w, ls[j], L);
+#pragma unroll
+      for (int c = 0; c < C; ++c) v[c] = fmaf(w, av[j][c], v[c]);
+    }
+    M = Mn;
+  }
+  const float inv = 1.0f / L;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int e = lane + c * WAVE;
+    if (e < hd) o[e] = (bf16)(v[c] * inv);
+  }
+}
+
 struct DecodeArgs {
   const int* pos;
   const int* row_req;
@@ -98,6 +166,7 @@ struct DecodeArgs {
   // n_ids page ids are asked for at once, before the row's position is known (one dependent load less in front
   // of the first keys).  A row that is beyond the bound after all takes the ids of its slice as it would without.
   int ids_whole, n_ids;
+  int merge_here;   // the last slice of a (row, group of heads) to finish merges them (else a second kernel does)
 };
 
 // Folds stream b (mb, lb, ab) into stream a.
@@ -483,34 +552,66 @@ __global__ __launch_bounds__(NW * WAVE, GT <= 4 ? (NW == 8 ? 4 : 3) : 2) void at
   }
   __syncthreads();
   // the waves' streams of head g meet in wave g % NW
-  if (grp != 0) return;
+  const bool merge_here = a.n_splits > 1 && a.merge_here;
+  if (grp == 0) {
+    for (int g = wave; g < gcount; g += NW) {
+      float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
+#pragma unroll
+      for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) {
+        float ab[EPL];
+#pragma unroll
+        for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
+        fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
+      }
+      const int head = kvh * G + g0 + g;
+      if (a.n_splits == 1) {
+        if (active) {
+          const float inv = 1.0f / ll;
+          bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
+#pragma unroll
+          for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
+        }
+      } else if (merge_here) {
+        // stores that another workgroup, on another L2, reads in this same kernel: written through
+        float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
+        if (sub == 0) store_through2(ps, mm, ll);
+        if (active) {
+#pragma unroll
+          for (int i = 0; i < EPL; i += 2) store_through2(ps + 2 + e0 + i, aa[i], aa[i + 1]);
+        }
+      } else {
+        float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
+        if (sub == 0) { ps[0] = mm; ps[1] = ll; }
+        if (active) {
+#pragma unroll
+          for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
+        }
+      }
+    }
+  }
+  if (!merge_here) return;
+  // The slice of a (row, group of heads) that finishes last merges them all.  Every wave waits until its own
+  // stores have arrived; then one thread counts the workgroup in.  The count, the stores above and the loads
+  // below are agent-scope accesses (they pass the L2 of their XCD); no fence is needed besides: a fence would
+  // write back and invalidate a whole L2 per workgroup.
+  __builtin_amdgcn_s_waitcnt(0);   // (every counter: the stores are vmcnt)
+  __syncthreads();
+  __shared__ int s_last;
+  int* counter = g_merge_counters + (size_t)row * gridDim.y + blockIdx.y;
+  if (threadIdx.x == 0) {
+    const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before == a.n_splits - 1;
+    if (s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // for the next call
+  }
+  __syncthreads();
+  if (!s_last) return;
+  constexpr int C = (MAX_HD + WAVE - 1) / WAVE;
   for (int g = wave; g < gcount; g += NW) {
-    float mm = s_ml[0][g][0], ll = s_ml[0][g][1], aa[EPL];
-#pragma unroll
-    for (int i = 0; i < EPL; ++i) aa[i] = s_acc[0][g][e0 + i];
-#pragma unroll
-    for (int w = 1; w < NW; ++w) {
-      float ab[EPL];
-#pragma unroll
-      for (int i = 0; i < EPL; ++i) ab[i] = s_acc[w][g][e0 + i];
-      fold<EPL>(mm, ll, aa, s_ml[w][g][0], s_ml[w][g][1], ab);
-    }
     const int head = kvh * G + g0 + g;
-    if (a.n_splits == 1) {
-      if (active) {
-        const float inv = 1.0f / ll;
-        bf16* o = out + (size_t)row * a.ldo + (size_t)head * hd + e0;
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) o[i] = (bf16)(aa[i] * inv);
-      }
-    } else {
-      float* ps = partial + (((size_t)row * a.nh + head) * a.n_splits + split) * (hd + 2);
-      if (sub == 0) { ps[0] = mm; ps[1] = ll; }
-      if (active) {
-#pragma unroll
-        for (int i = 0; i < EPL; ++i) ps[2 + e0 + i] = aa[i];
-      }
-    }
+    merge_slices_through<C>(partial + ((size_t)row * a.nh + head) * a.n_splits * (hd + 2), a.n_splits, hd,
+                            out + (size_t)row * a.ldo + (size_t)head * hd, lane);
   }
 }
 
@@ -546,7 +647,8 @@ void launch_waves(int waves, bool mm, int gt, dim3 grid, hipStream_t stream, con
   else launch_decode<LPK, RAW, 4, false>(gt, grid, stream, q, k, v, partial, out, a);
 }
 
-// kind: 0 = choose, 1 = vector units, 2 = matrix cores (refused where they cannot take the shape)
+// kind: 0 = choose, 1 = vector units, 2 = matrix cores (refused where they cannot take the shape); + 4: the slices
+// are merged by a second kernel even where the last slice to finish could do it
 template <bool RAW>
 int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* partial, DecodeArgs a, int n_rows, int waves,
                int kind, int max_keys, hipStream_t stream) {
@@ -556,6 +658,9 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   a.page_shift = (a.page_size & (a.page_size - 1)) == 0 ? __builtin_ctz(a.page_size) : -1;
   GIBBS_REQUIRE((long)a.nkv * a.head_chunks <= 65535, "attention_decode: too many heads");
   dim3 grid(n_rows, a.nkv * a.head_chunks, a.n_splits);
+  // The last slice to finish merges, where the counters reach; kind + 4 asks for the second kernel instead.
+  a.merge_here = a.n_splits > 1 && !(kind & 4) && (long)n_rows * grid.y <= MERGE_COUNTERS;
+  kind &= 3;
   const int lanes = a.hd / EPL;  // lanes that hold data; LPK is the next power of two
   // The matrix-core walk keeps the page ids of a whole key slice in LDS and takes head sizes in steps of
   // 16 up to 128.  The longest slice that the block table (or the caller's bound on the keys) allows:
@@ -574,7 +679,7 @@ int run_decode(const bf16* q, bf16* kpages, bf16* vpages, bf16* out, float* part
   else launch_waves<32, RAW>(waves, false, gt, grid, stream, q, kpages, vpages, partial, out, a);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return gibbs_fail("attention_decode: %s", hipGetErrorString(e));
-  if (a.n_splits > 1) {
+  if (a.n_splits > 1 && !a.merge_here) {
     dim3 mgrid(n_rows, ceil_div(a.nh, 4));
     launch_attention_merge(mgrid, stream, partial, out, a.nh, a.hd, a.n_splits, a.ldo);
   }

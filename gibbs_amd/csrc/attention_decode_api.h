@@ -11,7 +11,8 @@ long gibbs_attention_decode_workspace(int n_rows, int nh, int hd, int n_splits);
 
 // q: [N, >= nh*hd] bfloat16 (row stride ldq); pages: [num_pages, nkv, page_size, hd] bfloat16;
 // out: [N, nh*hd] bfloat16 (row stride ldo); partial: the workspace above, or null with n_splits 1.
-// kind: 0 choose, 1 vector units, 2 matrix cores; max_keys: a bound on the keys of any row (0: the
+// kind: 0 choose, 1 vector units, 2 matrix cores (+ 4: the key slices are merged by a second kernel, not by the
+// slice that finishes last); max_keys: a bound on the keys of any row (0: the
 // block table's width).  Returns 0, or non-zero with the reason in gibbs_last_error().
 int gibbs_attention_decode(const void* q, const void* kpages, const void* vpages, void* out, float* partial,
                            const int* pos, const int* row_req, const int* table, int max_pages, int page_size,

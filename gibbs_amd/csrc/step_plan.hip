@@ -65,6 +65,7 @@ int skinny_splits(int n_out, int inner, int want_blocks = 512, int features = 16
 // keys).  The matrix-core walk keeps the page ids of a whole slice in LDS: caches longer than that are cut
 // into as many slices as it takes.  kind: 0 the kernel's choice of walk, 1 vector units, 2 matrix cores.
 void decode_splits(int n_rows, int nkv, int group, int max_seq, int hd, int page_size, int kind, int* n_splits, int* waves) {
+  kind &= 3;   // (+ 4 only says which kernel merges the slices)
   const bool matrix = kind != 1 && hd > 0 && hd % 16 == 0 && hd <= 128;
   const int gt = group >= 8 ? 8 : (group > 2 ? 4 : group);
   const long per_split = std::max<long>(1, (long)n_rows * nkv * ceil_div_l(group, gt));

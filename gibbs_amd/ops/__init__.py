@@ -502,7 +502,8 @@ def attention_plain(q: torch.Tensor, n_rows: int, nh: int, nkv: int, hd: int, kp
 
 
 # how the decode attention walks its keys: chosen by the kernel, on the vector units, on the matrix cores
-DECODE_KINDS = {"auto": 0, "valu": 1, "mfma": 2}
+# (+ 4, "-merge-pass": the key slices are merged by a second kernel instead of by the slice that finishes last)
+DECODE_KINDS = {"auto": 0, "valu": 1, "mfma": 2, "auto-merge-pass": 4, "valu-merge-pass": 5, "mfma-merge-pass": 6}
 
 
 def slices_workspace(n_rows: int, nh: int, hd: int, n_splits: int) -> int:

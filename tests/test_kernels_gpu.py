@@ -304,7 +304,7 @@ def test_attention_plain_paged(dtype, nh, nkv, hd, page, window):
         at += len(ps)
 
 
-@pytest.mark.parametrize("kind", ["valu", "mfma"])
+@pytest.mark.parametrize("kind", ["valu", "mfma", "valu-merge-pass", "mfma-merge-pass"])
 @pytest.mark.parametrize("n_splits,waves", [(1, 4), (1, 8), (3, 8), (16, 4), (None, None)])
 @pytest.mark.parametrize("nh,nkv,hd,page,window", [(4, 2, 16, 16, None), (6, 1, 48, 8, None), (5, 5, 80, 32, 37),
                                                    (32, 8, 64, 16, None), (16, 2, 128, 16, None), (2, 2, 256, 64, 100),
@@ -320,7 +320,7 @@ def test_attention_decode_split_keys(nh, nkv, hd, page, window, n_splits, waves,
     pos, row_req = i32(positions), i32([0, 1, 2, 3])
     q = rnd(4, nh * hd, dtype=dtype, seed=9)
     scale = 1 / math.sqrt(hd)
-    if kind == "mfma" and (hd % 16 or hd > 128):
+    if kind.startswith("mfma") and (hd % 16 or hd > 128):
         with pytest.raises(ops.KernelError, match="matrix-core"):
             ops.attention_decode(q, 4, nh, nkv, hd, kp, vp, table, 4, pos, row_req, scale, window, max_seq=700,
                                  n_splits=n_splits, waves=waves, kind=kind)
@@ -784,7 +784,7 @@ def test_embed_and_residual_mirror():
     close(out, F.rms_norm(x.double(), (72,), None, 1e-5), torch.bfloat16, "gain-free norm")
 
 
-@pytest.mark.parametrize("kind", ["valu", "mfma"])
+@pytest.mark.parametrize("kind", ["valu", "mfma", "mfma-merge-pass"])
 @pytest.mark.parametrize("n_splits,table_len,waves", [(1, 0, 8), (4, 20, 4), (None, 1024, None)])   # rows at 699 and 32 beyond a table of 20
 @pytest.mark.parametrize("variant", ["half_split", "interleaved"])
 @pytest.mark.parametrize("nh,nkv,hd,rot,page,window", [(4, 2, 16, 16, 16, None), (32, 8, 64, 64, 16, None), (6, 1, 48, 32, 8, None),
@@ -815,6 +815,36 @@ def test_attention_decode_fused(nh, nkv, hd, rot, page, window, variant, n_split
     close(kp1, kp2, dtype, "new keys in the pages", bf16=8e-3)
     assert torch.equal(vp1, vp2)
     close(got, want, dtype, "fused decode attention", bf16=8e-3)
+
+
+@pytest.mark.parametrize("n_rows,nh,nkv,hd,n_splits", [(64, 32, 8, 64, 8), (3, 6, 2, 48, 5), (2, 4, 1, 128, 40),
+                                                       (4200, 8, 8, 16, 2)])
+def test_slices_merged_by_the_last_to_finish_or_by_a_second_kernel(n_rows, nh, nkv, hd, n_splits):
+    """The key slices of a row are merged by the workgroup that finishes last, through memory that the other
+    workgroups wrote in the same kernel; a second kernel does the same arithmetic where it is asked for, or where
+    rows x groups of heads exceed the counters (4,200 x 8).  Up to 8 slices both add in the same order: the results
+    are equal bit for bit, call after call (the counters are left at zero, no partial result is read before it has
+    arrived); beyond 8 they differ by rounding."""
+    from gibbs_amd import ops
+    dtype, page = torch.bfloat16, 16
+    long_rows = n_rows <= 64
+    seq_lens = [(900 + 37 * r) if long_rows else 20 + r % 13 for r in range(n_rows)]
+    kp, vp, table, ks, vs = paged_setup(dtype, nkv, hd, page, seq_lens, sum(-(-l // page) for l in seq_lens) + 8, seed=3)
+    pos = i32([l - 1 for l in seq_lens])
+    q = rnd(n_rows, nh * hd, dtype=dtype, seed=4)
+    scale = 1 / math.sqrt(hd)
+    want = ops.attention_decode(q, n_rows, nh, nkv, hd, kp, vp, table, n_rows, pos, None, scale, None, max_seq=max(seq_lens),
+                                n_splits=n_splits, waves=4, kind="mfma-merge-pass")
+    for call in range(12 if long_rows else 2):
+        got = ops.attention_decode(q, n_rows, nh, nkv, hd, kp, vp, table, n_rows, pos, None, scale, None,
+                                   max_seq=max(seq_lens), n_splits=n_splits, waves=4, kind="mfma")
+        if n_splits <= 8:
+            assert torch.equal(got, want), f"call {call}"
+        else:
+            close(got, want, dtype, f"merged in the kernel, call {call}", bf16=4e-3)
+    for r in range(min(n_rows, 3)):
+        ref = attention_reference(q[r:r + 1].view(1, nh, hd), ks[r], vs[r], [seq_lens[r] - 1], scale, None)
+        close(got[r].view(1, nh, hd), ref, dtype, f"row {r}", bf16=1e-2)
 
 
 def test_attention_block_table_segments():
