@@ -50,7 +50,7 @@ _SIGNATURES = {
     "gibbs_sched_plan": ([c_void_p, _lp, c_int, _lp, c_long, _lp], c_int),
     "gibbs_sched_apply": ([c_void_p, c_int, _ip, _ip, _ip, _lp, c_long, _lp], c_int),
     "gibbs_sched_fail_plan": ([c_void_p, _lp, c_long, _lp], c_int),
-    "gibbs_sched_burst_plan": ([c_void_p, c_long, _ip, c_int, _ip], c_long),
+    "gibbs_sched_burst_plan": ([c_void_p, c_long, _ip, c_int, _ip, _lp], c_long),
     "gibbs_sched_apply_burst": ([c_void_p, c_int, c_int, _ip, _lp, c_long, _lp], c_int),
     "gibbs_cache_fill_step": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, _lp, c_void_p, _lp],
                               c_int),

@@ -346,18 +346,25 @@ HOST_EXPORT int gibbs_sched_fail_plan(void* sched, long* events, long events_cap
 
 // Several decode steps back to back: when nothing waits and every running request decodes with one
 // token to feed, the requests (oldest first) into out and the steps all of them can still take (at most
-// cap); 0 when a step has anything else to do.
-HOST_EXPORT long gibbs_sched_burst_plan(const void* sched, long cap, int* out, int out_cap, int* n_out) {
+// cap); 0 when a step has anything else to do.  *longest: the steps until the last of them reaches its token
+// limit (at most cap, and within every request's context): a burst may run that long, the tokens that a request
+// samples beyond its limit are dropped when the burst is booked, as those behind an end-of-sequence token are.
+HOST_EXPORT long gibbs_sched_burst_plan(const void* sched, long cap, int* out, int out_cap, int* n_out, long* longest) {
   const Scheduler* s = (const Scheduler*)sched;
   *n_out = 0;
+  if (longest) *longest = 0;
   if (!s->waiting.empty() || s->active.empty() || (int)s->active.size() > out_cap) return 0;
-  long n = cap;
+  long n = cap, room = cap, last = 0;
   for (int id : s->active) {
     const Seq& q = s->seqs[id];
     if (q.state != DECODING || s->remaining(q) != 1) return 0;
-    n = std::min(n, std::min(q.max_new - q.output_len, s->context_len - q.total()));
+    room = std::min(room, (long)(s->context_len - q.total()));
+    n = std::min(n, (long)(q.max_new - q.output_len));
+    last = std::max(last, (long)(q.max_new - q.output_len));
   }
+  n = std::min(n, room);
   if (n < 1) return 0;
+  if (longest) *longest = std::max(n, std::min(last, room));
   std::vector<int> order = s->active;
   std::sort(order.begin(), order.end(), [&](int a, int b) { return s->seqs[a].submitted < s->seqs[b].submitted; });
   std::copy(order.begin(), order.end(), out);

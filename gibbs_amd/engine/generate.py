@@ -96,7 +96,7 @@ class Generator:
         plan = self.scheduler.burst_plan(self.decode_burst) if self.decode_burst > 0 else None
         if plan is None:
             return None
-        seqs, n = plan
+        seqs, n, longest = plan
         rids = [s.id for s in seqs]
         params = [s.params for s in seqs]
         greedy = all(p.greedy for p in params)
@@ -107,27 +107,36 @@ class Generator:
         last = [s.output_tokens[-1] for s in seqs]
         index = [len(s.output_tokens) for s in seqs]
         key = (loop_rows(len(seqs)), greedy)
-        try:
-            loop = self._loops.get(key)
-            if loop is None and n < MIN_STEPS_FOR_NEW_LOOP:
-                # capturing graphs for so few steps costs more than it saves; a loop that was made for more rows
-                # serves as well, while its step costs less than a step through the host (up to twice the rows)
-                loop = next((l for (rows, g), l in sorted(self._loops.items(), key=lambda kv: kv[0][0])
-                             if g == greedy and key[0] < rows <= 2 * key[0]), None)
-                if loop is None:
-                    return None
+        loop = self._loops.get(key)
+        # Requests that reach their token limits one after another would cut every burst at the next one to end.
+        # The rows of a loop cost what they cost, live or not: the burst runs until the last of them ends (where the
+        # pages allow it), and the tokens behind a request's limit are dropped like those behind an end of sequence.
+        spans = [longest, n] if longest > n else [n]
+        if loop is None and spans[0] < MIN_STEPS_FOR_NEW_LOOP:
+            # capturing graphs for so few steps costs more than it saves; a loop that was made for more rows
+            # serves as well, while its step costs less than a step through the host (up to twice the rows)
+            loop = next((l for (rows, g), l in sorted(self._loops.items(), key=lambda kv: kv[0][0])
+                         if g == greedy and key[0] < rows <= 2 * key[0]), None)
             if loop is None:
-                loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index, rows=key[0])
-            elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:
-                loop.rebind(rids, last, params, index)
-            else:
-                loop.params, loop.index = params, [i - loop.steps_done for i in index]
-            self._stepped = False
-            started = self.scheduler.clock()
-            loop.run(n)
-            tokens = loop.tokens(last=n)                    # (reading them back waits for the steps)
-        except OutOfPages:
-            return None                                     # let the scheduler make room
+                return None
+        tokens = None
+        for n in spans:
+            try:
+                if loop is None:
+                    loop = self._loops[key] = DecodeLoop(self.engine, rids, last, params, first_index=index, rows=key[0])
+                elif self._stepped or loop.rids != rids or loop.steps_done + n > loop.capacity:
+                    loop.rebind(rids, last, params, index)
+                else:
+                    loop.params, loop.index = params, [i - loop.steps_done for i in index]
+                self._stepped = False
+                started = self.scheduler.clock()
+                loop.run(n)
+                tokens = loop.tokens(last=n)                # (reading them back waits for the steps)
+                break
+            except OutOfPages:
+                continue                                    # the shorter span; or let the scheduler make room
+        if tokens is None:
+            return None
         if self.scheduler.tuner is not None:
             self.scheduler.tuner.record((self.scheduler.clock() - started) / n, 0, len(seqs))
         return self.scheduler.apply_burst(seqs, tokens)

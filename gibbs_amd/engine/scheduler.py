@@ -334,16 +334,19 @@ class ContinuousBatchScheduler:
         return StepOutput(entries, emitted, finished, preempted, prefill_tokens, decode_tokens, active, waiting)
 
     # ------------------------------------------------------------------ bursts of decode steps
-    def burst_plan(self, cap: int) -> Optional[Tuple[List[Sequence], int]]:
+    def burst_plan(self, cap: int) -> Optional[Tuple[List[Sequence], int, int]]:
         """When nothing waits and every running request decodes, several decode steps may run back to
         back on the device without the host in between (a captured graph per step).  Returns the
-        requests (oldest first) and how many steps all of them can still take, at most `cap`; None
-        when a step has anything else to do."""
-        n_out = ctypes.c_int(0)
-        n = self._lib.gibbs_sched_burst_plan(self._core, cap, self._numbers, len(self._numbers), ctypes.byref(n_out))
+        requests (oldest first), how many steps all of them can still take, at most `cap`, and how many
+        steps it is until the last of them reaches its token limit (at most `cap`; a burst may run that
+        long: `apply_burst` drops what a request samples beyond its limit); None when a step has anything
+        else to do."""
+        n_out, longest = ctypes.c_int(0), ctypes.c_long(0)
+        n = self._lib.gibbs_sched_burst_plan(self._core, cap, self._numbers, len(self._numbers), ctypes.byref(n_out),
+                                             ctypes.byref(longest))
         if n < 1:
             return None
-        return [self._seqs[self._numbers[i]] for i in range(n_out.value)], int(n)
+        return [self._seqs[self._numbers[i]] for i in range(n_out.value)], int(n), int(longest.value)
 
     def apply_burst(self, seqs: List[Sequence], tokens: List[List[int]]) -> StepOutput:
         """Books the tokens that a burst sampled (tokens[i]: those of seqs[i], all already cached):

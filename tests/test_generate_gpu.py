@@ -78,8 +78,8 @@ def test_greedy_generation_matches_plain(dirs, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decode_bursts_change_nothing(dirs, dtype):
     """Generation with bursts of captured decode steps gives the tokens that stepping through the
-    host gives: greedy and sampled, requests of different lengths that finish at different times,
-    an end-of-sequence token inside a burst."""
+    host gives: greedy and sampled, requests of different lengths that finish at different times
+    (inside bursts that run on until the longest request ends), an end-of-sequence token inside a burst."""
     from gibbs_amd import Engine, Generator, SamplingParams
     d = dirs["B"]
     prompts = [H.tokens(70 + i, n, 512) for i, n in enumerate([9, 21, 5])]
@@ -93,6 +93,10 @@ def test_decode_bursts_change_nothing(dirs, dtype):
             res = gen.run()
             runs.append([res[r].tokens for r in rids])
             assert [len(t) for t in runs[-1]] == [37, 20, 9]
+            if burst == 16:
+                # a burst is not cut where the next request reaches its limit: the prompts' step, then 16 + 16 + 4
+                # decode steps as three bursts (what the shorter requests sample beyond their limits is dropped)
+                assert gen.stats.steps == 4
             eng.cache.check()
             assert eng.cache.free_slots() == 4
         assert runs[0] == runs[1] == runs[2], f"temperature {temperature}"
