@@ -1,12 +1,12 @@
 """Steady decoding of a fixed set of live requests: one token per request per step, sampled on the
 device and fed back on the device, the whole step replayed as one captured HIP graph.
 
-The step is the engine's own: `model.forward` over a `StepBatch` whose metadata lives in static
-device buffers.  What changes between steps (positions, cached lengths, the sampled ids, the random
+The step is the engine's own: the native step (`NativePlan.step`) over a `StepBatch` whose metadata lives in
+static device buffers.  What changes between steps (positions, cached lengths, the sampled ids, the random
 draws) is updated by a kernel at the end of the step, so a replay needs no host work; pages for all
-steps of a `run` are reserved, and the block tables uploaded, before the first of them.  With the
-native step that same kernel also writes the sampled tokens' embeddings as the next step's residual
-rows, so a step is: layers, final norm, head, and one kernel for argmax, log, advance and embedding.
+steps of a `run` are reserved, and the block tables uploaded, before the first of them.  That same
+kernel also writes the sampled tokens' embeddings as the next step's residual rows, so a step is: layers,
+final norm, head, and one kernel for argmax, log, advance and embedding.
 """
 from __future__ import annotations
 
