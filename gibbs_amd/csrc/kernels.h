@@ -37,7 +37,7 @@ int gibbs_skinny_conv(const void* X, const void* W, void* Y, int N, int C, int I
                       const int* ctx, int K, hipStream_t stream);
 int gibbs_glu(const void* gu, void* out, int dtype, int n, int F, int act, hipStream_t stream);
 int gibbs_shortconv(const void* bcx, const float* taps, const float* bias, float* state, long slot_stride, const int* cu,
-                    const int* ctx, const int* slot, void* y, int dtype, int n_rows, int n_req, int C, int K,
+                    const int* ctx, const int* slot, void* y, int dtype, int n_rows, int n_req, int lead_single, int C, int K,
                     hipStream_t stream);
 int gibbs_qk_rope_kv(void* qkv, void* kpages, void* vpages, int dtype, const float* q_gain, const float* k_gain, float eps,
                      const float* inv_freq, int rot, int variant, const float* cs_table, int table_len, const int* pos,

@@ -20,13 +20,20 @@ template <typename T>
 __global__ __launch_bounds__(256) void shortconv_kernel(
     const T* __restrict__ bcx, const float* __restrict__ taps, const float* __restrict__ bias,
     float* __restrict__ state, long slot_stride, const int* __restrict__ cu, const int* __restrict__ ctx,
-    const int* __restrict__ slot, T* __restrict__ y, int n_req, int C, int K) {
-  int tile = blockIdx.y, r = 0, q = 0;
-  for (; r < n_req; ++r) {
-    q = cu[r + 1] - cu[r];
-    const int t = (q + TL - 1) / TL;
-    if (tile < t) break;
-    tile -= t;
+    const int* __restrict__ slot, T* __restrict__ y, int n_req, int C, int K, int lead_single) {
+  // The first lead_single requests bring one row each (decoded tokens): tile i is request i.  Behind them a walk
+  // over the requests finds the tile's request and rows.
+  int tile = blockIdx.y, r = tile, q = 1;
+  if (tile < lead_single) {
+    tile = 0;
+  } else {
+    tile -= lead_single;
+    for (r = lead_single; r < n_req; ++r) {
+      q = cu[r + 1] - cu[r];
+      const int t = (q + TL - 1) / TL;
+      if (tile < t) break;
+      tile -= t;
+    }
   }
   if (r >= n_req) return;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
@@ -80,16 +87,14 @@ template <int K>
 __global__ __launch_bounds__(64) void shortconv_bf16x8_kernel(
     const bf16* __restrict__ bcx, const float* __restrict__ taps, const float* __restrict__ bias,
     float* __restrict__ state, long slot_stride, const int* __restrict__ cu, const int* __restrict__ ctx,
-    const int* __restrict__ slot, bf16* __restrict__ y, int n_req, int C, int one_row_each) {
-  int tile = blockIdx.y, r = 0, q = 0;
-  // as many rows as requests: if every request brings one row (decoded tokens only), tile i is
-  // request i and there is no walk over the requests; any other split of the rows takes the walk
-  if (one_row_each && tile < n_req && cu[tile] == tile && cu[tile + 1] == tile + 1) {
-    r = tile;
-    q = 1;
+    const int* __restrict__ slot, bf16* __restrict__ y, int n_req, int C, int lead_single) {
+  // (the first lead_single requests bring one row each: tile i is request i, and there is no walk)
+  int tile = blockIdx.y, r = tile, q = 1;
+  if (tile < lead_single) {
     tile = 0;
   } else {
-    for (; r < n_req; ++r) {
+    tile -= lead_single;
+    for (r = lead_single; r < n_req; ++r) {
       q = cu[r + 1] - cu[r];
       const int t = (q + TLV - 1) / TLV;
       if (tile < t) break;
@@ -181,30 +186,34 @@ __global__ __launch_bounds__(64) void shortconv_bf16x8_kernel(
 }
 }  // namespace
 
+// lead_single: how many requests at the head of the batch bring exactly one row each (decoded tokens; 0 if unknown).
 GIBBS_EXPORT int gibbs_shortconv(const void* bcx, const float* taps, const float* bias, float* state,
                                  long slot_stride, const int* cu, const int* ctx, const int* slot, void* y,
-                                 int dtype, int n_rows, int n_req, int C, int K, hipStream_t stream) {
+                                 int dtype, int n_rows, int n_req, int lead_single, int C, int K, hipStream_t stream) {
   GIBBS_REQUIRE(n_rows >= 0 && n_req >= 0 && C > 0, "shortconv: bad sizes rows=%d requests=%d width=%d", n_rows, n_req, C);
   GIBBS_REQUIRE(K >= 2 && K - 1 <= TL, "shortconv: kernel length %d outside 2..%d", K, TL + 1);
   GIBBS_REQUIRE(slot_stride >= (long)(K - 1) * C, "shortconv: state slot stride %ld shorter than (K-1)*C", slot_stride);
+  GIBBS_REQUIRE(lead_single >= 0 && lead_single <= n_req && lead_single <= n_rows, "shortconv: %d leading single rows among %d requests, %d rows", lead_single, n_req, n_rows);
   if (n_rows == 0 || n_req == 0) return 0;
-  dim3 grid(ceil_div(C, 256), ceil_div(n_rows, TL) + n_req);
+  // tiles: one per leading single row; behind them at most ceil(rows / tile) + requests
+  const int rest_rows = n_rows - lead_single, rest_req = n_req - lead_single;
+  auto tiles = [&](int per) { return lead_single + (rest_req > 0 ? ceil_div(rest_rows, per) + rest_req : 0); };
+  dim3 grid(ceil_div(C, 256), tiles(TL));
   GIBBS_REQUIRE(grid.y <= 65535, "shortconv: too many row tiles (%d)", (int)grid.y);
   if (dtype == GIBBS_F32)
     shortconv_kernel<float><<<grid, 256, 0, stream>>>((const float*)bcx, taps, bias, state, slot_stride, cu, ctx,
-                                                      slot, (float*)y, n_req, C, K);
+                                                      slot, (float*)y, n_req, C, K, lead_single);
   else if (dtype == GIBBS_BF16 && C % 8 == 0 && K >= 2 && K <= 4 && ((uintptr_t)bcx % 16) == 0 && ((uintptr_t)y % 16) == 0) {
-    dim3 vgrid(ceil_div(C, 8 * 64), ceil_div(n_rows, TLV) + n_req);
+    dim3 vgrid(ceil_div(C, 8 * 64), tiles(TLV));
     GIBBS_REQUIRE(vgrid.y <= 65535, "shortconv: too many row tiles (%d)", (int)vgrid.y);
     const bf16* in = (const bf16*)bcx;
     bf16* out = (bf16*)y;
-    const int one = n_rows == n_req;
-    if (K == 2) shortconv_bf16x8_kernel<2><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
-    else if (K == 3) shortconv_bf16x8_kernel<3><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
-    else shortconv_bf16x8_kernel<4><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, one);
+    if (K == 2) shortconv_bf16x8_kernel<2><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, lead_single);
+    else if (K == 3) shortconv_bf16x8_kernel<3><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, lead_single);
+    else shortconv_bf16x8_kernel<4><<<vgrid, 64, 0, stream>>>(in, taps, bias, state, slot_stride, cu, ctx, slot, out, n_req, C, lead_single);
   } else if (dtype == GIBBS_BF16)
     shortconv_kernel<bf16><<<grid, 256, 0, stream>>>((const bf16*)bcx, taps, bias, state, slot_stride, cu, ctx,
-                                                     slot, (bf16*)y, n_req, C, K);
+                                                     slot, (bf16*)y, n_req, C, K, lead_single);
   else
     return gibbs_fail("shortconv: unknown dtype %d", dtype);
   GIBBS_LAUNCH_STATUS("shortconv");

@@ -388,7 +388,9 @@ struct ConvBody : Body {
     const int N = e.a.n_rows;
     void* bcx = e.linear(h, in, N, false, false, false, nullptr);
     void* y = e.take((long)N * C * e.esize);
-    RUN(e, gibbs_shortconv(bcx, taps, bias, state, slot_stride, e.a.cu, e.a.ctx, e.a.slot, y, e.p.dtype, N, e.a.n_req, C, K, e.a.stream));
+    // (requests at the head of the batch that bring one row each: all of them in a step of decoded tokens)
+    const int lead = e.a.max_q == 1 ? e.a.n_req : e.a.lead_single;
+    RUN(e, gibbs_shortconv(bcx, taps, bias, state, slot_stride, e.a.cu, e.a.ctx, e.a.slot, y, e.p.dtype, N, e.a.n_req, lead, C, K, e.a.stream));
     e.give(bcx);
     Pending delta;
     delta.data = e.linear(y, out, N, false, true, true, &delta.parts);

@@ -93,7 +93,7 @@ class DecodeLoop:
             n_rows=b, n_req=b, n_logits=b, ids=d[self._sec[0]], pos=d[self._sec[1]], row_req=d[self._sec[2]],
             cu=d[self._sec[3]], ctx=d[self._sec[4]], slot=d[self._sec[5]], logit_rows=d[self._sec[6]],
             tables=[d[self._sec[7 + g]].view(b, w) for g, w in enumerate(self.width)],
-            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, decode_graph=True)
+            q_lens=[1] * b, ctx_lens=[0] * b, slots=[0] * b, max_q=1, max_seq=0, lead_single=b, decode_graph=True)
         self.log = torch.zeros((self.capacity, b), dtype=torch.int32, device=dev)
         self.counter = torch.zeros(b, dtype=torch.int32, device=dev)          # steps done, per row
         self.live_mask = torch.zeros(b, dtype=torch.int32, device=dev) if self.padded else None   # 0: a row of padding

@@ -402,9 +402,11 @@ def glu(gu: torch.Tensor, activation: str = "silu", out: Optional[torch.Tensor] 
 
 def shortconv(bcx: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
               cu: torch.Tensor, ctx: torch.Tensor, slot: torch.Tensor, n_rows: int, n_req: int,
-              out: Optional[torch.Tensor] = None) -> torch.Tensor:
+              out: Optional[torch.Tensor] = None, lead_single: Optional[int] = None) -> torch.Tensor:
     """Gated short convolution of a ragged batch with its per-request state.
-    bcx: [N, 3C]; taps: [C, K] float32; state: [slots, K-1, C] float32 (slot stride free)."""
+    bcx: [N, 3C]; taps: [C, K] float32; state: [slots, K-1, C] float32 (slot stride free).
+    lead_single: how many requests at the head of the batch bring exactly one row each (the kernel finds their
+    rows without a walk over the requests); None: all of them if there are as many rows as requests, else none."""
     require_cuda(bcx, taps, bias, state, cu, ctx, slot)
     c, k = taps.shape
     assert bcx.shape == (n_rows, 3 * c) and bcx.is_contiguous()
@@ -417,7 +419,8 @@ def shortconv(bcx: torch.Tensor, taps: torch.Tensor, bias: Optional[torch.Tensor
         out = torch.empty((n_rows, c), dtype=bcx.dtype, device=bcx.device)
     assert out.shape == (n_rows, c) and out.dtype == bcx.dtype and out.is_contiguous()
     call("gibbs_shortconv", ptr(bcx), ptr(taps), ptr(bias), ptr(state), state.stride(0), ptr(cu), ptr(ctx),
-         ptr(slot), ptr(out), dtype_code(bcx.dtype), n_rows, n_req, c, k, stream())
+         ptr(slot), ptr(out), dtype_code(bcx.dtype), n_rows, n_req,
+         (n_req if n_rows == n_req else 0) if lead_single is None else int(lead_single), c, k, stream())
     return out
 
 

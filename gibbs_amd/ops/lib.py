@@ -47,7 +47,7 @@ _SIGNATURES = {
                                      c_int, c_int, c_int, c_int, c_long, c_long, c_float, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_glu": [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_shortconv": [c_void_p, c_void_p, c_void_p, c_void_p, c_long, c_void_p, c_void_p, c_void_p, c_void_p,
-                        c_int, c_int, c_int, c_int, c_int, c_void_p],
+                        c_int, c_int, c_int, c_int, c_int, c_int, c_void_p],
     "gibbs_rope_table": [c_void_p, c_void_p, c_int, c_int, c_void_p],
     "gibbs_qk_rope_kv": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_int, c_int,
                          c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_long,

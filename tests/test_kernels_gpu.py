@@ -248,6 +248,49 @@ def test_shortconv_ragged_with_state(dtype, K, C, bias):
     assert torch.all(state[1] == 7.0), "a slot of no request was written"
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C", [24, 520])
+@pytest.mark.parametrize("lens_now", [[1, 1, 1, 1, 1], [1, 1, 1, 40, 2], [1, 1, 70, 1, 1]])
+def test_shortconv_decoded_rows_at_the_head(dtype, C, lens_now):
+    """Requests that bring one row each at the head of the batch (decoded tokens) are found by their tile's number,
+    the others by a walk over the requests behind them: the same result whatever the caller says about the head
+    (nothing, its true length, less), and against conv1d over each whole sequence."""
+    from gibbs_amd import ops
+    K = 3
+    taps, b = rnd(C, K, seed=4), rnd(C, seed=5)
+    lens_before = [9, 1, 3, 0, 5]
+    slots = [4, 0, 3, 1, 5]
+    seqs = [rnd(lb + ln, 3 * C, dtype=dtype, seed=20 + i) for i, (lb, ln) in enumerate(zip(lens_before, lens_now))]
+    lead = next((i for i, n in enumerate(lens_now) if n != 1), len(lens_now))
+    results = []
+    for say in (None, lead, max(lead - 1, 0), 0):
+        state = torch.full((6, K - 1, C), 7.0, device=DEV)
+        with_history = [i for i, lb in enumerate(lens_before) if lb]
+        hist = torch.cat([seqs[i][:lens_before[i]] for i in with_history])
+        cu = i32(np.concatenate([[0], np.cumsum([lens_before[i] for i in with_history])]))
+        ops.shortconv(hist, taps, b, state, cu, i32([0] * len(with_history)), i32([slots[i] for i in with_history]),
+                      hist.shape[0], len(with_history))
+        now = torch.cat([s[lb:] for s, lb in zip(seqs, lens_before)])
+        cu = i32(np.concatenate([[0], np.cumsum(lens_now)]))
+        y = ops.shortconv(now, taps, b, state, cu, i32(lens_before), i32(slots), now.shape[0], len(lens_now), lead_single=say)
+        results.append((y, state))
+    for y, state in results[1:]:
+        assert torch.equal(y, results[0][0]) and torch.equal(state, results[0][1])
+    y, state = results[0]
+    at = 0
+    for seq, lb, ln, slot in zip(seqs, lens_before, lens_now, slots):
+        s = seq.double()
+        bx = s[:, :C] * s[:, 2 * C:]
+        cv = F.conv1d(bx.t()[None], taps.double()[:, None, :], b.double(), groups=C, padding=K - 1)[0, :, :seq.shape[0]].t()
+        close(y[at:at + ln], (s[:, C:2 * C] * cv)[lb:], dtype, "shortconv rows")
+        at += ln
+        full = torch.cat([torch.zeros(K - 1, C, device=DEV, dtype=torch.float64), bx])
+        close(state[slot], full[-(K - 1):], torch.float32, "state", f32=1e-6)
+    assert torch.all(state[2] == 7.0), "a slot of no request was written"
+    with pytest.raises(ops.KernelError, match="leading single rows"):
+        ops.shortconv(now, taps, b, state, cu, i32(lens_before), i32(slots), now.shape[0], len(lens_now), lead_single=6)
+
+
 def paged_setup(dtype, nkv, hd, page_size, seq_lens, num_pages, seed=0):
     """Random keys and values of several requests scattered over shuffled pages (the rest of the
     pool holds large garbage)."""
