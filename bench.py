@@ -6,7 +6,7 @@ decode at batch 1 and 64 beside it.
                     [--batch B] [--prompt-len P --context C] [--suite bench/SUITE.json]
 
 `--prompt-len` / `--context` move the same measurement to longer contexts (16k, 32k, 100k);
-`--prefill-tokens` times a prompt of another length than 2,048; `--suite` runs the rows of a suite file of `gibbs --bench` afterwards
+`--prefill-tokens` times a prompt of another length than 2,048; `--page-size` another page size than the engine's 16; `--suite` runs the rows of a suite file of `gibbs --bench` afterwards
 (the serving workloads of the 350M and 2.6B shapes in bench/lfm2.json) and puts them into the line
 under `rows`.
 
@@ -55,7 +55,7 @@ def shape_for(layers: int) -> dict:
     return cfg
 
 
-def build_engine(dtype: str, layers: int, max_requests: int, context: int = CONTEXT):
+def build_engine(dtype: str, layers: int, max_requests: int, context: int = CONTEXT, page_size: int = 0):
     import torch
 
     from gibbs_amd import Engine
@@ -67,7 +67,7 @@ def build_engine(dtype: str, layers: int, max_requests: int, context: int = CONT
     compute = torch.bfloat16 if dtype == "bfloat16" else torch.float32
     weights = random_weights_on_device(decls, seed=0, compute_dtype=compute, device="cuda:0")
     return Engine(config=cfg, weights=weights, dtype=dtype, max_tokens=max_requests * context,
-                  max_requests=max_requests, ctx=context)
+                  max_requests=max_requests, ctx=context, **({"page_size": page_size} if page_size else {}))
 
 
 def seeded_prompt(seed: int, n: int, vocab: int):
@@ -285,6 +285,7 @@ def main() -> int:
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="tokens every request holds before decoding starts")
     ap.add_argument("--context", type=int, default=None, help="context limit (default 4096, or what --prompt-len needs)")
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT_LEN, help="length of the timed prompt (default 2,048)")
+    ap.add_argument("--page-size", type=int, default=0, help="tokens per cache page (default: the engine's, 16)")
     ap.add_argument("--suite", help="a suite file of `gibbs --bench` whose rows are run afterwards and reported under `rows`")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-parity", action="store_true", help="skip the correctness gate")
@@ -305,7 +306,7 @@ def main() -> int:
     from gibbs_amd import roofline as R
     gate = None if args.no_parity else parity()
     engine = build_engine(args.dtype, args.layers, max_requests=args.batch if args.no_points else max(64, args.batch),
-                          context=context)
+                          context=context, page_size=args.page_size)
 
     ceiling = R.measured_hbm_bytes_per_s()
     prefill_s = time_prefill(engine, n_tokens=args.prefill_tokens)
