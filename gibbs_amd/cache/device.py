@@ -8,6 +8,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from .manager import CacheManager
+from .needs import StateNeed
 
 
 @dataclass
@@ -17,13 +18,14 @@ class LayerCache:
     kpages: Optional[torch.Tensor]              # [num_pages, kv_heads, page_size, head_dim]
     vpages: Optional[torch.Tensor]              # [num_pages, kv_heads, page_size, value head_dim]
     owns_pages: bool                            # False: reads another layer's pages, writes none
-    states: Dict[str, torch.Tensor]             # name -> [slots, *shape] float32 (slot stride = arena row)
+    states: Dict[str, torch.Tensor]             # name -> [slots, *shape] in the state's type (slot stride = arena row)
 
 
 class DeviceCache:
     """Keys and values of a group are laid out [layer of group, page, kv head, slot in page, head_dim]
     (values with their own head size) in the cache dtype (the activation dtype of the run); every
-    group has as many pages as its pool; states are float32.
+    group has as many pages as its pool; a slot of the arena is a row of 4-byte words that holds the layers' states
+    (float32 unless a mixer names another type).
 
     Behind the pool's pages every group holds one more page, and behind the requests' slots the arena
     one more slot, that the cache manager never hands out (`scratch_page`, `scratch_slot`): rows of a
@@ -57,12 +59,12 @@ class DeviceCache:
             idx = m.group_layers[group].index(src)
             k, v = self.kpages[group][idx], self.vpages[group][idx]
         states = {}
-        for (li, name), (off, shape) in m.state_layout.items():
+        for (li, name), (off, shape, dtype) in m.state_layout.items():
             if li == layer:
-                n = 1
-                for s in shape:
-                    n *= s
-                states[name] = self.arena[:, off:off + n].unflatten(1, shape) if shape else self.arena[:, off]
+                need = StateNeed(name, shape, dtype)
+                words = self.arena[:, off:off + need.words]
+                flat = words if dtype == "float32" else words.view(getattr(torch, dtype))[:, :need.numel]
+                states[name] = flat.unflatten(1, shape) if shape else flat[:, 0]
         return LayerCache(group, k, v, kv_source is None and group is not None, states)
 
     def clear_fresh_slots(self) -> None:

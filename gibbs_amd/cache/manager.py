@@ -79,16 +79,16 @@ class CacheManager:
             raise ValueError(f"{len(per_group)} page counts for {n_groups} cache groups")
         if any(n <= 0 for n in per_group):
             raise ValueError(f"a page pool needs at least one page, not {min(per_group)}")
-        # state layout of a slot: (layer, name) -> (offset, shape), in float32 elements
-        self.state_layout: Dict[Tuple[int, str], Tuple[int, Tuple[int, ...]]] = {}
+        # state layout of a slot: (layer, name) -> (offset in 4-byte words, shape, type)
+        self.state_layout: Dict[Tuple[int, str], Tuple[int, Tuple[int, ...], str]] = {}
         off = 0
         for i, layer_states in enumerate(states):
             for s in layer_states:
                 if (i, s.name) in self.state_layout:
                     raise ValueError(f"layer {i} declares state {s.name!r} twice")
-                self.state_layout[(i, s.name)] = (off, tuple(s.shape))
-                off += s.numel
-        self.slot_floats = off
+                self.state_layout[(i, s.name)] = (off, tuple(s.shape), s.dtype)
+                off += s.words
+        self.slot_floats = off        # 4-byte words of a slot
         self._lib = host.library()
         windows = host.ints([int(n.window or 0) for n in self.group_needs])
         self._core = self._lib.gibbs_cache_create(n_groups, windows, page_size, host.ints(per_group), max_requests)

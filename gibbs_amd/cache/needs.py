@@ -21,12 +21,21 @@ class CacheNeed:
         return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
+STATE_DTYPES = {"float32": 4, "int32": 4, "bfloat16": 2, "float16": 2}
+
+
 @dataclass(frozen=True)
 class StateNeed:
-    """A float32 tensor of fixed shape per request (for instance a short convolution's last
-    K-1 inputs), kept in the request's slot."""
+    """A tensor of fixed shape per request (for instance a short convolution's last K-1 inputs), kept in the
+    request's slot: float32 unless the mixer names another type of `STATE_DTYPES`.  A slot is a row of 4-byte
+    words; every state starts at a word, and a slot is all zero bits when a request takes it."""
     name: str
     shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+    def __post_init__(self):
+        if self.dtype not in STATE_DTYPES:
+            raise ValueError(f"state {self.name!r}: type {self.dtype!r} is none of {sorted(STATE_DTYPES)}")
 
     @property
     def numel(self) -> int:
@@ -34,3 +43,8 @@ class StateNeed:
         for s in self.shape:
             n *= s
         return n
+
+    @property
+    def words(self) -> int:
+        """4-byte words of a slot that the state takes."""
+        return -(-self.numel * STATE_DTYPES[self.dtype] // 4)

@@ -56,7 +56,12 @@ def test_pool_basics():
 def test_groups_and_state_layout():
     m = manager(needs=(None, FULL, WIN, FULL, None, WIN))
     assert m.group_needs == [FULL, WIN] and m.group_layers == [[1, 3], [2, 5]]
-    assert m.state_layout == {(0, "conv"): (0, (2, 8)), (4, "conv"): (16, (2, 8))} and m.slot_floats == 32
+    assert m.state_layout == {(0, "conv"): (0, (2, 8), "float32"), (4, "conv"): (16, (2, 8), "float32")} and m.slot_floats == 32
+    typed = CacheManager([None], [(StateNeed("a", (3,), "bfloat16"), StateNeed("n", (1,), "int32"), StateNeed("b", (2, 2)))], 8, 4, 2)
+    assert typed.state_layout == {(0, "a"): (0, (3,), "bfloat16"), (0, "n"): (2, (1,), "int32"), (0, "b"): (3, (2, 2), "float32")}
+    assert typed.slot_floats == 7
+    with pytest.raises(ValueError, match="float64"):
+        StateNeed("x", (1,), "float64")
 
 
 def test_reserve_commit_release():

@@ -487,7 +487,9 @@ def register_toy():
     @register_mixer("toy_ema")
     class ToyEma(Mixer):
         def state_needs(self):
-            return (StateNeed("ema", (self.hidden,)),)
+            # (a float32 average, a count of the request's tokens so far as an integer, and that count modulo 7, 5
+            # and 3 in bfloat16: states of other types than float32, one of an odd size)
+            return (StateNeed("ema", (self.hidden,)), StateNeed("seen", (1,), "int32"), StateNeed("last", (3,), "bfloat16"))
 
         def tensor_decls(self):
             return [TensorDecl(self.spec.tensors["proj"], (self.hidden, self.hidden))]
@@ -498,14 +500,20 @@ def register_toy():
         def forward(self, h, batch, cache):
             u = linear(h, self.w).float()
             decay = self.spec.params["decay"]
-            state = cache.states["ema"]
+            state, seen, last = cache.states["ema"], cache.states["seen"], cache.states["last"]
+            assert seen.dtype == torch.int32 and last.dtype == torch.bfloat16 and last.shape[1:] == (3,)
             out = torch.empty_like(u)
             row = 0
             for q, slot in zip(batch.q_lens, batch.slots):
                 s = state[slot].clone()
+                mods = torch.tensor([7, 5, 3], device=u.device)
                 for t in range(q):
                     s = decay * s + u[row + t]
                     out[row + t] = s
+                    # (the count of tokens so far and its remainders, as the states hold them)
+                    out[row + t, :3] += 0.05 * int(seen[slot, 0]) + 0.5 * last[slot].float()
+                    seen[slot, 0] += 1
+                    last[slot] = (seen[slot, 0] % mods).bfloat16()
                 state[slot] = s
                 row += q
             return out.to(self.rt.act_dtype)
@@ -562,7 +570,8 @@ def toy_plain(cfg, w, ids):
             u, s, a = P.linear(h, w[f"{p}.ema.proj"]), np.zeros(cfg["width"]), []
             for t in range(T):
                 s = cfg["decay"] * s + u[t]
-                a.append(s)
+                a.append(s.copy())
+                a[-1][:3] += 0.05 * t + 0.5 * np.array([t % 7, t % 5, t % 3])
             a = np.stack(a)
         else:
             inv = P.rope_inv_freq(hd, cfg["theta"])
@@ -591,7 +600,8 @@ def test_toy_mixer_with_state_registers_builds_and_steps(name, dtype, tmp_path):
     eng = Engine(folder, dtype=name, max_tokens=128, max_requests=2, page_size=8)     # the class is chosen by config.json
     assert [type(b.mixer).__name__ for b in eng.model.blocks] == ["ToyEma", "AttentionMixer", "ToyEma"]
     assert eng.plan.op_count() == 6, "the toy mixer is a part of the native step's program like any other"
-    assert set(eng.cache.state_layout) == {(0, "ema"), (2, "ema")}
+    assert set(eng.cache.state_layout) == {(i, n) for i in (0, 2) for n in ("ema", "seen", "last")}
+    assert eng.cache.slot_floats == 2 * (40 + 1 + 2), "a float32 row, an integer and three bfloat16 values in two words"
     weights, _ = P.load_model_dir(folder)
     seqs = {"a": H.tokens(1, 30, 83), "b": H.tokens(2, 17, 83)}
     got = {}
