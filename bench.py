@@ -75,12 +75,14 @@ def seeded_prompt(seed: int, n: int, vocab: int):
     return np.random.default_rng(seed).integers(0, vocab, size=n).tolist()
 
 
-def time_prefill(engine, runs: int = 3, n_tokens: int = PROMPT_LEN):
-    """Median time of a whole prompt of `n_tokens` (2,048 unless asked otherwise) in one step (one warm-up first)."""
+def time_prefill(engine, runs: int = 5, n_tokens: int = PROMPT_LEN, warmups: int = 3):
+    """Median time of a whole prompt of `n_tokens` (2,048 unless asked otherwise) in one step.  Three untimed steps
+    first: the first holds the library's choice of algorithms, and the next two still run 5 to 10 % slower than the
+    steady state that follows (clocks, caches)."""
     import torch
     vocab = engine.spec.vocab
     times = []
-    for i in range(runs + 1):
+    for i in range(warmups + runs):
         ids = seeded_prompt(1000 + i, n_tokens, vocab)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -88,7 +90,8 @@ def time_prefill(engine, runs: int = 3, n_tokens: int = PROMPT_LEN):
         torch.cuda.synchronize()
         times.append(time.perf_counter() - t0)
         engine.release("prefill")
-    return sorted(times[1:])[len(times[1:]) // 2]
+    timed = sorted(times[warmups:])
+    return timed[len(timed) // 2]
 
 
 def time_decode(engine, batch: int, steps: int, warmup: int, runs: int = RUNS, profile: bool = False,
