@@ -32,6 +32,8 @@ _SIGNATURES = {
     "gibbs_cache_pages_needed": ([c_void_p, c_int, c_long, _ip], c_int),
     "gibbs_cache_reserve": ([c_void_p, c_int, c_long], c_int),
     "gibbs_cache_commit": ([c_void_p, c_int, c_long], c_int),
+    "gibbs_cache_reserve_all": ([c_void_p, _ip, c_int, c_long, c_long, _ip], c_int),
+    "gibbs_cache_commit_all": ([c_void_p, _ip, c_int, c_long], c_int),
     "gibbs_cache_release": ([c_void_p, c_int], c_int),
     "gibbs_cache_take_fresh_slots": ([c_void_p, _ip, c_int], c_int),
     "gibbs_cache_table_width": ([c_void_p, _ip, c_int, c_int], c_int),
@@ -51,7 +53,7 @@ _SIGNATURES = {
     "gibbs_sched_apply": ([c_void_p, c_int, _ip, _ip, _ip, _lp, c_long, _lp], c_int),
     "gibbs_sched_fail_plan": ([c_void_p, _lp, c_long, _lp], c_int),
     "gibbs_sched_burst_plan": ([c_void_p, c_long, _ip, c_int, _ip, _lp], c_long),
-    "gibbs_sched_apply_burst": ([c_void_p, c_int, c_int, _ip, _lp, c_long, _lp], c_int),
+    "gibbs_sched_apply_burst": ([c_void_p, c_int, _ip, c_int, _ip, _ip, c_int, _ip, _lp, c_long, _lp], c_int),
     "gibbs_cache_fill_step": ([c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, _lp, c_void_p, _lp],
                               c_int),
 }

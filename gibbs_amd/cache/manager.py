@@ -167,6 +167,25 @@ class CacheManager:
             self._raise(code, rid)
         return True
 
+    def reserve_all(self, rids: Sequence[Hashable], n_new: int, limit: int = 0) -> Optional[bool]:
+        """Pages for the next `n_new` positions of every one of the requests, all or nothing, in one call of the
+        core: True if pages were taken, False if none were needed, None if they do not fit (`pages_needed_all` then
+        says how many every group would have needed).  `limit`: the positions a request may hold (0: no check)."""
+        slots = host.ints([self._slots[r] for r in rids])
+        code = self._lib.gibbs_cache_reserve_all(self._core, slots, len(rids), n_new, limit, self._needed)
+        self.pages_needed_all = list(self._needed[:self.n_groups])
+        if code == host.ERR_NO_ROOM:
+            return None
+        if code < 0:
+            self._raise(code, rids[0] if rids else None)
+        return code > 0
+
+    def commit_all(self, rids: Sequence[Hashable], n_new: int) -> None:
+        """`n_new` more positions of every one of the requests are cached now."""
+        code = self._lib.gibbs_cache_commit_all(self._core, host.ints([self._slots[r] for r in rids]), len(rids), n_new)
+        if code < 0:
+            self._raise(code, rids[0] if rids else None)
+
     def commit(self, rid: Hashable, n_new: int) -> None:
         """`n_new` more positions are cached now.  A window group gives back every page that
         no later query can see: page j holds positions [j*ps, (j+1)*ps), the next query is at

@@ -145,6 +145,49 @@ HOST_EXPORT int gibbs_cache_commit(void* core, int slot, long n_new) {
   return 0;
 }
 
+// The same for several requests at once (the rows of a decode loop): pages for n_new more positions of every one
+// of them, all or nothing.  Returns 1 if pages were taken, 0 if none were needed, ERR_NO_ROOM (nothing taken; need[g]
+// says how many pages group g would have needed) or another error.  limit > 0: a request that would then hold more
+// than `limit` positions is an argument error.
+HOST_EXPORT int gibbs_cache_reserve_all(void* core, const int* slots, int n, long n_new, long limit, int* need) {
+  CacheCore* c = (CacheCore*)core;
+  std::vector<int> wanted(c->n_groups(), 0);
+  for (int i = 0; i < n; ++i) {
+    if (int e = need_live(c, slots[i])) return e;
+    const Request& r = c->requests[slots[i]];
+    if (limit > 0 && r.tokens + n_new > limit)
+      return fail(ERR_ARGUMENT, "the request in slot %d would pass the context limit %ld", slots[i], limit);
+    for (int g = 0; g < c->n_groups(); ++g) wanted[g] += c->pages_needed(r, n_new, g);
+  }
+  bool any = false, room = true;
+  for (int g = 0; g < c->n_groups(); ++g) {
+    if (need) need[g] = wanted[g];
+    any = any || wanted[g] > 0;
+    room = room && wanted[g] <= c->pools[g].n_free();
+  }
+  if (!room) return fail(ERR_NO_ROOM, "the decode steps want more pages than are free");
+  for (int i = 0; i < n; ++i) {
+    Request& r = c->requests[slots[i]];
+    for (int g = 0; g < c->n_groups(); ++g) c->pools[g].allocate(c->pages_needed(r, n_new, g), r.pages[g]);
+  }
+  return any ? 1 : 0;
+}
+
+// n_new more positions of every one of several requests are cached now.
+HOST_EXPORT int gibbs_cache_commit_all(void* core, const int* slots, int n, long n_new) {
+  CacheCore* c = (CacheCore*)core;
+  for (int i = 0; i < n; ++i) {      // (all of them or none)
+    if (int e = need_live(c, slots[i])) return e;
+    const Request& r = c->requests[slots[i]];
+    for (int g = 0; g < c->n_groups(); ++g)
+      if (c->pages_for(r.tokens + n_new) > (long)r.pages[g].size())
+        return fail(ERR_PAGE, "commit of %ld tokens beyond its reserved pages", n_new);
+  }
+  for (int i = 0; i < n; ++i)
+    if (int e = gibbs_cache_commit(core, slots[i], n_new)) return e;
+  return 0;
+}
+
 // Gives back every page and the slot of a request that ended.
 HOST_EXPORT int gibbs_cache_release(void* core, int slot) {
   CacheCore* c = (CacheCore*)core;

@@ -372,16 +372,24 @@ HOST_EXPORT long gibbs_sched_burst_plan(const void* sched, long cap, int* out, i
   return n;
 }
 
-// Books the tokens of a burst for one request (all already cached), token by token, by the rules of a
-// step; returns how many of them count as output (the request may end among them).
-HOST_EXPORT int gibbs_sched_apply_burst(void* sched, int id, int n, const int* is_eos, long* events, long events_cap,
-                                        long* n_events) {
+// Books the tokens of a burst (all already cached), request by request and token by token, by the rules of a step:
+// tokens[i * n + j] is what request ids[i] sampled at step j, eos the ids that end a sequence.  took[i]: how many of
+// request i's tokens count as output (the request may end among them).
+HOST_EXPORT int gibbs_sched_apply_burst(void* sched, int n_req, const int* ids, int n, const int* tokens, const int* eos,
+                                        int n_eos, int* took, long* events, long events_cap, long* n_events) {
   Scheduler* s = (Scheduler*)sched;
   s->events.clear();
-  if (id < 0 || id >= (int)s->seqs.size()) return fail(ERR_ARGUMENT, "no request %d", id);
-  const long before = s->seqs[id].output_len;
-  for (int i = 0; i < n; ++i)
-    if (!s->take_token(id, is_eos[i] != 0)) break;
+  for (int i = 0; i < n_req; ++i)
+    if (ids[i] < 0 || ids[i] >= (int)s->seqs.size()) return fail(ERR_ARGUMENT, "no request %d", ids[i]);
+  for (int i = 0; i < n_req; ++i) {
+    const long before = s->seqs[ids[i]].output_len;
+    for (int j = 0; j < n; ++j) {
+      const int token = tokens[(long)i * n + j];
+      const bool is_eos = std::find(eos, eos + n_eos, token) != eos + n_eos;
+      if (!s->take_token(ids[i], is_eos)) break;
+    }
+    took[i] = (int)(s->seqs[ids[i]].output_len - before);
+  }
   *n_events = copy_events(s, events, events_cap);
-  return (int)(s->seqs[id].output_len - before);
+  return 0;
 }

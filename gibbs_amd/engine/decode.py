@@ -178,19 +178,14 @@ class DecodeLoop:
 
     def _reserve(self, n_steps: int) -> None:
         cm = self.engine.cache
-        for rid in self.rids:
-            if cm.tokens(rid) + self.pending + n_steps > self.engine.ctx_limit:
-                raise StepError(f"request {rid!r} would pass the context limit {self.engine.ctx_limit}")
-        need = [0] * cm.n_groups
-        for rid in self.rids:
-            for g, k in enumerate(cm.pages_needed(rid, self.pending + n_steps)):
-                need[g] += k
-        for g, k in enumerate(need):
-            if k > cm.free_pages(g):
-                raise OutOfPages(f"{n_steps} decode steps need {k} pages of cache group {g}, {cm.free_pages(g)} are free")
-        grew = any(need)
-        for rid in self.rids:
-            assert cm.reserve(rid, self.pending + n_steps)
+        try:
+            grew = cm.reserve_all(self.rids, self.pending + n_steps, self.engine.ctx_limit)
+        except ValueError as e:
+            raise StepError(str(e)) from None
+        if grew is None:
+            need = cm.pages_needed_all
+            g = next(g for g, k in enumerate(need) if k > cm.free_pages(g))
+            raise OutOfPages(f"{n_steps} decode steps need {need[g]} pages of cache group {g}, {cm.free_pages(g)} are free")
         if grew:
             self._fill_tables()
             for g in range(cm.n_groups):
@@ -287,8 +282,7 @@ class DecodeLoop:
 
     def sync_cache(self) -> None:
         """Tells the cache manager about the positions the device has filled."""
-        for rid in self.rids:
-            self.engine.cache.commit(rid, self.pending)
+        self.engine.cache.commit_all(self.rids, self.pending)
         self.pending = 0
 
     def tokens(self, last: Optional[int] = None) -> List[List[int]]:

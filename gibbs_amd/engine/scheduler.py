@@ -350,19 +350,20 @@ class ContinuousBatchScheduler:
 
     def apply_burst(self, seqs: List[Sequence], tokens: List[List[int]]) -> StepOutput:
         """Books the tokens that a burst sampled (tokens[i]: those of seqs[i], all already cached):
-        the same emitting and finishing rules as a step, token by token."""
-        self.steps += len(tokens[0]) if tokens else 0
+        the same emitting and finishing rules as a step, token by token (one call of the core for all of them)."""
+        k, n = len(seqs), len(tokens[0]) if tokens else 0
+        self.steps += n
+        flat = (ctypes.c_int * max(1, k * n))(*[int(t) for toks in tokens for t in toks])
+        took = (ctypes.c_int * max(1, k))()
+        if self._lib.gibbs_sched_apply_burst(self._core, k, host.ints([s.submitted for s in seqs]), n, flat,
+                                             host.ints(sorted(self.eos)), len(self.eos), took, self._events,
+                                             len(self._events), ctypes.byref(self._n_events)) < 0:
+            raise RuntimeError(host.last_error())
         emitted: List[Tuple[Hashable, int]] = []
-        finished: List[Hashable] = []
-        for seq, toks in zip(seqs, tokens):
-            is_eos = (ctypes.c_int * max(1, len(toks)))(*[int(t in self.eos) for t in toks])
-            took = self._lib.gibbs_sched_apply_burst(self._core, seq.submitted, len(toks), is_eos, self._events,
-                                                     len(self._events), ctypes.byref(self._n_events))
-            if took < 0:
-                raise RuntimeError(host.last_error())
-            seq.output_tokens.extend(int(t) for t in toks[:took])
-            emitted.extend((seq.id, int(t)) for t in toks[:took])
-            finished += self._book()[0]
+        for seq, toks, t in zip(seqs, tokens, took):
+            seq.output_tokens.extend(int(x) for x in toks[:t])
+            emitted.extend((seq.id, int(x)) for x in toks[:t])
+        finished = self._book()[0]
         waiting, active = self._counts()
         return StepOutput([], emitted, finished, [], 0, len(emitted), active, waiting)
 

@@ -86,6 +86,31 @@ def test_reserve_commit_release():
     m.check()
 
 
+def test_reserve_and_commit_for_several_requests_at_once():
+    """What a decode loop asks before and after its steps: pages for the next positions of all its requests, all or
+    nothing, and the commit of all of them, each in one call of the core."""
+    m = manager()                                                # 12 pages of 16 tokens
+    for r in "abc":
+        assert m.admit(r)
+    assert m.reserve("a", 30) and m.reserve("b", 16) and m.reserve("c", 5)
+    m.commit("a", 30); m.commit("b", 16); m.commit("c", 5)
+    assert m.free_pages() == 8
+    assert m.reserve_all(["a", "b", "c"], 2) is True and m.pages_needed_all == [1], "only b stands at a page's edge"
+    assert m.free_pages() == 7
+    assert m.reserve_all(["a", "b", "c"], 2) is False and m.free_pages() == 7, "asking again takes nothing"
+    m.commit_all(["a", "b", "c"], 2)
+    assert [m.tokens(r) for r in "abc"] == [32, 18, 7]
+    assert m.reserve_all(["a", "b", "c"], 16 * 3) is None and m.pages_needed_all == [9] and m.free_pages() == 7, \
+        "3 + 3 + 3 pages do not fit 7: nothing is taken"
+    assert m.reserve_all(["a", "b"], 16 * 3) is True and m.free_pages() == 1
+    with pytest.raises(ValueError, match="context limit"):
+        m.reserve_all(["c"], 10, limit=16)
+    with pytest.raises(PageError, match="beyond its reserved pages"):
+        m.commit_all(["a", "c"], 48)
+    assert m.tokens("a") == 32, "a commit that one request cannot take changes none"
+    m.check()
+
+
 def test_slots_and_fresh():
     m = manager(reqs=2)
     assert m.admit(1) and m.admit(2) and not m.admit(3)
