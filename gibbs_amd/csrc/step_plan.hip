@@ -215,7 +215,9 @@ struct Exec {
   bool dry;
   int status = 0;
   int esize;                  // bytes of an activation element
-  bool bf16_run, fused_step;
+  bool bf16_run;
+  bool few_rows;              // a bfloat16 step of so few rows that the weight-streaming products with fused epilogues take it
+  bool fused_step;            // and every row is one token of a request of its own (decoded tokens)
   int fused_halves = 0;
   Exec(const Plan& plan, const GibbsStepArgs& args);
   void* take(long bytes) {
@@ -262,7 +264,9 @@ struct NormPart {
 struct Body {
   virtual ~Body() = default;
   virtual Pending general(Exec& e, void* h) const = 0;    // the delta of normed rows h [N, hidden]
-  virtual bool fusable() const { return false; }         // has fused decode kernels for its sizes
+  // has fused few-row kernels for its sizes and for this step (single: every row is one token of its own request;
+  // a part that works on rows one by one, as a feed-forward does, need not ask for that)
+  virtual bool fusable(bool single) const { return false; }
   virtual void fused(Exec& e, float eps, float* x, void* mirror) const {}   // x += body(x / rms(x)), mirror kept
   virtual int cache_group() const { return -1; }
 };
@@ -294,7 +298,8 @@ Exec::Exec(const Plan& plan, const GibbsStepArgs& args)
     : p(plan), a(args), arena(args.workspace, args.workspace_bytes, args.workspace == nullptr), dry(args.workspace == nullptr) {
   esize = p.dtype == GIBBS_BF16 ? 2 : 4;
   bf16_run = p.dtype == GIBBS_BF16;
-  fused_step = bf16_run && a.max_q == 1 && a.n_rows <= std::min(p.fused_rows, FUSED_ROWS);
+  few_rows = bf16_run && a.n_rows <= std::min(p.fused_rows, FUSED_ROWS);
+  fused_step = few_rows && a.max_q == 1;
 }
 
 void* Exec::linear(const void* x, const Matrix& m, int n, bool out_f32, bool partial_ok, bool use_packed, int* parts) {
@@ -375,7 +380,7 @@ struct ConvBody : Body {
   int C = 0, K = 0;
   float* state = nullptr;        // [slots, K - 1, C] float32
   long slot_stride = 0;
-  bool fusable() const override { return in.I % 8 == 0 && C % 8 == 0 && K <= 8; }
+  bool fusable(bool single) const override { return single && in.I % 8 == 0 && C % 8 == 0 && K <= 8; }
   void fused(Exec& e, float eps, float* x, void* mirror) const override {
     const int N = e.a.n_rows, H = in.I;
     void* y = e.take((long)N * C * 2);
@@ -384,14 +389,19 @@ struct ConvBody : Body {
     e.skinny_residual(y, out, x, mirror);
     e.give(y);
   }
-  Pending general(Exec& e, void* h) const override {
+  // the gated convolution of the projected rows [N, 3 C] with the requests' states; gives the rows back
+  void* convolve(Exec& e, void* bcx) const {
     const int N = e.a.n_rows;
-    void* bcx = e.linear(h, in, N, false, false, false, nullptr);
     void* y = e.take((long)N * C * e.esize);
     // (requests at the head of the batch that bring one row each: all of them in a step of decoded tokens)
     const int lead = e.a.max_q == 1 ? e.a.n_req : e.a.lead_single;
     RUN(e, gibbs_shortconv(bcx, taps, bias, state, slot_stride, e.a.cu, e.a.ctx, e.a.slot, y, e.p.dtype, N, e.a.n_req, lead, C, K, e.a.stream));
     e.give(bcx);
+    return y;
+  }
+  Pending general(Exec& e, void* h) const override {
+    const int N = e.a.n_rows;
+    void* y = convolve(e, e.linear(h, in, N, false, false, false, nullptr));
     Pending delta;
     delta.data = e.linear(y, out, N, false, true, true, &delta.parts);
     e.give(y);
@@ -420,7 +430,7 @@ struct AttnBody : Body {
   bool fast() const { return !slopes && !hook; }   // the fast kernels know rotations only (or no encoding at all)
   // what the kernel that takes the raw projection (q/k norm, rotation, cache write and attention in one) needs
   bool raw_ok() const { return fast() && owns && hd % 16 == 0 && hd <= 256 && (!inv_freq || rot % 16 == 0); }
-  bool fusable() const override { return raw_ok() && qkv.I % 8 == 0 && (nh * hd) % 8 == 0; }
+  bool fusable(bool single) const override { return single && raw_ok() && qkv.I % 8 == 0 && (nh * hd) % 8 == 0; }
 
   // decoded tokens from the raw projection: q/k norm, rotation, the cache write and attention in one kernel
   void* attend_decoded(Exec& e, const void* raw) const {
@@ -478,11 +488,11 @@ struct AttnBody : Body {
       RUN(e, gibbs_qk_rope_kv(raw, kpages, vpages, e.p.dtype, nullptr, nullptr, qk_eps, nullptr, 0, 0, nullptr, 0, e.a.pos, e.a.row_req,
                               table, width, page_size, num_pages, N, nh, kv, hd, ldq, e.a.stream));
   }
-  Pending general(Exec& e, void* h) const override {
+  // attention of the projected rows raw [N, (nh + 2 kv) hd]: whatever the step's rows are
+  void* attend(Exec& e, void* raw) const {
     const GibbsStepArgs& a = e.a;
     const int N = a.n_rows, kv = owns ? nkv : 0;
     const long ldq = (long)(nh + 2 * kv) * hd, ldo = (long)nh * hd;
-    void* raw = e.linear(h, qkv, N, false, false, false, nullptr);
     void* att;
     if (e.bf16_run && a.max_q == 1 && raw_ok()) {
       att = attend_decoded(e, raw);
@@ -512,6 +522,12 @@ struct AttnBody : Body {
                                      nkv, hd, ldq, ldo, scale, window, slopes, a.stream));
       }
     }
+    return att;
+  }
+  Pending general(Exec& e, void* h) const override {
+    const int N = e.a.n_rows;
+    void* raw = e.linear(h, qkv, N, false, false, false, nullptr);
+    void* att = attend(e, raw);
     e.give(raw);
     Pending delta;
     delta.data = e.linear(att, out, N, false, true, true, &delta.parts);
@@ -525,7 +541,7 @@ struct GluBody : Body {
   Matrix gate_up, down;
   const void* gate_up_packed2 = nullptr;   // gate and up packed as two row groups, for the fused kernel
   int F = 0, act = 0;
-  bool fusable() const override { return gate_up.I % 8 == 0 && F % 8 == 0; }
+  bool fusable(bool) const override { return gate_up.I % 8 == 0 && F % 8 == 0; }   // (rows one by one: any few rows)
   void fused(Exec& e, float eps, float* x, void* mirror) const override {
     const int N = e.a.n_rows, H = gate_up.I;
     void* y = e.take((long)N * F * 2);
@@ -566,10 +582,10 @@ struct HostBody : Body {
 void Exec::run() {
   const int N = a.n_rows, H = p.hidden;
   float* x = a.x_in;
-  void* mirror = fused_step ? a.mirror_in : nullptr;
+  void* mirror = few_rows ? a.mirror_in : nullptr;
   if (!x) {
     x = (float*)take((long)N * H * 4);
-    mirror = fused_step ? take((long)N * H * 2) : nullptr;
+    mirror = few_rows ? take((long)N * H * 2) : nullptr;
     RUN(*this, gibbs_embed(p.table, p.table_dtype, a.ids, x, mirror, N, H, p.vocab, a.stream));
   }
   Pending pending;
@@ -584,7 +600,7 @@ void Exec::run() {
         const NormPart& n = *p.norms[op.norm];
         const Body& b = *p.bodies[op.body];
         float eps = 0.f;
-        if (fused_step && b.fusable() && n.folded_rms(&eps)) {
+        if (few_rows && b.fusable(fused_step) && n.folded_rms(&eps)) {
           with_mirror(x, pending, &mirror);
           b.fused(*this, eps, x, mirror);
           ++fused_halves;
