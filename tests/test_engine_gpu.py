@@ -188,9 +188,15 @@ def test_decoded_tokens_at_the_head_of_a_mixed_step(model_dirs, name, dtype):
             entries.append((r, seqs[r][at[r]:at[r] + n], list(range(n))))
             at[r] += n
         steps.append((entries, []))
-    got = run_steps(make_engine(d, dtype, max_tokens=512, max_requests=5), steps)
+    eng = make_engine(d, dtype, max_tokens=512, max_requests=5)
+    got = run_steps(eng, steps)
     assert ("s3", 74) in got and ("s0", 31) in got
     check(d, seqs, got, dtype, f"decoded tokens first {name} {dtype}")
+    # the last step had 38 rows, 34 of them a prompt portion: in bfloat16 its feed-forward halves took the fused
+    # few-row kernels (they work on rows one by one), its mixers the kernels for rows of any kind
+    assert eng.plan.last_fused() == (len(eng.model.blocks) if dtype == "bfloat16" else 0)
+    run_steps(eng, [([(r, [seqs[r][at[r]]], [0]) for r in ("s0", "s2")], [])])
+    assert eng.plan.last_fused() == (2 * len(eng.model.blocks) if dtype == "bfloat16" else 0), "decoded tokens only: both halves"
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
