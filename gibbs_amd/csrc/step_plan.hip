@@ -44,7 +44,7 @@ long ceil_div_l(long a, long b) { return (a + b - 1) / b; }
 
 // ------------------------------------------------------------------------------------------------- rules
 constexpr int FUSED_ROWS = 64;            // rows that the few-row products (and so the fused decode kernels) take
-constexpr int SKINNY_ROWS = 32;           // rows up to which a plain product takes the weight-streaming kernel
+constexpr int SKINNY_ROWS = 64;           // rows up to which a plain product takes the weight-streaming kernel
 constexpr int SKINNY_ROWS_F32_OUT = 48;   // the same for float32 output (the head: it streams faster than the tiled product)
 constexpr int MATRIX_SLICE_PAGES = 510;   // page ids of a key slice that the decode attention's matrix-core walk keeps in LDS
 
