@@ -153,12 +153,16 @@ class Generator:
         torch.cuda.synchronize(self.engine.device)
         now = time.perf_counter()
         dt = now - t0
-        for rid, _ in out.emitted:
-            t = self._times.get(rid)
+        last = t = object()
+        for rid, _ in out.emitted:          # (a burst's tokens come request by request)
+            if rid is not last and rid != last:
+                last, t = rid, self._times.get(rid)
+                if t is not None:
+                    if t[3] == 0:
+                        t[1] = now
+                    t[2] = now
             if t is not None:
-                if t[3] == 0:
-                    t[1] = now
-                t[2], t[3] = now, t[3] + 1
+                t[3] += 1
         self.stats.steps += 1
         if out.prefill_tokens:
             self.stats.prefill_tokens += out.prefill_tokens

@@ -34,6 +34,7 @@ from __future__ import annotations
 
 import ctypes
 import dataclasses
+import itertools
 import time
 from collections import deque
 from dataclasses import dataclass, field
@@ -353,7 +354,7 @@ class ContinuousBatchScheduler:
         the same emitting and finishing rules as a step, token by token (one call of the core for all of them)."""
         k, n = len(seqs), len(tokens[0]) if tokens else 0
         self.steps += n
-        flat = (ctypes.c_int * max(1, k * n))(*[int(t) for toks in tokens for t in toks])
+        flat = (ctypes.c_int * max(1, k * n))(*[t for toks in tokens for t in toks])
         took = (ctypes.c_int * max(1, k))()
         if self._lib.gibbs_sched_apply_burst(self._core, k, host.ints([s.submitted for s in seqs]), n, flat,
                                              host.ints(sorted(self.eos)), len(self.eos), took, self._events,
@@ -361,8 +362,9 @@ class ContinuousBatchScheduler:
             raise RuntimeError(host.last_error())
         emitted: List[Tuple[Hashable, int]] = []
         for seq, toks, t in zip(seqs, tokens, took):
-            seq.output_tokens.extend(int(x) for x in toks[:t])
-            emitted.extend((seq.id, int(x)) for x in toks[:t])
+            mine = toks[:t]
+            seq.output_tokens.extend(mine)
+            emitted.extend(zip(itertools.repeat(seq.id), mine))
         finished = self._book()[0]
         waiting, active = self._counts()
         return StepOutput([], emitted, finished, [], 0, len(emitted), active, waiting)
